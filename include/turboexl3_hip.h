@@ -1,0 +1,170 @@
+/*
+ * turboexl3 on MI355X (gfx950): the C ABI of the EXL3 projection engine.
+ *
+ * Every entry point takes plain pointers, sizes and small POD descriptors; no C++ or framework types cross the
+ * boundary. A descriptor (`t3_array`) stands where the reference passes an `mlx_array` handle: a device pointer
+ * to row-contiguous data with its shape and dtype. Work is enqueued on the caller's HIP stream (`void*` =
+ * `hipStream_t`, NULL = the null stream) and never synchronised here. Outputs and scratch are the caller's:
+ * ask `*_workspace_bytes`, allocate once, pass the pointer. Inputs are borrowed, never copied or kept.
+ *
+ * Refusal convention (turboexl3 docs/core/api.md:10-12): a call this library does not serve returns a named
+ * status before it launches anything and leaves every output untouched; the caller runs its own chain.
+ * The status names are the reference's Zig error names.
+ *
+ * Paths in comments are relative to the turboexl3 source tree.
+ */
+#ifndef TURBOEXL3_HIP_H
+#define TURBOEXL3_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define T3_ABI_VERSION 1
+
+typedef void* t3_stream; /* hipStream_t */
+
+/* ---- status ----------------------------------------------------------------------------------------------- */
+
+typedef enum t3_status {
+    T3_OK = 0,
+    T3_BadExl3Shape = 1,                /* src/root.zig:93-101,128-141,309-326 */
+    T3_BadExl3Dtype = 2,                /* src/root.zig:102,135-139,322 */
+    T3_Exl3EngineNotImplemented = 3,    /* src/root.zig:841,851; docs/core/api.md:10-12 */
+    T3_Exl3EngineCacheFull = 4,         /* src/root.zig:143-151 (kept for the name; this library has no cache to fill) */
+    T3_Exl3GateUpRateMismatch = 5,      /* src/root.zig:117 */
+    T3_InvalidExl3Clamp = 6,            /* src/root.zig:1002 */
+    T3_Exl3TopKExceedsReduceBank = 7,   /* src/core/spec.zig:75-77 */
+    T3_Exl3WindowUnsupported = 8,       /* src/core/spec.zig:49 */
+    T3_ExpertLayoutUnsupported = 9,     /* src/core/spec.zig:38-48 */
+    T3_InvalidTurboexl3Config = 10,     /* src/core/config.zig:175-178 */
+    T3_WorkspaceTooSmall = 11,          /* this ABI: the caller's scratch is smaller than *_workspace_bytes says */
+    T3_HipFailed = 12,                  /* src/hip/runtime.zig:6 */
+    T3_BadArgs = 13                     /* src/hip/runtime.zig:6: a null pointer or a descriptor that is not one */
+} t3_status;
+
+/* The reference's error name of a status ("BadExl3Shape", ...); "ok" for T3_OK; never NULL. */
+const char* t3_error_name(int32_t status);
+
+/* ---- descriptors ------------------------------------------------------------------------------------------ */
+
+typedef enum t3_dtype {
+    T3_F32 = 0, T3_F16 = 1, T3_BF16 = 2, /* activations, scores (src/hip/plan.zig:72-73 numbering) */
+    T3_U16 = 3, T3_I16 = 4,              /* trellis halfwords (src/root.zig:87-91) */
+    T3_U32 = 5, T3_I32 = 6               /* expert ids (src/root.zig:136) */
+} t3_dtype;
+
+#define T3_MAX_DIMS 8
+
+/* A row-contiguous device array: what an mlx_array handle carries for this path. */
+typedef struct t3_array {
+    void* data;
+    int32_t ndim;
+    int32_t dtype; /* t3_dtype */
+    int64_t shape[T3_MAX_DIMS];
+} t3_array;
+
+/* How a pack's trellis decodes (src/core/format.zig:71-78): codebook 0 = MUL1, 1 = MCG; window 8..16 bits. */
+typedef struct t3_decode {
+    int32_t codebook;
+    int32_t window_bits;
+} t3_decode;
+
+/* One projection's arrays (src/root.zig:73-75): dense: trellis [in/16, out/16, n], suh [in], svh [out];
+ * bank: a leading expert axis on each. trellis U16 or I16; suh, svh F16. */
+typedef struct t3_proj {
+    t3_array trellis, suh, svh;
+} t3_proj;
+
+typedef struct t3_bank {
+    t3_proj gate, up, down;
+} t3_bank;
+
+/* ---- configuration (src/core/config.zig; only the fields this path reads) --------------------------------- */
+
+typedef struct t3_config {
+    int32_t decode_form;   /* 3: the five-launch chain; 9 (default): the fused form; others refused */
+    int32_t dec_one;       /* 1 (default): dense decode rows in one launch; 0: the three-launch chain */
+    int32_t prefill;       /* 1 (default); 0: routed calls above 16 rows refuse Exl3EngineNotImplemented */
+    int32_t mcg_pair;      /* 1 (default): MCG's GEMV feeds the hashed pair to the matrix core unrounded; 0: the f16 weight */
+    int32_t mul1_defer;    /* 1 (default): MUL1's affine map applied once an output (src/core/dense.zig deferFor); 0: per weight */
+} t3_config;
+
+/* The served configuration. */
+void t3_config_default(t3_config* out);
+/* Set once before the first call; a value this library does not serve returns T3_InvalidTurboexl3Config and
+ * changes nothing (src/core/config.zig:175-178). */
+int32_t t3_configure(const t3_config* cfg);
+/* Kept for surface parity with src/root.zig:1148-1181: this library compiles nothing at run time and holds no
+ * per-geometry state, so there is nothing to free. */
+void t3_release_engines(void);
+
+/* ---- dense projection (src/root.zig:309-351 `linear`) ------------------------------------------------------- */
+
+/* y [..., out] in x's dtype for x [..., in]. Rows = the product of x's leading dims.
+ * 1..32 rows: the trellis GEMV on the matrix cores; more: W_hat decode + f16 GEMM. `y` is the caller's, shaped as x
+ * with the last dim `out`. Status as root.linearOn's checks. */
+int32_t t3_linear(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
+                  const t3_array* svh, t3_decode dec, t3_array* y, void* workspace, size_t workspace_bytes);
+/* Scratch bytes `t3_linear` needs for this call's shapes (the byte rules of src/hip/plan.zig:137-146 for this
+ * library's own partition). */
+int32_t t3_linear_workspace_bytes(const t3_array* x, const t3_array* trellis, t3_decode dec, size_t* bytes);
+
+/* The three-launch chain of the same call (prepare, GEMV, finish): the chain `t3_linear`'s one launch must equal
+ * byte for byte (src/core/gpu_test.zig:1016 holds DEC-ONE to the chain the same way). Rows 1..32 only. */
+int32_t t3_linear_chain(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
+                        const t3_array* svh, t3_decode dec, t3_array* y, void* workspace, size_t workspace_bytes);
+
+/* W_hat f16 [in, out] from trellis [in/16, out/16, n], bit-exact to format.reconstructInner
+ * (src/core/format.zig:276-291; the role of src/core/dense.zig:909-922 `dequantize`). */
+int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_array* w_hat);
+
+/* ---- routed experts (src/root.zig:822-904,976-1004) ------------------------------------------------------- */
+
+/* x [B, S, D]; inds (U32/I32) and scores (F32/BF16/F16) [B, S, K], K <= 32; y [B, S, D] in x's dtype.
+ * `verify_rows` is accepted and ignored, as in the reference (src/root.zig:822-825). */
+int32_t t3_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
+               const t3_array* scores, t3_decode dec, int32_t verify_rows, t3_array* y, void* workspace,
+               size_t workspace_bytes);
+/* `t3_moe` with the SwiGLU's gate clamped from above and up to [-limit, limit]; limit 1..128 else
+ * T3_InvalidExl3Clamp (src/root.zig:1001-1004). */
+int32_t t3_moe_clamped(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
+                       const t3_array* scores, t3_decode dec, int32_t limit, t3_array* y, void* workspace,
+                       size_t workspace_bytes);
+/* `t3_moe` plus an already gated shared-expert output of x's shape and dtype, added at the routed output's
+ * rounding point (src/root.zig:976-984). */
+int32_t t3_moe_with_shared(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
+                           const t3_array* scores, t3_decode dec, int32_t verify_rows, const t3_array* shared,
+                           t3_array* y, void* workspace, size_t workspace_bytes);
+int32_t t3_moe_workspace_bytes(const t3_array* x, const t3_bank* bank, const t3_array* inds, size_t* bytes);
+
+/* ---- pack contract (src/core/spec.zig) ------------------------------------------------------------------- */
+
+#define T3_DECODE_ROWS_MAX 16 /* src/core/spec.zig:59 */
+#define T3_REDUCE_MAX_TOPK 32 /* src/core/spec.zig:61 */
+
+/* n halfwords a tile: even, 16..128 (src/core/format.zig:96-100). */
+int32_t t3_rate_admitted(int64_t n);
+/* T3_Exl3TopKExceedsReduceBank above 32 (src/core/spec.zig:75-77). */
+int32_t t3_admit_topk(int64_t topk);
+/* A stacked trellis [E, in/16, out/16, n] at or under rate n_max (src/core/spec.zig:80-88): 1 admitted, 0 not. */
+int32_t t3_trellis_admitted(const int64_t* shape, int32_t ndim, int64_t experts, int64_t in_dim, int64_t out_dim,
+                            int64_t n_max);
+
+/* ---- device self-tests (the roles of src/kernels/hip/test/lane.hip) ------------------------------------------ */
+
+/* mcg, mul1, t: device u16 [65536]: every codeword's MCG value, MUL1 value and MUL1 byte sum. */
+int32_t t3_test_codebooks(t3_stream stream, uint16_t* mcg, uint16_t* mul1, uint16_t* t);
+/* trellis: device u16 [tiles, n]; cw, mcg, mul1: device u16 [tiles, 256] by code position. */
+int32_t t3_test_lane(t3_stream stream, const uint16_t* trellis, int64_t n, int32_t window_bits, int64_t tiles,
+                     uint16_t* cw, uint16_t* mcg, uint16_t* mul1);
+/* a f16 [16, 32], b f16 [32, 16] (bits), d f32 [16, 16] = a b through the kernels' MFMA fragments. */
+int32_t t3_test_mfma(t3_stream stream, const uint16_t* a, const uint16_t* b, float* d);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,90 @@
+"""Loads libturboexl3_hip.so (built in-tree by turboexl3_amd.build) and declares the C ABI of
+include/turboexl3_hip.h to ctypes. There is no fallback: a missing library is an error."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libturboexl3_hip.so")
+
+T3_MAX_DIMS = 8
+
+# t3_dtype
+F32, F16, BF16, U16, I16, U32, I32 = range(7)
+
+STATUS_NAMES = [
+    "ok", "BadExl3Shape", "BadExl3Dtype", "Exl3EngineNotImplemented", "Exl3EngineCacheFull",
+    "Exl3GateUpRateMismatch", "InvalidExl3Clamp", "Exl3TopKExceedsReduceBank", "Exl3WindowUnsupported",
+    "ExpertLayoutUnsupported", "InvalidTurboexl3Config", "WorkspaceTooSmall", "HipFailed", "BadArgs",
+]
+
+
+class Array(C.Structure):
+    _fields_ = [("data", C.c_void_p), ("ndim", C.c_int32), ("dtype", C.c_int32), ("shape", C.c_int64 * T3_MAX_DIMS)]
+
+
+class Decode(C.Structure):
+    _fields_ = [("codebook", C.c_int32), ("window_bits", C.c_int32)]
+
+
+class Proj(C.Structure):
+    _fields_ = [("trellis", Array), ("suh", Array), ("svh", Array)]
+
+
+class Bank(C.Structure):
+    _fields_ = [("gate", Proj), ("up", Proj), ("down", Proj)]
+
+
+class Config(C.Structure):
+    _fields_ = [("decode_form", C.c_int32), ("dec_one", C.c_int32), ("prefill", C.c_int32),
+                ("mcg_pair", C.c_int32), ("mul1_defer", C.c_int32)]
+
+
+# every symbol include/turboexl3_hip.h declares: name -> (restype, argtypes)
+_AP, _BP = C.POINTER(Array), C.POINTER(Bank)
+_u16p = C.POINTER(C.c_uint16)
+SYMBOLS = {
+    "t3_error_name": (C.c_char_p, [C.c_int32]),
+    "t3_config_default": (None, [C.POINTER(Config)]),
+    "t3_configure": (C.c_int32, [C.POINTER(Config)]),
+    "t3_release_engines": (None, []),
+    "t3_linear": (C.c_int32, [C.c_void_p, _AP, _AP, _AP, _AP, Decode, _AP, C.c_void_p, C.c_size_t]),
+    "t3_linear_workspace_bytes": (C.c_int32, [_AP, _AP, Decode, C.POINTER(C.c_size_t)]),
+    "t3_linear_chain": (C.c_int32, [C.c_void_p, _AP, _AP, _AP, _AP, Decode, _AP, C.c_void_p, C.c_size_t]),
+    "t3_dequant": (C.c_int32, [C.c_void_p, _AP, Decode, _AP]),
+    "t3_moe": (C.c_int32, [C.c_void_p, _AP, _BP, _AP, _AP, Decode, C.c_int32, _AP, C.c_void_p, C.c_size_t]),
+    "t3_moe_clamped": (C.c_int32, [C.c_void_p, _AP, _BP, _AP, _AP, Decode, C.c_int32, _AP, C.c_void_p, C.c_size_t]),
+    "t3_moe_with_shared": (C.c_int32, [C.c_void_p, _AP, _BP, _AP, _AP, Decode, C.c_int32, _AP, _AP, C.c_void_p,
+                                        C.c_size_t]),
+    "t3_moe_workspace_bytes": (C.c_int32, [_AP, _BP, _AP, C.POINTER(C.c_size_t)]),
+    "t3_rate_admitted": (C.c_int32, [C.c_int64]),
+    "t3_admit_topk": (C.c_int32, [C.c_int64]),
+    "t3_trellis_admitted": (C.c_int32, [C.POINTER(C.c_int64), C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_int64]),
+    "t3_test_codebooks": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "t3_test_lane": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int64, C.c_void_p, C.c_void_p,
+                                 C.c_void_p]),
+    "t3_test_mfma": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+}
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    """The loaded library with every entry point typed. Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m turboexl3_amd.build` "
+                "(there is no CPU or PyTorch fallback for the HIP kernels)")
+        L = C.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(L, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = L
+    return _lib
+
+
+def error_name(status: int) -> str:
+    return lib().t3_error_name(status).decode()

@@ -1,0 +1,238 @@
+"""The module entry points of turboexl3's projection path over torch device tensors, mirroring
+src/root.zig's `linear` (:309-351), `moe` (:822-904), `moeWithShared` (:976-984), `moeClamped` (:1001-1004) and
+`configure`: same names, argument meaning and refusals (a refusal raises `T3Error` carrying the reference's
+error name). torch is plumbing here: it owns device memory and the stream; all arithmetic runs in
+libturboexl3_hip.so through the C ABI."""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+import torch
+
+from . import _lib
+from ._lib import Array, Bank as CBank, Config, Decode as CDecode, Proj as CProj
+
+MUL1, MCG = 0, 1
+
+
+class T3Error(RuntimeError):
+    """A named refusal or failure; `.name` is the reference's Zig error name."""
+
+    def __init__(self, status: int):
+        self.status = status
+        self.name = _lib.error_name(status)
+        super().__init__(self.name)
+
+
+@dataclass(frozen=True)
+class Decode:
+    """format.Decode: codebook (0 MUL1 / 1 MCG) and codeword window (8..16 bits)."""
+    codebook: int = MUL1
+    window_bits: int = 16
+
+    def c(self) -> CDecode:
+        return CDecode(self.codebook, self.window_bits)
+
+
+Decode.mul1 = Decode(MUL1, 16)
+Decode.mcg = Decode(MCG, 16)
+
+
+@dataclass
+class Proj:
+    """One projection's arrays (root.Proj): trellis U16/I16 [E, in/16, out/16, n], suh F16 [E, in], svh F16 [E, out]."""
+    trellis: torch.Tensor
+    suh: torch.Tensor
+    svh: torch.Tensor
+
+
+@dataclass
+class Bank:
+    gate: Proj
+    up: Proj
+    down: Proj
+
+
+_DTYPES = {
+    torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16,
+    torch.uint16: _lib.U16, torch.int16: _lib.I16, torch.uint32: _lib.U32, torch.int32: _lib.I32,
+}
+
+
+def _arr(t: torch.Tensor) -> Array:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError("expected a torch.Tensor")
+    if t.dtype not in _DTYPES:
+        raise T3Error(2)  # BadExl3Dtype
+    if t.dim() > _lib.T3_MAX_DIMS:
+        raise T3Error(1)
+    if not t.is_cuda:
+        raise ValueError("turboexl3_amd runs on device tensors only")
+    if not t.is_contiguous():
+        t = t.contiguous()
+    a = Array()
+    a.data = t.data_ptr()
+    a.ndim = t.dim()
+    a.dtype = _DTYPES[t.dtype]
+    for i, d in enumerate(t.shape):
+        a.shape[i] = d
+    a._keep = t
+    return a
+
+
+def _check(status: int) -> None:
+    if status != 0:
+        raise T3Error(status)
+
+
+def _stream_ptr(stream) -> int:
+    s = torch.cuda.current_stream() if stream is None else stream
+    return s.cuda_stream
+
+
+_workspaces: dict = {}
+
+
+def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+    """A grow-only scratch buffer per device (the caller of the C ABI owns scratch; this harness keeps one)."""
+    key = (device.type, device.index)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def configure(**fields) -> None:
+    """root.configure: set once before the first call; an unserved value raises InvalidTurboexl3Config."""
+    cfg = Config()
+    _lib.lib().t3_config_default(C.byref(cfg))
+    for k, v in fields.items():
+        if not hasattr(cfg, k):
+            raise T3Error(10)
+        setattr(cfg, k, int(v))
+    _check(_lib.lib().t3_configure(C.byref(cfg)))
+
+
+def release_engines() -> None:
+    _lib.lib().t3_release_engines()
+
+
+def _linear(entry, x, trellis, suh, svh, dec: Decode, stream=None) -> torch.Tensor:
+    L = _lib.lib()
+    ax, at, asu, asv = _arr(x), _arr(trellis), _arr(suh), _arr(svh)
+    need = C.c_size_t(0)
+    _check(L.t3_linear_workspace_bytes(C.byref(ax), C.byref(at), dec.c(), C.byref(need)))
+    out_dim = trellis.shape[1] * 16
+    y = torch.empty(*x.shape[:-1], out_dim, dtype=x.dtype, device=x.device)
+    ay = _arr(y)
+    ws = _workspace(x.device, need.value)
+    _check(entry(_stream_ptr(stream), C.byref(ax), C.byref(at), C.byref(asu), C.byref(asv), dec.c(), C.byref(ay),
+                 ws.data_ptr(), ws.numel()))
+    return y
+
+
+def linear(x, trellis, suh, svh, dec: Decode = Decode.mul1, stream=None) -> torch.Tensor:
+    """root.linear: y [..., out] in x's dtype for x [..., in]."""
+    return _linear(_lib.lib().t3_linear, x, trellis, suh, svh, dec, stream)
+
+
+def linear_chain(x, trellis, suh, svh, dec: Decode = Decode.mul1, stream=None) -> torch.Tensor:
+    """The three-launch chain `linear`'s fused launch must equal byte for byte."""
+    return _linear(_lib.lib().t3_linear_chain, x, trellis, suh, svh, dec, stream)
+
+
+def dequant(trellis, dec: Decode = Decode.mul1, stream=None) -> torch.Tensor:
+    """W_hat f16 [in, out]: format.reconstructInner on the device, bit-exact."""
+    at = _arr(trellis)
+    if trellis.dim() != 3:
+        raise T3Error(1)
+    w = torch.empty(trellis.shape[0] * 16, trellis.shape[1] * 16, dtype=torch.float16, device=trellis.device)
+    aw = _arr(w)
+    _check(_lib.lib().t3_dequant(_stream_ptr(stream), C.byref(at), dec.c(), C.byref(aw)))
+    return w
+
+
+def _cbank(bank: Bank):
+    keep = []
+
+    def proj(p: Proj) -> CProj:
+        a = (_arr(p.trellis), _arr(p.suh), _arr(p.svh))
+        keep.append(a)
+        return CProj(*a)
+
+    return CBank(proj(bank.gate), proj(bank.up), proj(bank.down)), keep
+
+
+def _moe_workspace(L, ax, cb, ai, device):
+    need = C.c_size_t(0)
+    _check(L.t3_moe_workspace_bytes(C.byref(ax), C.byref(cb), C.byref(ai), C.byref(need)))
+    return _workspace(device, need.value)
+
+
+def moe(x, bank: Bank, inds, scores, dec: Decode = Decode.mul1, verify_rows: bool = False, stream=None) -> torch.Tensor:
+    """root.moe: routed SwiGLU experts over x [B, S, D] for inds/scores [B, S, K]."""
+    L = _lib.lib()
+    ax, ai, asc = _arr(x), _arr(inds), _arr(scores)
+    cb, _keep = _cbank(bank)
+    ws = _moe_workspace(L, ax, cb, ai, x.device)
+    y = torch.empty_like(x)
+    ay = _arr(y)
+    _check(L.t3_moe(_stream_ptr(stream), C.byref(ax), C.byref(cb), C.byref(ai), C.byref(asc), dec.c(),
+                    int(verify_rows), C.byref(ay), ws.data_ptr(), ws.numel()))
+    return y
+
+
+def moe_clamped(x, bank: Bank, inds, scores, dec: Decode, limit: int, stream=None) -> torch.Tensor:
+    """root.moeClamped: gate clamped from above, up to [-limit, limit]; limit 1..128."""
+    L = _lib.lib()
+    ax, ai, asc = _arr(x), _arr(inds), _arr(scores)
+    cb, _keep = _cbank(bank)
+    if not (0 < int(limit) <= 128):
+        raise T3Error(6)
+    ws = _moe_workspace(L, ax, cb, ai, x.device)
+    y = torch.empty_like(x)
+    ay = _arr(y)
+    _check(L.t3_moe_clamped(_stream_ptr(stream), C.byref(ax), C.byref(cb), C.byref(ai), C.byref(asc), dec.c(),
+                            int(limit), C.byref(ay), ws.data_ptr(), ws.numel()))
+    return y
+
+
+def moe_with_shared(x, bank: Bank, inds, scores, dec: Decode, verify_rows: bool, shared, stream=None) -> torch.Tensor:
+    """root.moeWithShared: `moe` plus an already gated shared-expert output of x's shape and dtype."""
+    L = _lib.lib()
+    ax, ai, asc, ash = _arr(x), _arr(inds), _arr(scores), _arr(shared)
+    cb, _keep = _cbank(bank)
+    ws = _moe_workspace(L, ax, cb, ai, x.device)
+    y = torch.empty_like(x)
+    ay = _arr(y)
+    _check(L.t3_moe_with_shared(_stream_ptr(stream), C.byref(ax), C.byref(cb), C.byref(ai), C.byref(asc), dec.c(),
+                                int(verify_rows), C.byref(ash), C.byref(ay), ws.data_ptr(), ws.numel()))
+    return y
+
+
+# ---- device self-tests -------------------------------------------------------------------------------------
+
+def test_codebooks(device="cuda"):
+    mcg = torch.empty(65536, dtype=torch.int16, device=device)
+    mul1 = torch.empty_like(mcg)
+    t = torch.empty_like(mcg)
+    _check(_lib.lib().t3_test_codebooks(_stream_ptr(None), mcg.data_ptr(), mul1.data_ptr(), t.data_ptr()))
+    return mcg, mul1, t
+
+
+def test_lane(trellis: torch.Tensor, n: int, window_bits: int):
+    tiles = trellis.numel() // n
+    cw = torch.empty(tiles, 256, dtype=torch.int16, device=trellis.device)
+    mcg = torch.empty_like(cw)
+    mul1 = torch.empty_like(cw)
+    _check(_lib.lib().t3_test_lane(_stream_ptr(None), trellis.data_ptr(), n, window_bits, tiles, cw.data_ptr(),
+                                   mcg.data_ptr(), mul1.data_ptr()))
+    return cw, mcg, mul1
+
+
+def test_mfma(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    d = torch.empty(16, 16, dtype=torch.float32, device=a.device)
+    _check(_lib.lib().t3_test_mfma(_stream_ptr(None), a.data_ptr(), b.data_ptr(), d.data_ptr()))
+    return d

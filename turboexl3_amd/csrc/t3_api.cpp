@@ -1,0 +1,100 @@
+// The C ABI of the gfx950 EXL3 projection engine (include/turboexl3_hip.h): validation with the reference's refusal
+// names, this library's launch partitions and workspace layout, and the launches. Host logic only; the kernels live in
+// the .hip files beside this one.
+
+#include "../../include/turboexl3_hip.h"
+
+#include <atomic>
+#include <cstring>
+
+#include "t3_host.hpp"
+
+namespace {
+
+std::atomic<bool> g_configured{false};
+t3_config g_config = {9, 1, 1, 1, 1};
+
+}  // namespace
+
+namespace t3 {
+
+const t3_config& config() { return g_config; }
+
+}  // namespace t3
+
+extern "C" {
+
+const char* t3_error_name(int32_t status) {
+    switch (status) {
+        case T3_OK: return "ok";
+        case T3_BadExl3Shape: return "BadExl3Shape";
+        case T3_BadExl3Dtype: return "BadExl3Dtype";
+        case T3_Exl3EngineNotImplemented: return "Exl3EngineNotImplemented";
+        case T3_Exl3EngineCacheFull: return "Exl3EngineCacheFull";
+        case T3_Exl3GateUpRateMismatch: return "Exl3GateUpRateMismatch";
+        case T3_InvalidExl3Clamp: return "InvalidExl3Clamp";
+        case T3_Exl3TopKExceedsReduceBank: return "Exl3TopKExceedsReduceBank";
+        case T3_Exl3WindowUnsupported: return "Exl3WindowUnsupported";
+        case T3_ExpertLayoutUnsupported: return "ExpertLayoutUnsupported";
+        case T3_InvalidTurboexl3Config: return "InvalidTurboexl3Config";
+        case T3_WorkspaceTooSmall: return "WorkspaceTooSmall";
+        case T3_HipFailed: return "HipFailed";
+        case T3_BadArgs: return "BadArgs";
+        default: return "UnknownStatus";
+    }
+}
+
+void t3_config_default(t3_config* out) {
+    if (!out) return;
+    const t3_config d = {9, 1, 1, 1, 1};
+    *out = d;
+}
+
+int32_t t3_configure(const t3_config* cfg) {
+    if (!cfg) return T3_BadArgs;
+    const bool flags_ok = (cfg->dec_one == 0 || cfg->dec_one == 1) && (cfg->prefill == 0 || cfg->prefill == 1) &&
+                          (cfg->mcg_pair == 0 || cfg->mcg_pair == 1) && (cfg->mul1_defer == 0 || cfg->mul1_defer == 1);
+    if ((cfg->decode_form != 3 && cfg->decode_form != 9) || !flags_ok) return T3_InvalidTurboexl3Config;
+    g_config = *cfg;
+    g_configured.store(true);
+    return T3_OK;
+}
+
+void t3_release_engines(void) {}
+
+int32_t t3_rate_admitted(int64_t n) { return t3::rate_ok(n) ? 1 : 0; }
+
+int32_t t3_admit_topk(int64_t topk) { return topk > T3_REDUCE_MAX_TOPK ? T3_Exl3TopKExceedsReduceBank : T3_OK; }
+
+int32_t t3_trellis_admitted(const int64_t* shape, int32_t ndim, int64_t experts, int64_t in_dim, int64_t out_dim,
+                            int64_t n_max) {
+    if (!shape || ndim != 4) return 0;
+    for (int i = 0; i < 4; ++i)
+        if (shape[i] <= 0) return 0;
+    if (in_dim % 16 != 0 || out_dim % 16 != 0) return 0;
+    if (shape[0] != experts || shape[1] != in_dim / 16 || shape[2] != out_dim / 16) return 0;
+    if (!t3::rate_ok(shape[3])) return 0;
+    return shape[3] <= n_max ? 1 : 0;
+}
+
+int32_t t3_test_codebooks(t3_stream stream, uint16_t* mcg, uint16_t* mul1, uint16_t* t) {
+    if (!mcg || !mul1 || !t) return T3_BadArgs;
+    return t3::hip_status(t3::launch_test_codebooks(mcg, mul1, t, static_cast<hipStream_t>(stream)));
+}
+
+int32_t t3_test_lane(t3_stream stream, const uint16_t* trellis, int64_t n, int32_t window_bits, int64_t tiles,
+                     uint16_t* cw, uint16_t* mcg, uint16_t* mul1) {
+    if (!trellis || !cw || !mcg || !mul1) return T3_BadArgs;
+    if (!t3::rate_ok(n) || tiles <= 0 || tiles > (1 << 24)) return T3_BadExl3Shape;
+    if (window_bits < 8 || window_bits > 16) return T3_Exl3WindowUnsupported;
+    return t3::hip_status(t3::launch_test_lane(reinterpret_cast<const uint32_t*>(trellis), static_cast<uint32_t>(n),
+                                               static_cast<uint32_t>(window_bits), static_cast<uint32_t>(tiles), cw, mcg,
+                                               mul1, static_cast<hipStream_t>(stream)));
+}
+
+int32_t t3_test_mfma(t3_stream stream, const uint16_t* a, const uint16_t* b, float* d) {
+    if (!a || !b || !d) return T3_BadArgs;
+    return t3::hip_status(t3::launch_test_mfma(a, b, d, static_cast<hipStream_t>(stream)));
+}
+
+}  // extern "C"

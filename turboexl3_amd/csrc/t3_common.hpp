@@ -1,0 +1,97 @@
+// Shared device helpers of the gfx950 EXL3 kernels: dtypes, f16/bf16 conversions, the 128-point Hadamard of one
+// wave64, and the constants of the format (turboexl3 src/core/format.zig:10-16).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace t3 {
+
+// activation numbering shared with the C ABI (turboexl3 src/hip/plan.zig:72-73)
+enum Dtype : int { kF32 = 0, kF16 = 1, kBf16 = 2 };
+
+constexpr float kHadScale = 0.08838834764831845f;  // 1 / sqrt(128)
+constexpr int kWave = 64;
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+
+// A raw buffer over `bytes` bytes from p: loads take a per-lane byte offset (VGPR) plus a uniform byte offset (SGPR),
+// so a streaming loop spends no vector ALU on addresses, and a read past the end returns zero instead of faulting.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint64_t bytes) {
+    const uint32_t n = bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : static_cast<uint32_t>(bytes);
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, static_cast<int>(n), 0x00020000);
+}
+__device__ __forceinline__ uint32_t buf_load_u32(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+    return __builtin_amdgcn_raw_buffer_load_b32(r, static_cast<int>(voff), static_cast<int>(soff), 0);
+}
+__device__ __forceinline__ uint4v buf_load_u128(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, static_cast<int>(voff), static_cast<int>(soff), 0);
+}
+
+__device__ __forceinline__ float half_value(uint32_t bits) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(bits)));
+}
+__device__ __forceinline__ uint16_t half_bits(float v) {
+    return __builtin_bit_cast(uint16_t, static_cast<_Float16>(v));
+}
+__device__ __forceinline__ float round_half(float v) { return half_value(half_bits(v)); }
+
+__device__ __forceinline__ float bf16_value(uint16_t b) {
+    return __builtin_bit_cast(float, static_cast<uint32_t>(b) << 16);
+}
+// f32 -> bf16, nearest even; a NaN stays a (quiet) NaN
+__device__ __forceinline__ uint16_t bf16_bits(float v) {
+    uint32_t u = __builtin_bit_cast(uint32_t, v);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return static_cast<uint16_t>(u >> 16);
+}
+
+template <int DT>
+__device__ __forceinline__ float load_act(const void* p, size_t i) {
+    if constexpr (DT == kF32) return static_cast<const float*>(p)[i];
+    else if constexpr (DT == kF16) return half_value(static_cast<const uint16_t*>(p)[i]);
+    else return bf16_value(static_cast<const uint16_t*>(p)[i]);
+}
+template <int DT>
+__device__ __forceinline__ void store_act(void* p, size_t i, float v) {
+    if constexpr (DT == kF32) static_cast<float*>(p)[i] = v;
+    else if constexpr (DT == kF16) static_cast<uint16_t*>(p)[i] = half_bits(v);
+    else static_cast<uint16_t*>(p)[i] = bf16_bits(v);
+}
+
+// The unscaled Hadamard of a 128-block held by one wave64: lane L owns elements L and L + 64 (v[0], v[1]).
+// Six cross-lane stages over element bits 0..5, then the lane's own stage over bit 6. The stage order is fixed: every
+// kernel that transforms a block uses this function, so a block's bits do not depend on which kernel transformed it.
+__device__ __forceinline__ void h128_wave(float (&v)[2], uint32_t lane) {
+#pragma unroll
+    for (uint32_t s = 0; s < 6u; ++s) {
+        const uint32_t bit = 1u << s;
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j) {
+            const float p = __shfl_xor(v[j], static_cast<int>(bit), 64);
+            v[j] = (lane & bit) ? (p - v[j]) : (v[j] + p);
+        }
+    }
+    const float a = v[0] + v[1], b = v[0] - v[1];
+    v[0] = a;
+    v[1] = b;
+}
+
+// Slot of element r (0..15) of a 16-input tile in "quad order": the four inputs a lane's weights multiply,
+// tile rows 2q + {0, 1, 8, 9}, sit at slots 4q..4q+3 (turboexl3 src/kernels/hip/common.hpp:70-75 uses the same order).
+__device__ __forceinline__ uint32_t quad_slot(uint32_t r) {
+    const uint32_t q = (r & 7u) >> 1u;
+    const uint32_t m = (r & 1u) | ((r >> 3u) << 1u);
+    return 4u * q + m;
+}
+
+// MUL1's affine map w = A h + B with h = 1024 + t (format.zig:158-167): A = f16 0x1EEE, B = f16 0xC931
+__device__ __forceinline__ float mul1_a() { return half_value(0x1EEEu); }
+__device__ __forceinline__ float mul1_b() { return half_value(0xC931u); }
+
+}  // namespace t3

@@ -1,0 +1,106 @@
+// W_hat: the trellis decoded to f16 [in][out], bit-exact to format.reconstructInner (turboexl3
+// src/core/format.zig:276-291), and the test kernels that pin the reader and the codebooks on the device
+// (the roles of turboexl3 src/kernels/hip/test/lane.hip's two kernels).
+
+#include "t3_decode.hpp"
+#include "t3_kernels.hpp"
+
+namespace t3 {
+namespace {
+
+// Grid (out / 64, in / 16), 256 threads: wave sg decodes tile (tk, 4 blockIdx.x + sg); the four tiles' rows leave
+// through LDS as 128-byte row segments.
+template <int CB, bool WIDE>
+__global__ void __launch_bounds__(256) dequant_kernel(const uint32_t* __restrict__ w, uint16_t* __restrict__ w_hat,
+                                                      uint32_t out, uint32_t n, uint32_t wbits) {
+    __shared__ __attribute__((aligned(16))) uint16_t stage[16][64 + 8];
+    const uint32_t sg = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+    const uint32_t tk = blockIdx.y, tn = blockIdx.x * 4u + sg;
+    const uint32_t out_tiles = out >> 4, nw = n >> 1;
+    const QuadPlan<WIDE> plan = quad_plan<WIDE>(n, lane);
+    const QuadWords<WIDE> words = quad_load<WIDE>(w + (static_cast<size_t>(tk) * out_tiles + tn) * nw, plan);
+    uint32_t cw[4];
+    quad_codewords<WIDE>(words, plan, wbits, cw);
+#pragma unroll
+    for (uint32_t m = 0; m < 4u; ++m) stage[quad_row(lane, m)][sg * 16u + quad_col(lane)] = decode_exact<CB>(cw[m]);
+    __syncthreads();
+    const uint32_t r = threadIdx.x >> 4, c4 = (threadIdx.x & 15u) * 4u;
+    const uint2 v = *reinterpret_cast<const uint2*>(&stage[r][c4]);
+    *reinterpret_cast<uint2*>(w_hat + (static_cast<size_t>(tk) * 16u + r) * out + blockIdx.x * 64u + c4) = v;
+}
+
+__global__ void __launch_bounds__(256) test_codebooks_kernel(uint16_t* mcg, uint16_t* mul1, uint16_t* t) {
+    const uint32_t cw = blockIdx.x * 256u + threadIdx.x;
+    mcg[cw] = decode_mcg(cw);
+    mul1[cw] = decode_mul1(cw);
+    t[cw] = static_cast<uint16_t>(mul1_t(cw));
+}
+
+// Grid (tiles), 64 threads: the quad reader's codewords by code position and both codebooks' values of them.
+template <bool WIDE>
+__global__ void __launch_bounds__(64) test_lane_kernel(const uint32_t* trellis, uint32_t n, uint32_t wbits,
+                                                       uint16_t* cw_out, uint16_t* mcg, uint16_t* mul1) {
+    const uint32_t lane = threadIdx.x, tile = blockIdx.x;
+    const QuadPlan<WIDE> plan = quad_plan<WIDE>(n, lane);
+    const QuadWords<WIDE> words = quad_load<WIDE>(trellis + static_cast<size_t>(tile) * (n >> 1), plan);
+    uint32_t cw[4];
+    quad_codewords<WIDE>(words, plan, wbits, cw);
+    const uint32_t p = quad_first_position(lane);
+#pragma unroll
+    for (uint32_t m = 0; m < 4u; ++m) {
+        const size_t at = static_cast<size_t>(tile) * 256u + p + m;
+        cw_out[at] = static_cast<uint16_t>(cw[m]);
+        mcg[at] = decode_mcg(cw[m]);
+        mul1[at] = decode_mul1(cw[m]);
+    }
+}
+
+// One wave: D [16][16] = A [16][32] B [32][16] (row-major f16 in, f32 out) with the GEMV's fragment assumptions:
+// lane l supplies A[l % 16][8 (l / 16) .. + 7] and B[8 (l / 16) .. + 7][l % 16], and receives D[4 (l / 16) + r][l % 16].
+__global__ void __launch_bounds__(64) test_mfma_kernel(const uint16_t* a, const uint16_t* b, float* d) {
+    const uint32_t lane = threadIdx.x, i = lane & 15u, g = lane >> 4;
+    half8 av, bv;
+#pragma unroll
+    for (uint32_t k = 0; k < 8u; ++k) {
+        av[k] = __builtin_bit_cast(_Float16, a[i * 32u + 8u * g + k]);
+        bv[k] = __builtin_bit_cast(_Float16, b[(8u * g + k) * 16u + i]);
+    }
+    float4v acc = {0.f, 0.f, 0.f, 0.f};
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bv, acc, 0, 0, 0);
+#pragma unroll
+    for (uint32_t r = 0; r < 4u; ++r) d[(4u * g + r) * 16u + i] = acc[r];
+}
+
+}  // namespace
+
+hipError_t launch_dequant(const uint32_t* trellis, uint16_t* w_hat, uint32_t in, uint32_t out, uint32_t n,
+                          uint32_t wbits, int codebook, hipStream_t s) {
+    const dim3 grid(out / 64u, in / 16u), block(256);
+    const bool wide = quad_needs_wide(n);
+    const bool mcg = codebook == kMcg || codebook == kMcgPair;
+    if (mcg && wide) hipLaunchKernelGGL((dequant_kernel<kMcg, true>), grid, block, 0, s, trellis, w_hat, out, n, wbits);
+    else if (mcg) hipLaunchKernelGGL((dequant_kernel<kMcg, false>), grid, block, 0, s, trellis, w_hat, out, n, wbits);
+    else if (wide) hipLaunchKernelGGL((dequant_kernel<kMul1, true>), grid, block, 0, s, trellis, w_hat, out, n, wbits);
+    else hipLaunchKernelGGL((dequant_kernel<kMul1, false>), grid, block, 0, s, trellis, w_hat, out, n, wbits);
+    return hipGetLastError();
+}
+
+hipError_t launch_test_codebooks(uint16_t* mcg, uint16_t* mul1, uint16_t* t, hipStream_t s) {
+    hipLaunchKernelGGL(test_codebooks_kernel, dim3(256), dim3(256), 0, s, mcg, mul1, t);
+    return hipGetLastError();
+}
+
+hipError_t launch_test_lane(const uint32_t* trellis, uint32_t n, uint32_t wbits, uint32_t tiles, uint16_t* cw,
+                            uint16_t* mcg, uint16_t* mul1, hipStream_t s) {
+    if (quad_needs_wide(n))
+        hipLaunchKernelGGL(test_lane_kernel<true>, dim3(tiles), dim3(64), 0, s, trellis, n, wbits, cw, mcg, mul1);
+    else hipLaunchKernelGGL(test_lane_kernel<false>, dim3(tiles), dim3(64), 0, s, trellis, n, wbits, cw, mcg, mul1);
+    return hipGetLastError();
+}
+
+hipError_t launch_test_mfma(const uint16_t* a, const uint16_t* b, float* d, hipStream_t s) {
+    hipLaunchKernelGGL(test_mfma_kernel, dim3(1), dim3(64), 0, s, a, b, d);
+    return hipGetLastError();
+}
+
+}  // namespace t3

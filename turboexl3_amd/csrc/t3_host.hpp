@@ -1,0 +1,82 @@
+// Host-side helpers shared by the C ABI's translation units: descriptor checks, the decode descriptor, workspace
+// carving and this library's launch partitions.
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+
+#include "../../include/turboexl3_hip.h"
+#include "t3_kernels.hpp"
+
+namespace t3 {
+
+const t3_config& config();
+
+inline bool rate_ok(int64_t n) { return n % 2 == 0 && n >= 16 && n <= 128; }
+
+inline int32_t hip_status(hipError_t e) { return e == hipSuccess ? T3_OK : T3_HipFailed; }
+
+inline bool array_ok(const t3_array* a) {
+    if (!a || !a->data || a->ndim < 0 || a->ndim > T3_MAX_DIMS) return false;
+    for (int i = 0; i < a->ndim; ++i)
+        if (a->shape[i] < 0) return false;
+    return true;
+}
+
+inline bool is_act_dtype(int32_t d) { return d == T3_F32 || d == T3_F16 || d == T3_BF16; }
+inline size_t dtype_size(int32_t d) { return d == T3_F32 || d == T3_U32 || d == T3_I32 ? 4 : 2; }
+
+// The decode a call runs with: the reference's (codebook, window) plus this library's GEMV-only codebook forms.
+struct Dec {
+    int codebook;    // t3::Codebook numbering for exact decode (0 MUL1, 1 MCG)
+    int gemv_form;   // the codebook the GEMV kernels run: exact, or kMul1Defer / kMcgPair by configuration
+    uint32_t wbits;
+};
+
+inline int32_t resolve_decode(t3_decode dec, Dec* out) {
+    if (dec.codebook != 0 && dec.codebook != 1) return T3_BadArgs;
+    if (dec.window_bits < 8 || dec.window_bits > 16) return T3_Exl3WindowUnsupported;
+    out->codebook = dec.codebook;
+    out->wbits = static_cast<uint32_t>(dec.window_bits);
+    if (dec.codebook == 1) out->gemv_form = config().mcg_pair ? 3 : 1;
+    else out->gemv_form = config().mul1_defer ? 2 : 0;
+    return T3_OK;
+}
+
+// Scratch carved from the caller's workspace in 256-byte steps.
+struct Carver {
+    unsigned char* base;
+    size_t used = 0;
+    explicit Carver(void* p) : base(static_cast<unsigned char*>(p)) {}
+    template <typename T>
+    T* take(size_t bytes) {
+        T* p = base ? reinterpret_cast<T*>(base + used) : nullptr;
+        used += (bytes + 255u) & ~static_cast<size_t>(255u);
+        return p;
+    }
+};
+
+// ---- partitions -----------------------------------------------------------------------------------------------
+// The K split of a GEMV depends on the matrix's shape alone, never on the rows of a call, so a row's sums (and bytes)
+// are those of the row alone. The reference fixes its split the same way (turboexl3 src/core/dense.zig:553-562); the
+// numbers here are sized for 256 CUs, not for its 40-core target.
+
+constexpr uint32_t kGemvBt = 4;          // output tiles a wave
+constexpr uint32_t kGemvTargetWgs = 768; // three workgroups a CU
+constexpr uint32_t kGemvMinPer = 4;      // input tiles a wave at least
+
+// K slices of a GEMV over in_tiles input tiles and `groups` workgroup columns: the smallest divisor d of
+// in_tiles / 4 that reaches the target workgroup count while every wave keeps kGemvMinPer tiles.
+inline uint32_t gemv_slices(uint32_t in_tiles, uint32_t groups) {
+    const uint32_t q = in_tiles / 4u;
+    uint32_t best = 1;
+    for (uint32_t d = 1; d <= q; ++d) {
+        if (q % d != 0) continue;
+        if (q / d < kGemvMinPer && d > 1) break;
+        best = d;
+        if (static_cast<uint64_t>(groups) * d >= kGemvTargetWgs) break;
+    }
+    return best;
+}
+
+}  // namespace t3

@@ -1,0 +1,127 @@
+// `linear`: one dense EXL3 projection (turboexl3 src/root.zig:309-351), its chain form, and W_hat's decode.
+
+#include "t3_host.hpp"
+
+namespace t3 {
+namespace {
+
+struct DenseCall {
+    DenseLaunch launch;
+    size_t workspace = 0;
+};
+
+// root.linearOn's operand checks (src/root.zig:326-341), the loader's dtype rules (table/table.zig:129-145) and the
+// dense plan's shape rule (src/hip/plan.zig:125-129).
+int32_t check_dense(const t3_array* x, const t3_array* trellis, const t3_array* suh, const t3_array* svh,
+                    t3_decode dec, const t3_array* y, uint32_t max_rows, DenseCall* call) {
+    if (!array_ok(x) || !array_ok(trellis) || (suh && !array_ok(suh)) || (svh && !array_ok(svh)) || (y && !array_ok(y)))
+        return T3_BadArgs;
+    if (x->ndim < 1 || trellis->ndim != 3) return T3_BadExl3Shape;
+    const int64_t in = trellis->shape[0] * 16, out = trellis->shape[1] * 16, n = trellis->shape[2];
+    if (!rate_ok(n)) return T3_BadExl3Shape;
+    if (in <= 0 || out <= 0 || in % 128 != 0 || out % 128 != 0 || in > (1ll << 30) || out > (1ll << 30))
+        return T3_BadExl3Shape;
+    if (x->shape[x->ndim - 1] != in) return T3_BadExl3Shape;
+    if (suh && (suh->ndim < 1 || suh->shape[0] != in)) return T3_BadExl3Shape;
+    if (svh && (svh->ndim < 1 || svh->shape[0] != out)) return T3_BadExl3Shape;
+    if (!is_act_dtype(x->dtype)) return T3_BadExl3Dtype;
+    if (trellis->dtype != T3_U16 && trellis->dtype != T3_I16) return T3_BadExl3Dtype;
+    if ((suh && suh->dtype != T3_F16) || (svh && svh->dtype != T3_F16)) return T3_BadExl3Dtype;
+    int64_t rows = 1;
+    for (int i = 0; i + 1 < x->ndim; ++i) {
+        rows *= x->shape[i];
+        if (rows > (1ll << 30)) return T3_BadExl3Shape;
+    }
+    if (rows < 1) return T3_BadExl3Shape;
+    if (y) {
+        if (y->ndim != x->ndim || y->shape[y->ndim - 1] != out) return T3_BadExl3Shape;
+        for (int i = 0; i + 1 < x->ndim; ++i)
+            if (y->shape[i] != x->shape[i]) return T3_BadExl3Shape;
+        if (y->dtype != x->dtype) return T3_BadExl3Dtype;
+    }
+    Dec d;
+    if (const int32_t st = resolve_decode(dec, &d); st != T3_OK) return st;
+    if (max_rows != 0 && rows > max_rows) return T3_Exl3EngineNotImplemented;
+
+    DenseLaunch& l = call->launch;
+    l.x = x->data;
+    l.suh = suh ? static_cast<const uint16_t*>(suh->data) : nullptr;
+    l.svh = svh ? static_cast<const uint16_t*>(svh->data) : nullptr;
+    l.trellis = static_cast<const uint32_t*>(trellis->data);
+    l.y = y ? y->data : nullptr;
+    l.in = static_cast<uint32_t>(in);
+    l.out = static_cast<uint32_t>(out);
+    l.rows = static_cast<uint32_t>(rows);
+    l.n = static_cast<uint32_t>(n);
+    l.wbits = d.wbits;
+    l.codebook = d.gemv_form;
+    l.dtype = x->dtype;
+    l.bt = kGemvBt;
+    l.ks = gemv_slices(l.in / 16u, (l.out / 16u) / l.bt);
+    return T3_OK;
+}
+
+// xq u32 [rows][in], xs f32 [rows][in / 128], z f32 [ks][rows][out], arrival counters u32 [out / 128]
+void carve_dense(DenseCall* call, void* workspace) {
+    DenseLaunch& l = call->launch;
+    Carver c(workspace);
+    l.xq = c.take<uint32_t>(static_cast<size_t>(l.rows) * l.in * 4u);
+    l.xs = c.take<float>(static_cast<size_t>(l.rows) * (l.in / 128u) * 4u);
+    l.z = c.take<float>(static_cast<size_t>(l.ks) * l.rows * l.out * 4u);
+    l.arrive = c.take<uint32_t>(static_cast<size_t>(l.out / 128u) * 4u);
+    call->workspace = c.used;
+}
+
+int32_t run_chain(const DenseCall& call, hipStream_t s) {
+    if (const int32_t st = hip_status(launch_dense_prep(call.launch, s)); st != T3_OK) return st;
+    if (const int32_t st = hip_status(launch_dense_gemv(call.launch, s)); st != T3_OK) return st;
+    return hip_status(launch_dense_finish(call.launch, s));
+}
+
+}  // namespace
+}  // namespace t3
+
+extern "C" {
+
+int32_t t3_linear_workspace_bytes(const t3_array* x, const t3_array* trellis, t3_decode dec, size_t* bytes) {
+    if (!bytes) return T3_BadArgs;
+    t3::DenseCall call;
+    if (const int32_t st = t3::check_dense(x, trellis, nullptr, nullptr, dec, nullptr, 32, &call); st != T3_OK) return st;
+    t3::carve_dense(&call, nullptr);
+    *bytes = call.workspace;
+    return T3_OK;
+}
+
+int32_t t3_linear_chain(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
+                        const t3_array* svh, t3_decode dec, t3_array* y, void* workspace, size_t workspace_bytes) {
+    if (!suh || !svh || !y) return T3_BadArgs;
+    t3::DenseCall call;
+    if (const int32_t st = t3::check_dense(x, trellis, suh, svh, dec, y, 32, &call); st != T3_OK) return st;
+    if (!workspace) return T3_BadArgs;
+    t3::carve_dense(&call, workspace);
+    if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
+    return t3::run_chain(call, static_cast<hipStream_t>(stream));
+}
+
+int32_t t3_linear(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
+                  const t3_array* svh, t3_decode dec, t3_array* y, void* workspace, size_t workspace_bytes) {
+    return t3_linear_chain(stream, x, trellis, suh, svh, dec, y, workspace, workspace_bytes);
+}
+
+int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_array* w_hat) {
+    if (!t3::array_ok(trellis) || !t3::array_ok(w_hat)) return T3_BadArgs;
+    if (trellis->ndim != 3 || w_hat->ndim != 2) return T3_BadExl3Shape;
+    const int64_t in = trellis->shape[0] * 16, out = trellis->shape[1] * 16, n = trellis->shape[2];
+    if (!t3::rate_ok(n) || in <= 0 || out <= 0 || out % 64 != 0 || in > (1ll << 30) || out > (1ll << 30))
+        return T3_BadExl3Shape;
+    if (w_hat->shape[0] != in || w_hat->shape[1] != out) return T3_BadExl3Shape;
+    if ((trellis->dtype != T3_U16 && trellis->dtype != T3_I16) || w_hat->dtype != T3_F16) return T3_BadExl3Dtype;
+    t3::Dec d;
+    if (const int32_t st = t3::resolve_decode(dec, &d); st != T3_OK) return st;
+    return t3::hip_status(t3::launch_dequant(static_cast<const uint32_t*>(trellis->data),
+                                             static_cast<uint16_t*>(w_hat->data), static_cast<uint32_t>(in),
+                                             static_cast<uint32_t>(out), static_cast<uint32_t>(n), d.wbits, d.codebook,
+                                             static_cast<hipStream_t>(stream)));
+}
+
+}  // extern "C"
