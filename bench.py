@@ -1,0 +1,195 @@
+#!/usr/bin/env python3
+"""Benchmark of the EXL3 projection path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sweep]
+
+A step is one `linear` call of the dense decode-row GEMV workload BASELINE.json quotes its metric on
+(in=4096, out=12288, K=4 bits/weight, 1 row, MCG codebook, f16 activations with 1 % outliers x20; synthetic seeded
+codes). Calls rotate over enough distinct weight copies (> 512 MB in total) that every call reads its codes from
+HBM, not from the 256 MB Infinity Cache. Inputs are resident in HBM before the timed region starts.
+
+Prints ONE JSON line: the whole-call rate as GB/s of trellis code bytes (`value`), the dominant kernel's roofline
+(`roofline`: algorithmic code bytes of one launch / its average duration, timed alone with HIP events on the launch
+stream, against 8 TB/s), and the CPU oracle (`format.project` restated in C) timed on this box's host cores
+(`cpu_baseline`). `--sweep` adds K = 3, 4, 5 x rows = 1, 4, 16, 32.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+IN_F, OUT_F = 4096, 12288
+HBM_PEAK = 8.0e12
+MIN_ROTATION_BYTES = 512 << 20
+
+
+def code_bytes(in_f: int, out_f: int, n: int) -> int:
+    """Algorithmic bytes of one projection: (in/16)(out/16) tiles of n halfwords."""
+    return (in_f // 16) * (out_f // 16) * n * 2
+
+
+def make_weights(torch, n: int, copies: int, seed: int):
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    trellis = torch.randint(-32768, 32768, (copies, IN_F // 16, OUT_F // 16, n), dtype=torch.int16, device="cuda",
+                            generator=g)
+    sign = lambda k: (torch.randint(0, 2, (k,), device="cuda", generator=g) * 2 - 1).to(torch.float32)
+    suh = (sign(IN_F) * (1.0 + 0.1 * torch.randn(IN_F, device="cuda", generator=g))).to(torch.float16)
+    svh = (sign(OUT_F) * (1.0 + 0.1 * torch.randn(OUT_F, device="cuda", generator=g)) / (IN_F ** 0.5)).to(torch.float16)
+    return trellis, suh, svh
+
+
+def make_x(torch, rows: int, seed: int):
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    x = torch.randn(rows, IN_F, device="cuda", generator=g)
+    outl = torch.rand(rows, IN_F, device="cuda", generator=g) < 0.01
+    return torch.where(outl, x * 20.0, x).to(torch.float16)
+
+
+class DenseRunner:
+    """Pre-built descriptors for back-to-back C-ABI calls: nothing is allocated inside the timed region."""
+
+    def __init__(self, torch, api, trellis, suh, svh, x, dec):
+        import ctypes as C
+
+        from turboexl3_amd import _lib
+        self.C, self.L, self.torch = C, _lib.lib(), torch
+        self.copies = trellis.shape[0]
+        self.dec = dec.c()
+        self.ax = api._arr(x)
+        self.at = [api._arr(trellis[i]) for i in range(self.copies)]
+        self.asu, self.asv = api._arr(suh), api._arr(svh)
+        self.y = torch.empty(x.shape[0], OUT_F, dtype=x.dtype, device="cuda")
+        self.ay = api._arr(self.y)
+        need = C.c_size_t(0)
+        st = self.L.t3_linear_workspace_bytes(C.byref(self.ax), C.byref(self.at[0]), self.dec, C.byref(need))
+        assert st == 0, _lib.error_name(st)
+        self.ws = torch.empty(need.value, dtype=torch.uint8, device="cuda")
+        self.stream = torch.cuda.current_stream().cuda_stream
+
+    def call(self, i: int, stages: int = 0):
+        C = self.C
+        t = self.at[i % self.copies]
+        if stages:
+            st = self.L.t3_linear_stages(self.stream, C.byref(self.ax), C.byref(t), C.byref(self.asu), C.byref(self.asv),
+                                         self.dec, C.byref(self.ay), self.ws.data_ptr(), self.ws.numel(), stages)
+        else:
+            st = self.L.t3_linear(self.stream, C.byref(self.ax), C.byref(t), C.byref(self.asu), C.byref(self.asv),
+                                  self.dec, C.byref(self.ay), self.ws.data_ptr(), self.ws.numel())
+        if st != 0:
+            raise RuntimeError(self.L.t3_error_name(st).decode())
+
+    def time(self, steps: int, warmup: int, stages: int = 0) -> float:
+        """Seconds per call over `steps` back-to-back calls, events on the launch stream."""
+        torch = self.torch
+        for i in range(warmup):
+            self.call(i, stages)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(steps):
+            self.call(warmup + i, stages)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / steps
+
+
+def cpu_baseline(n: int, seed: int, budget_s: float = 20.0):
+    """format.project (the C oracle) on the host: the same shape and seeded distributions, one row, one thread,
+    re-decoding every tile as the reference does. A bounded sample: whole calls until ~budget_s is spent."""
+    from oracle import oracle
+    rng = np.random.default_rng(seed)
+    trellis, suh, svh = oracle.synth_linear(rng, IN_F, OUT_F, n)
+    x = rng.standard_normal(IN_F).astype(np.float32)
+    oracle.project(x[:128], trellis[:8, :8], suh[:128], svh[:128], 128, 128, n, oracle.MCG)  # load the library
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 5 and (time.perf_counter() - t_start < budget_s or not times):
+        t0 = time.perf_counter()
+        oracle.project(x, trellis, suh, svh, IN_F, OUT_F, n, oracle.MCG)
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    cores = os.cpu_count() or 1
+    threads = min(cores, 16)
+    t0 = time.perf_counter()
+    oracle.project_rows(x[None, :], trellis, suh, svh, IN_F, OUT_F, n, oracle.MCG, threads=threads)
+    par = time.perf_counter() - t0
+    return {
+        "value": code_bytes(IN_F, OUT_F, n) / med / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+        "sample": f"{len(times)} whole calls of the same workload (in={IN_F}, out={OUT_F}, n={n}, 1 row), median "
+                  f"{med * 1e3:.1f} ms a call; scalar single thread as the reference's format.project",
+        "ms_per_call": med * 1e3,
+        "all_cores": {"value": code_bytes(IN_F, OUT_F, n) / par / 1e9, "unit": "GB/s", "threads": threads,
+                      "note": "decode-once + OpenMP over output blocks, same bits"},
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--sweep", action="store_true", help="also time K = 3, 4, 5 x rows = 1, 4, 16, 32")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--k", type=int, default=4)
+    ap.add_argument("--rows", type=int, default=1)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build measures one GPU (the path has no collective); --gpus {args.gpus} is not served",
+              file=sys.stderr)
+        return 2
+
+    import torch
+
+    from turboexl3_amd import api
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    torch.cuda.set_device(0)
+    dec = api.Decode.mcg
+
+    def measure(k: int, rows: int, steps: int, warmup: int):
+        n = 16 * k
+        cb = code_bytes(IN_F, OUT_F, n)
+        copies = -(-MIN_ROTATION_BYTES // cb) + 1
+        trellis, suh, svh = make_weights(torch, n, copies, seed=1000 + k)
+        x = make_x(torch, rows, seed=7)
+        run = DenseRunner(torch, api, trellis, suh, svh, x, dec)
+        t_call = run.time(steps, warmup)
+        t_gemv = run.time(steps, warmup, stages=2)
+        return {"k": k, "rows": rows, "code_bytes": cb, "copies": copies, "us_per_call": t_call * 1e6,
+                "call_gbps": cb / t_call / 1e9, "gemv_us": t_gemv * 1e6, "gemv_gbps": cb / t_gemv / 1e9,
+                "gemv_frac_of_hbm": cb / t_gemv / HBM_PEAK}
+
+    head = measure(args.k, args.rows, args.steps, args.warmup)
+    out = {
+        "metric": "EXL3 GEMV HBM GB/s (% of 8 TB/s) at decode rows; MoE prefill GEMM TFLOP/s",
+        "value": head["call_gbps"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": head["us_per_call"] * 1e-3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"dense decode-row GEMV in={IN_F} out={OUT_F} K={args.k} rows={args.rows} MCG w16, "
+                               f"f16 activations, {head['copies']} rotating weight copies",
+                   "pct_of_8TBps": 100.0 * head["call_gbps"] * 1e9 / HBM_PEAK},
+        "roofline": {"bound": "hbm", "achieved": head["gemv_gbps"], "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": head["gemv_frac_of_hbm"], "traffic": None, "kernel": "t3::dense_gemv",
+                     "us_per_launch": head["gemv_us"], "algorithmic_bytes_per_launch": head["code_bytes"]},
+    }
+    if args.sweep:
+        out["sweep"] = [measure(k, r, max(50, args.steps // 4), 10) for k in (3, 4, 5) for r in (1, 4, 16, 32)]
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(16 * args.k, seed=11)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -118,6 +118,16 @@ int32_t t3_linear_workspace_bytes(const t3_array* x, const t3_array* trellis, t3
 int32_t t3_linear_chain(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
                         const t3_array* svh, t3_decode dec, t3_array* y, void* workspace, size_t workspace_bytes);
 
+/* `t3_linear_chain` with a choice of its launches, for profilers and hosts that bind the chain's roles themselves
+ * (src/hip/plan.zig:161-204): stage bit 0 = prepare, bit 1 = GEMV, bit 2 = finish; the workspace carries xq, xs and
+ * the planes between calls. */
+#define T3_STAGE_PREPARE 1u
+#define T3_STAGE_GEMV 2u
+#define T3_STAGE_FINISH 4u
+int32_t t3_linear_stages(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
+                         const t3_array* svh, t3_decode dec, t3_array* y, void* workspace, size_t workspace_bytes,
+                         uint32_t stages);
+
 /* W_hat f16 [in, out] from trellis [in/16, out/16, n], bit-exact to format.reconstructInner
  * (src/core/format.zig:276-291; the role of src/core/dense.zig:909-922 `dequantize`). */
 int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_array* w_hat);

@@ -42,6 +42,8 @@ int32_t check_dense(const t3_array* x, const t3_array* trellis, const t3_array* 
     Dec d;
     if (const int32_t st = resolve_decode(dec, &d); st != T3_OK) return st;
     if (max_rows != 0 && rows > max_rows) return T3_Exl3EngineNotImplemented;
+    // the kernels address one matrix, and one call's prepared rows, through 32-bit byte offsets
+    if ((in / 16) * (out / 16) * n * 2 >= (1ll << 31) || rows * in * 4 >= (1ll << 31)) return T3_Exl3EngineNotImplemented;
 
     DenseLaunch& l = call->launch;
     l.x = x->data;
@@ -72,10 +74,13 @@ void carve_dense(DenseCall* call, void* workspace) {
     call->workspace = c.used;
 }
 
-int32_t run_chain(const DenseCall& call, hipStream_t s) {
-    if (const int32_t st = hip_status(launch_dense_prep(call.launch, s)); st != T3_OK) return st;
-    if (const int32_t st = hip_status(launch_dense_gemv(call.launch, s)); st != T3_OK) return st;
-    return hip_status(launch_dense_finish(call.launch, s));
+int32_t run_chain(const DenseCall& call, hipStream_t s, uint32_t stages) {
+    if (stages & T3_STAGE_PREPARE)
+        if (const int32_t st = hip_status(launch_dense_prep(call.launch, s)); st != T3_OK) return st;
+    if (stages & T3_STAGE_GEMV)
+        if (const int32_t st = hip_status(launch_dense_gemv(call.launch, s)); st != T3_OK) return st;
+    if (stages & T3_STAGE_FINISH) return hip_status(launch_dense_finish(call.launch, s));
+    return T3_OK;
 }
 
 }  // namespace
@@ -94,13 +99,21 @@ int32_t t3_linear_workspace_bytes(const t3_array* x, const t3_array* trellis, t3
 
 int32_t t3_linear_chain(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
                         const t3_array* svh, t3_decode dec, t3_array* y, void* workspace, size_t workspace_bytes) {
+    return t3_linear_stages(stream, x, trellis, suh, svh, dec, y, workspace, workspace_bytes,
+                            T3_STAGE_PREPARE | T3_STAGE_GEMV | T3_STAGE_FINISH);
+}
+
+int32_t t3_linear_stages(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
+                         const t3_array* svh, t3_decode dec, t3_array* y, void* workspace, size_t workspace_bytes,
+                         uint32_t stages) {
     if (!suh || !svh || !y) return T3_BadArgs;
+    if (stages == 0u || stages > 7u) return T3_BadArgs;
     t3::DenseCall call;
     if (const int32_t st = t3::check_dense(x, trellis, suh, svh, dec, y, 32, &call); st != T3_OK) return st;
     if (!workspace) return T3_BadArgs;
     t3::carve_dense(&call, workspace);
     if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
-    return t3::run_chain(call, static_cast<hipStream_t>(stream));
+    return t3::run_chain(call, static_cast<hipStream_t>(stream), stages);
 }
 
 int32_t t3_linear(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
