@@ -89,17 +89,29 @@ class DenseRunner:
             raise RuntimeError(self.L.t3_error_name(st).decode())
 
     def time(self, steps: int, warmup: int, stages: int = 0) -> float:
-        """Seconds per call over `steps` back-to-back calls, events on the launch stream."""
+        """Seconds per call over exactly `steps` back-to-back calls. The calls are captured once into a HIP graph
+        (as a serving loop would hold its decode step) so the host's per-launch cost stays out of the GPU's
+        timeline; events bracket the replay on the launch stream."""
         torch = self.torch
-        for i in range(warmup):
+        for i in range(max(warmup, 1)):
             self.call(i, stages)
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for i in range(steps):
-            self.call(warmup + i, stages)
-        e1.record()
-        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            self.stream = side.cuda_stream
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(steps):
+                    self.call(warmup + i, stages)
+            torch.cuda.synchronize()
+            graph.replay()  # untimed: the graph's first replay uploads it
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(side)
+            graph.replay()
+            e1.record(side)
+            torch.cuda.synchronize()
+        self.stream = torch.cuda.current_stream().cuda_stream
         return e0.elapsed_time(e1) * 1e-3 / steps
 
 

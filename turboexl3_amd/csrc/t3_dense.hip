@@ -13,7 +13,7 @@
 // The role of each launch follows the reference's HIP plan (src/hip/plan.zig:161-204) but the launch shapes, the lane
 // plan and the use of MFMA are this library's own.
 
-#include "t3_decode.hpp"
+#include "t3_gemv_core.hpp"
 #include "t3_kernels.hpp"
 
 namespace t3 {
@@ -51,16 +51,21 @@ __global__ void __launch_bounds__(64) dense_prep(const void* x, const uint16_t* 
 }
 
 // Grid (out / 16 / BT, KS), 256 threads (4 waves). A workgroup owns BT adjacent output tiles and K slice blockIdx.y;
-// wave sg takes part sg of the slice, `per` = in_tiles / (4 KS) input tiles (the host divides: the GPU has no scalar divide). RB = 16-row blocks of x (1 or 2).
-// z f32 [KS][rows][out]: the four waves' sums, wave 0 first.
+// wave sg takes part sg of the slice, `per` = in_tiles / (4 KS) input tiles (the host divides: the GPU has no scalar
+// divide). RB = 16-row blocks of x (1 or 2). z f32 [KS][rows][out]: the four waves' sums, wave 0 first.
 template <int CB, bool WIDE, int RB, int BT>
 __global__ void __launch_bounds__(256) dense_gemv(const uint32_t* __restrict__ w, const uint32_t* __restrict__ xq,
                                                   float* __restrict__ z, uint32_t in, uint32_t out, uint32_t rows,
                                                   uint32_t n, uint32_t wbits, uint32_t per) {
-    __shared__ float4v red[4][RB * BT * 64];
+    constexpr int ST = 8;  // tile rows in flight a wave
+    constexpr uint32_t kStage = gemv_stage_bytes<BT>();
+    constexpr uint32_t kRed = 4u * RB * BT * 64u * 16u;
+    // the waves' LDS stages while they stream; the four waves' partial sums afterwards
+    __shared__ __attribute__((aligned(16))) unsigned char smem[kRed > 4u * kStage ? kRed : 4u * kStage];
+    float4v(*red)[RB * BT * 64] = reinterpret_cast<float4v(*)[RB * BT * 64]>(smem);
     const uint32_t blk = blockIdx.x, ksl = blockIdx.y;
     const uint32_t sg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
-    const uint32_t in_tiles = in >> 4, out_tiles = out >> 4, nw = n >> 1;
+    const uint32_t out_tiles = out >> 4, nw = n >> 1;
     const uint32_t tk0 = (ksl * 4u + sg) * per;
     const QuadPlan<WIDE> plan = quad_plan<WIDE>(n, lane);
 
@@ -72,81 +77,18 @@ __global__ void __launch_bounds__(256) dense_gemv(const uint32_t* __restrict__ w
 
     // x fragment: activation row (lane % 16) of block r, K slots 8g..8g+7 = quad g's four inputs, each doubled.
     // Rows past the call's last alias row 0: their sums are computed and never stored.
-    const uint32_t g = lane >> 4;
     uint32_t xoff[RB];
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
         const uint32_t row = static_cast<uint32_t>(r) * 16u + (lane & 15u);
-        xoff[r] = ((row < rows ? row : 0u) * in + 4u * g) * 4u;
-    }
-    // Per-lane byte offsets inside the workgroup's BT adjacent tiles; the tile row's offset stays scalar.
-    uint32_t off_bp[BT], off_bl[BT], off_ap[BT], off_al[BT];
-#pragma unroll
-    for (int t = 0; t < BT; ++t) {
-        off_bp[t] = (static_cast<uint32_t>(t) * nw + plan.ib_prev) * 4u;
-        off_bl[t] = (static_cast<uint32_t>(t) * nw + plan.ib_last) * 4u;
-        off_ap[t] = (static_cast<uint32_t>(t) * nw + plan.ia_prev) * 4u;
-        off_al[t] = (static_cast<uint32_t>(t) * nw + plan.ia_last) * 4u;
+        xoff[r] = ((row < rows ? row : 0u) * in + 4u * (lane >> 4)) * 4u;
     }
     const uint64_t wstride = static_cast<uint64_t>(out_tiles) * nw;  // words a tile row
-    const uint64_t wfirst = static_cast<uint64_t>(blk) * BT * nw + tk0 * wstride;
-    const __amdgpu_buffer_rsrc_t wres = make_rsrc(w + wfirst, (static_cast<uint64_t>(in_tiles) * wstride - wfirst) * 4u);
-    const __amdgpu_buffer_rsrc_t xres = make_rsrc(xq, static_cast<uint64_t>(rows) * in * 4u);
-    const uint32_t wstep = static_cast<uint32_t>(wstride) * 4u;  // bytes; the host holds a matrix under 2^31 bytes
-    const uint32_t wstep2 = 2u * wstep;
-
-    auto load_tiles = [&](uint32_t soff, QuadWords<WIDE>(&dst)[BT]) {
-#pragma unroll
-        for (int t = 0; t < BT; ++t) {
-            dst[t].b_prev = buf_load_u32(wres, off_bp[t], soff);
-            dst[t].b_last = buf_load_u32(wres, off_bl[t], soff);
-            if constexpr (WIDE) {
-                dst[t].a_prev = buf_load_u32(wres, off_ap[t], soff);
-                dst[t].a_last = buf_load_u32(wres, off_al[t], soff);
-            }
-        }
-    };
-    auto load_x = [&](uint32_t soff, uint4v(&dst)[RB]) {
-#pragma unroll
-        for (int r = 0; r < RB; ++r) dst[r] = buf_load_u128(xres, xoff[r], soff);
-    };
-
-    auto consume = [&](const QuadWords<WIDE>(&words)[BT], const uint4v(&xv)[RB]) {
-#pragma unroll
-        for (int t = 0; t < BT; ++t) {
-            uint32_t cw[4];
-            quad_codewords<WIDE>(words[t], plan, wbits, cw);
-            uint4v a;
-#pragma unroll
-            for (int m = 0; m < 4; ++m) a[m] = weight_pair<CB>(cw[m]);
-#pragma unroll
-            for (int r = 0; r < RB; ++r)
-                acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a),
-                                                                   __builtin_bit_cast(half8, xv[r]), acc[r][t], 0, 0, 0);
-        }
-    };
-
-    // Two register sets in turn: while one tile row decodes, the next one's words are in flight.
-    QuadWords<WIDE> wa[BT], wb[BT];
-    uint4v xa[RB], xb[RB];
-    uint32_t wo = 0u, xo = tk0 * 64u;  // scalar byte offsets of the tile row in flight
-    load_tiles(wo, wa);
-    load_x(xo, xa);
-    uint32_t i = 0;
-    for (; i + 1u < per; i += 2u) {
-        load_tiles(wo + wstep, wb);
-        load_x(xo + 64u, xb);
-        __builtin_amdgcn_sched_barrier(0);
-        consume(wa, xa);
-        const bool two = i + 2u < per;  // the last odd step rereads the row already held
-        wo += two ? wstep2 : wstep;
-        xo += two ? 128u : 64u;
-        load_tiles(wo, wa);
-        load_x(xo, xa);
-        __builtin_amdgcn_sched_barrier(0);
-        consume(wb, xb);
-    }
-    if (i < per) consume(wa, xa);
+    const uint32_t* wbase = w + static_cast<uint64_t>(blk) * BT * nw + tk0 * wstride;
+    gemv_stream<CB, WIDE, RB, BT, ST>(wbase, static_cast<uint32_t>(wstride) * 4u, per, n, plan, wbits, xq,
+                                      static_cast<uint64_t>(rows) * in * 4u, xoff, tk0 * 64u, smem + sg * kStage, lane,
+                                      acc);
+    __syncthreads();  // every wave is done with its stage before the sums take the memory
 
     // lane holds, for activation row (lane % 16) of block r, output columns 4g..4g+3 of tile t
 #pragma unroll
@@ -205,11 +147,8 @@ hipError_t launch_gemv_bt(const DenseLaunch& d, hipStream_t s) {
                            d.n, d.wbits, (d.in / 16u) / (4u * d.ks));
         return hipGetLastError();
     };
-    switch (d.bt) {
-        case 1: return go(dense_gemv<CB, WIDE, RB, 1>, 1u);
-        case 2: return go(dense_gemv<CB, WIDE, RB, 2>, 2u);
-        default: return go(dense_gemv<CB, WIDE, RB, 4>, 4u);
-    }
+    if (d.bt == 8u) return go(dense_gemv<CB, WIDE, RB, 8>, 8u);
+    return go(dense_gemv<CB, WIDE, RB, 4>, 4u);
 }
 
 template <int CB>

@@ -61,7 +61,8 @@ struct Carver {
 // are those of the row alone. The reference fixes its split the same way (turboexl3 src/core/dense.zig:553-562); the
 // numbers here are sized for 256 CUs, not for its 40-core target.
 
-constexpr uint32_t kGemvBt = 4;          // output tiles a wave
+// output tiles a wave: one 128-bit load a lane covers a tile row's BT * 2n bytes (at most 1 KB)
+inline uint32_t gemv_bt(uint32_t n) { return n <= 64u ? 8u : 4u; }
 constexpr uint32_t kGemvTargetWgs = 768; // three workgroups a CU
 constexpr uint32_t kGemvMinPer = 4;      // input tiles a wave at least
 
