@@ -73,7 +73,7 @@ class DenseRunner:
         need = C.c_size_t(0)
         st = self.L.t3_linear_workspace_bytes(C.byref(self.ax), C.byref(self.at[0]), self.dec, C.byref(need))
         assert st == 0, _lib.error_name(st)
-        self.ws = torch.empty(need.value, dtype=torch.uint8, device="cuda")
+        self.ws = torch.zeros(need.value, dtype=torch.uint8, device="cuda")
         self.stream = torch.cuda.current_stream().cuda_stream
 
     def call(self, i: int, stages: int = 0):
@@ -154,7 +154,11 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--k", type=int, default=4)
     ap.add_argument("--rows", type=int, default=1)
+    ap.add_argument("--in-f", type=int, default=4096)
+    ap.add_argument("--out-f", type=int, default=12288)
     args = ap.parse_args()
+    global IN_F, OUT_F
+    IN_F, OUT_F = args.in_f, args.out_f
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU (the path has no collective); --gpus {args.gpus} is not served",
               file=sys.stderr)

@@ -7,6 +7,10 @@
  * `hipStream_t`, NULL = the null stream) and never synchronised here. Outputs and scratch are the caller's:
  * ask `*_workspace_bytes`, allocate once, pass the pointer. Inputs are borrowed, never copied or kept.
  *
+ * Workspace contract: its first T3_WORKSPACE_COUNTER_BYTES bytes hold the arrival counters of the fused launches.
+ * They must be zero when a workspace is first passed (zero-fill it once when you allocate it); every call leaves
+ * them zero. Calls that share a workspace must be ordered on one stream: overlapping calls race on it.
+ *
  * Refusal convention (turboexl3 docs/core/api.md:10-12): a call this library does not serve returns a named
  * status before it launches anything and leaves every output untouched; the caller runs its own chain.
  * The status names are the reference's Zig error names.
@@ -24,6 +28,7 @@ extern "C" {
 #endif
 
 #define T3_ABI_VERSION 1
+#define T3_WORKSPACE_COUNTER_BYTES 65536
 
 typedef void* t3_stream; /* hipStream_t */
 

@@ -81,6 +81,37 @@ def test_dense_chain_rows_1_to_32(oracle, t3, in_f, out_f, n, codebook, wbits, d
     print(f"dense {in_f}x{out_f} n={n} cb={codebook} {dtype}: worst {worst:.3e} (bar {bar})")
 
 
+@pytest.mark.parametrize("in_f,out_f,n,codebook,wbits,dtype", [
+    (4096, 2048, 64, MCG, 16, torch.bfloat16),   # per = 8: one launch up to 4 rows
+    (4096, 1024, 48, MUL1, 16, torch.float16),   # deferred map: the block sums cross workgroups
+    (2560, 640, 80, MUL1, 16, torch.float32),    # per = 40 > 16: prepare + arriving GEMV at every row count
+    (512, 256, 36, MCG, 16, torch.float32),      # a K part that is not whole 128-blocks
+    (1024, 512, 96, MCG, 12, torch.float16),     # wide reader, BT 4: two workgroup columns a 128-column block
+])
+def test_fused_launches_equal_the_chain_bytes(oracle, t3, in_f, out_f, n, codebook, wbits, dtype):
+    # the served `linear` (one launch up to 4 rows, else prepare + arriving GEMV) against the three-launch chain,
+    # byte for byte, twice in a row (the arrival counters must come back to zero)
+    case = DenseCase(oracle, t3, 0xF00D + in_f + n, in_f, out_f, n, codebook, wbits)
+    x_dev, _ = make_x(case.rng, 32, in_f, dtype)
+    for rows in (1, 2, 4, 5, 16, 17, 32):
+        chain = t3.linear_chain(x_dev[:rows], case.d_trellis, case.d_suh, case.d_svh, case.dec)
+        for _ in range(2):
+            fused = t3.linear(x_dev[:rows], case.d_trellis, case.d_suh, case.d_svh, case.dec)
+            assert bytes_of(fused) == bytes_of(chain), f"rows {rows}: the fused launch differs from the chain"
+
+
+def test_dec_one_off_runs_the_chain(oracle, t3):
+    case = DenseCase(oracle, t3, 3, 4096, 1024, 64, MCG)
+    x_dev, _ = make_x(case.rng, 2, 4096, torch.float16)
+    want = t3.linear(x_dev, case.d_trellis, case.d_suh, case.d_svh, case.dec)
+    t3.configure(dec_one=0)
+    try:
+        got = t3.linear(x_dev, case.d_trellis, case.d_suh, case.d_svh, case.dec)
+    finally:
+        t3.configure()
+    assert bytes_of(got) == bytes_of(want)
+
+
 def test_dense_exact_codebook_forms_stay_within_bar(oracle, t3):
     # the f16-weight forms (mcg_pair off, mul1_defer off) against the same reference
     t3.configure(mcg_pair=0, mul1_defer=0)

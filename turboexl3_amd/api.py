@@ -99,7 +99,8 @@ def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
     key = (device.type, device.index)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        # zero-filled once: the head of a workspace holds the fused launches' arrival counters
+        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
 

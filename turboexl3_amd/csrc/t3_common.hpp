@@ -32,6 +32,19 @@ __device__ __forceinline__ uint4v buf_load_u128(__amdgpu_buffer_rsrc_t r, uint32
     return __builtin_amdgcn_raw_buffer_load_b128(r, static_cast<int>(voff), static_cast<int>(soff), 0);
 }
 
+// Device-coherent accesses for data that crosses workgroups inside one launch. The GPU's eight dies each have their
+// own L2, so a device-scope fence writes back and invalidates a whole L2: ruinous when every workgroup runs one.
+// Relaxed device-scope atomic loads and stores go to the coherent level by themselves (the sc1 cache policy) and leave
+// every other access cached.
+__device__ __forceinline__ void store_coherent(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_coherent(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// every store this lane has issued is acknowledged at its coherence level (with store_coherent: device-wide)
+__device__ __forceinline__ void wait_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 __device__ __forceinline__ float half_value(uint32_t bits) {
     return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(bits)));
 }

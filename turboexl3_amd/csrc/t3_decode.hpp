@@ -109,18 +109,19 @@ __device__ __forceinline__ QuadPlan<WIDE> quad_plan(uint32_t n, uint32_t lane) {
     for (uint32_t m = 0; m < 4u; ++m) e[m] = ((p + m + 1u) * n) >> 4;
     QuadPlan<WIDE> q;
     {
-        const uint32_t end = e[3] + total;  // one period added keeps the word index positive
+        // one period added keeps the word index positive: w is in [nw, 2 nw), so the modulo is one subtraction
+        const uint32_t end = e[3] + total;
         const uint32_t w = (end - 1u) >> 5;
         q.shb = 32u * (w + 1u) - end;
-        q.ib_last = w % nw;
-        q.ib_prev = (w - 1u) % nw;
+        q.ib_last = w - nw;
+        q.ib_prev = w - 1u >= nw ? w - 1u - nw : w - 1u;
     }
     if constexpr (WIDE) {
         const uint32_t end = e[1] + total;
         const uint32_t w = (end - 1u) >> 5;
         q.sha = 32u * (w + 1u) - end;
-        q.ia_last = w % nw;
-        q.ia_prev = (w - 1u) % nw;
+        q.ia_last = w - nw;
+        q.ia_prev = w - 1u >= nw ? w - 1u - nw : w - 1u;
         q.o[0] = e[1] - e[0];
         q.o[1] = 0u;
         q.o[2] = e[3] - e[2];

@@ -10,7 +10,13 @@
 // own row of x alone, so a row's bytes do not depend on the rows beside it (the reference's row-alone invariant,
 // turboexl3 src/hip_tests.zig:338-346).
 //
-// The role of each launch follows the reference's HIP plan (src/hip/plan.zig:161-204) but the launch shapes, the lane
+// Three launch forms run the same statements in the same order, so their bytes agree (the reference holds its
+// one-launch DEC-ONE to its chain the same way, src/core/gpu_test.zig:1016):
+//   chain   three launches: dense_prep, dense_gemv<kChain>, dense_finish;
+//   arrive  two launches: dense_prep, dense_gemv<kArrive>: the workgroup that completes a 128-column block's planes
+//           (an integer arrival counter over device-coherent stores, nothing spins) runs the block's finish;
+//   one     one launch, up to 4 rows: dense_gemv<kOne> prepares its own K part in LDS, then as arrive.
+// The role of each launch follows the reference's HIP plan (src/hip/plan.zig:161-204); the launch shapes, the lane
 // plan and the use of MFMA are this library's own.
 
 #include "t3_gemv_core.hpp"
@@ -19,55 +25,148 @@
 namespace t3 {
 namespace {
 
-// Grid (in / 128, rows), 64 threads. xq: uint32 [rows][in], word (tk 16 + quad_slot(r)) = the f16 value of input
-// tk 16 + r in both halves. xs: f32 [rows][in / 128].
-template <int DT>
-__device__ __forceinline__ void prep_block(const void* x, const uint16_t* suh, uint32_t* xq, float* xs, uint32_t in,
-                                           uint32_t row_in, uint32_t row_out, uint32_t b, uint32_t lane) {
+enum Fuse : int { kChain = 0, kArrive = 1, kOne = 2 };
+
+__device__ __forceinline__ float load_act_rt(int dt, const void* p, size_t i) {
+    if (dt == kF32) return load_act<kF32>(p, i);
+    if (dt == kF16) return load_act<kF16>(p, i);
+    return load_act<kBf16>(p, i);
+}
+__device__ __forceinline__ void store_act_rt(int dt, void* p, size_t i, float v) {
+    if (dt == kF32) store_act<kF32>(p, i, v);
+    else if (dt == kF16) store_act<kF16>(p, i, v);
+    else store_act<kBf16>(p, i, v);
+}
+
+// One 128-block of one row, one wave: lane L owns elements L and L + 64. Returns the lane's two prepared f16 values
+// (bits) and the block's sum of them (the same in every lane).
+__device__ __forceinline__ void prep_values(int dt, const void* x, const uint16_t* suh, uint32_t in, uint32_t row,
+                                            uint32_t b, uint32_t lane, uint32_t (&hv)[2], float& sum) {
     float v[2];
 #pragma unroll
     for (uint32_t j = 0; j < 2u; ++j) {
         const uint32_t i = b * 128u + lane + 64u * j;
-        v[j] = round_half(load_act<DT>(x, static_cast<size_t>(row_in) * in + i)) * half_value(suh[i]);
+        v[j] = round_half(load_act_rt(dt, x, static_cast<size_t>(row) * in + i)) * half_value(suh[i]);
     }
     h128_wave(v, lane);
-    float sum = 0.0f;
+    sum = 0.0f;
 #pragma unroll
     for (uint32_t j = 0; j < 2u; ++j) {
-        const uint32_t i = b * 128u + lane + 64u * j;
-        const uint32_t hv = half_bits(v[j] * kHadScale);
-        xq[static_cast<size_t>(row_out) * in + (i & ~15u) + quad_slot(i & 15u)] = hv | (hv << 16);
-        sum += half_value(hv);
+        hv[j] = half_bits(v[j] * kHadScale);
+        sum += half_value(hv[j]);
     }
 #pragma unroll
     for (int m = 32; m > 0; m >>= 1) sum += __shfl_xor(sum, m, 64);
-    if (lane == 0u) xs[static_cast<size_t>(row_out) * (in / 128u) + b] = sum;
 }
 
-template <int DT>
+// Grid (in / 128, rows), 64 threads. xq: uint32 [rows][in], word (tk 16 + quad_slot(r)) = the f16 value of input
+// tk 16 + r in both halves. xs: f32 [rows][in / 128].
 __global__ void __launch_bounds__(64) dense_prep(const void* x, const uint16_t* suh, uint32_t* xq, float* xs,
-                                                 uint32_t in) {
-    prep_block<DT>(x, suh, xq, xs, in, blockIdx.y, blockIdx.y, blockIdx.x, threadIdx.x);
+                                                 uint32_t in, int dt) {
+    const uint32_t b = blockIdx.x, row = blockIdx.y, lane = threadIdx.x;
+    uint32_t hv[2];
+    float sum;
+    prep_values(dt, x, suh, in, row, b, lane, hv, sum);
+#pragma unroll
+    for (uint32_t j = 0; j < 2u; ++j) {
+        const uint32_t i = b * 128u + lane + 64u * j;
+        xq[static_cast<size_t>(row) * in + (i & ~15u) + quad_slot(i & 15u)] = hv[j] | (hv[j] << 16);
+    }
+    if (lane == 0u) xs[static_cast<size_t>(row) * (in / 128u) + b] = sum;
 }
+
+// One wave finishes outputs b 128 + L and + 64 of one row. xs_row: the row's in / 128 block sums. ZCOH / XCOH: the
+// planes / the block sums were written by other workgroups of this launch. Loads go out eight at a time and are added
+// in slice (or block) order: the sums do not depend on the batching.
+template <bool ZCOH, bool XCOH>
+__device__ __forceinline__ void finish_block(int dt, const float* z, const float* xs_row, const uint16_t* svh, void* y,
+                                             uint32_t out, uint32_t rows, uint32_t ks, uint32_t inblk, int defer,
+                                             uint32_t row, uint32_t b, uint32_t lane) {
+    auto get_z = [](const float* p) { return ZCOH ? load_coherent(p) : *p; };
+    auto get_x = [](const float* p) { return XCOH ? load_coherent(p) : *p; };
+    float xsum = 0.0f;
+    if (defer)
+        for (uint32_t q0 = 0; q0 < inblk; q0 += 8u) {
+            float part[8];
+#pragma unroll
+            for (uint32_t q = 0; q < 8u; ++q) part[q] = q0 + q < inblk ? get_x(xs_row + q0 + q) : 0.0f;
+#pragma unroll
+            for (uint32_t q = 0; q < 8u; ++q)
+                if (q0 + q < inblk) xsum += part[q];
+        }
+    float v[2];
+    const size_t plane = static_cast<size_t>(rows) * out;
+    const float* z0 = z + static_cast<size_t>(row) * out + b * 128u + lane;
+    float acc[2] = {0.0f, 0.0f};
+    for (uint32_t k0 = 0; k0 < ks; k0 += 8u) {
+        float part[8][2];
+#pragma unroll
+        for (uint32_t k = 0; k < 8u; ++k)
+#pragma unroll
+            for (uint32_t j = 0; j < 2u; ++j) part[k][j] = k0 + k < ks ? get_z(z0 + (k0 + k) * plane + 64u * j) : 0.0f;
+#pragma unroll
+        for (uint32_t k = 0; k < 8u; ++k)
+            if (k0 + k < ks) {
+                // the first plane starts the sum (0 + z would turn a -0 into +0)
+                acc[0] = k0 + k == 0u ? part[k][0] : acc[0] + part[k][0];
+                acc[1] = k0 + k == 0u ? part[k][1] : acc[1] + part[k][1];
+            }
+    }
+#pragma unroll
+    for (uint32_t j = 0; j < 2u; ++j) {
+        float s = acc[j];
+        if (defer) s = __builtin_fmaf(s, mul1_a(), mul1_b() * xsum);
+        v[j] = round_half(s);
+    }
+    h128_wave(v, lane);
+#pragma unroll
+    for (uint32_t j = 0; j < 2u; ++j) {
+        const uint32_t o = b * 128u + lane + 64u * j;
+        store_act_rt(dt, y, static_cast<size_t>(row) * out + o, round_half(v[j] * kHadScale * half_value(svh[o])));
+    }
+}
+
+// Grid (out / 128, rows), 64 threads.
+__global__ void __launch_bounds__(64) dense_finish(const float* z, const float* xs, const uint16_t* svh, void* y,
+                                                   uint32_t out, uint32_t rows, uint32_t ks, uint32_t inblk, int defer,
+                                                   int dt) {
+    finish_block<false, false>(dt, z, xs + static_cast<size_t>(blockIdx.y) * inblk, svh, y, out, rows, ks, inblk, defer,
+                        blockIdx.y, blockIdx.x, threadIdx.x);
+}
+
+struct GemvArgs {
+    const uint32_t* w;
+    const uint32_t* xq;   // kChain, kArrive: the prepared rows
+    float* z;
+    float* xs;            // block sums: [rows][in / 128]; kOne: [out / 128][rows][in / 128], a copy a column block,
+                          // each written by that block's own workgroups (one shared copy would be stored to by
+                          // every workgroup at once: 3,000 coherent stores to one cache line serialise for ~80 us)
+    const void* x;        // kOne: the raw activations
+    const uint16_t* suh;  // kOne
+    const uint16_t* svh;  // kArrive, kOne
+    void* y;              // kArrive, kOne
+    uint32_t* arrive;     // kArrive, kOne: one counter a 128-column block, zero between calls
+    uint32_t in, out, rows, n, wbits, per, ks;
+    int dt, defer;
+};
 
 // Grid (out / 16 / BT, KS), 256 threads (4 waves). A workgroup owns BT adjacent output tiles and K slice blockIdx.y;
 // wave sg takes part sg of the slice, `per` = in_tiles / (4 KS) input tiles (the host divides: the GPU has no scalar
 // divide). RB = 16-row blocks of x (1 or 2). z f32 [KS][rows][out]: the four waves' sums, wave 0 first.
-template <int CB, bool WIDE, int RB, int BT>
-__global__ void __launch_bounds__(256) dense_gemv(const uint32_t* __restrict__ w, const uint32_t* __restrict__ xq,
-                                                  float* __restrict__ z, uint32_t in, uint32_t out, uint32_t rows,
-                                                  uint32_t n, uint32_t wbits, uint32_t per) {
-    constexpr int ST = 8;  // tile rows in flight a wave
+template <int CB, bool WIDE, int RB, int BT, int FUSE>
+__global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
+    constexpr int ST = 2;  // tile rows in flight a wave: occupancy hides more latency here than a deeper ring does
     constexpr uint32_t kStage = gemv_stage_bytes<BT>();
     constexpr uint32_t kRed = 4u * RB * BT * 64u * 16u;
+    constexpr uint32_t kMain = kRed > 4u * kStage ? kRed : 4u * kStage;
     // the waves' LDS stages while they stream; the four waves' partial sums afterwards
-    __shared__ __attribute__((aligned(16))) unsigned char smem[kRed > 4u * kStage ? kRed : 4u * kStage];
+    __shared__ __attribute__((aligned(16))) unsigned char smem[kMain];
+    __shared__ uint32_t last_flag;
     float4v(*red)[RB * BT * 64] = reinterpret_cast<float4v(*)[RB * BT * 64]>(smem);
     const uint32_t blk = blockIdx.x, ksl = blockIdx.y;
     const uint32_t sg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
-    const uint32_t out_tiles = out >> 4, nw = n >> 1;
+    const uint32_t out_tiles = a.out >> 4, nw = a.n >> 1, rows = a.rows, per = a.per;
     const uint32_t tk0 = (ksl * 4u + sg) * per;
-    const QuadPlan<WIDE> plan = quad_plan<WIDE>(n, lane);
 
     float4v acc[RB][BT];
 #pragma unroll
@@ -75,19 +174,59 @@ __global__ void __launch_bounds__(256) dense_gemv(const uint32_t* __restrict__ w
 #pragma unroll
         for (int t = 0; t < BT; ++t) acc[r][t] = float4v{0.f, 0.f, 0.f, 0.f};
 
+    const uint64_t wstride = static_cast<uint64_t>(out_tiles) * nw;  // words a tile row
+    const uint32_t* wbase = a.w + static_cast<uint64_t>(blk) * BT * nw + tk0 * wstride;
+    const uint32_t wstep = static_cast<uint32_t>(wstride) * 4u;
+
     // x fragment: activation row (lane % 16) of block r, K slots 8g..8g+7 = quad g's four inputs, each doubled.
     // Rows past the call's last alias row 0: their sums are computed and never stored.
     uint32_t xoff[RB];
+    constexpr uint32_t kShare = 8u / BT;  // workgroup columns a 128-column block
+    const uint32_t b128 = blk / kShare;
+    const uint32_t inblk = a.in / 128u;
+    if constexpr (FUSE == kOne) {
+        static_assert(FUSE != kOne || RB == 1, "the one-launch form serves up to 4 rows");
+        extern __shared__ __attribute__((aligned(16))) unsigned char xdyn[];
+        unsigned char* xst = xdyn + sg * ((per + 1u) * (kXldsRows * 64u));
+        const uint32_t row = lane & 15u;
+        xoff[0] = (row < rows ? row : 0u) * 64u + (lane >> 4) * 16u;
+        GemvStream<CB, WIDE, RB, BT, ST, XLds> stream(wbase, wstep, per, a.n, a.wbits, XLds{xst}, xoff,
+                                                      smem + sg * kStage, lane);
+        stream.issue();
+        // While the codes fly, the wave prepares its own K part: per / 8 whole 128-blocks a row, the statements of
+        // dense_prep, into its LDS x stage [per + 1][4][64 bytes] (the last tile row zeros). The block sums go to the
+        // column block's own copy of xs (deferred MUL1 map only; the block's second workgroup column, if any, would
+        // store the same values again).
+        const uint32_t blocks = per >> 3;
+        for (uint32_t r = 0; r < rows; ++r)
+            for (uint32_t b = 0; b < blocks; ++b) {
+                uint32_t hv[2];
+                float sum;
+                prep_values(a.dt, a.x, a.suh, a.in, r, (tk0 >> 3) + b, lane, hv, sum);
 #pragma unroll
-    for (int r = 0; r < RB; ++r) {
-        const uint32_t row = static_cast<uint32_t>(r) * 16u + (lane & 15u);
-        xoff[r] = ((row < rows ? row : 0u) * in + 4u * (lane >> 4)) * 4u;
+                for (uint32_t j = 0; j < 2u; ++j) {
+                    const uint32_t i = lane + 64u * j;  // element of the block: tile row b 8 + i / 16
+                    const uint32_t at = ((b * 8u + (i >> 4)) * kXldsRows + r) * 64u + quad_slot(i & 15u) * 4u;
+                    *reinterpret_cast<uint32_t*>(xst + at) = hv[j] | (hv[j] << 16);
+                }
+                if (a.defer && lane == 0u && blk % kShare == 0u)
+                    store_coherent(a.xs + (static_cast<size_t>(b128) * rows + r) * inblk + (tk0 >> 3) + b, sum);
+            }
+        for (uint32_t i = lane; i < kXldsRows * 16u; i += 64u)
+            *reinterpret_cast<uint32_t*>(xst + per * (kXldsRows * 64u) + i * 4u) = 0u;
+        stream.run(acc);
+    } else {
+#pragma unroll
+        for (int r = 0; r < RB; ++r) {
+            const uint32_t row = static_cast<uint32_t>(r) * 16u + (lane & 15u);
+            xoff[r] = ((row < rows ? row : 0u) * a.in + 4u * (lane >> 4)) * 4u;
+        }
+        GemvStream<CB, WIDE, RB, BT, ST, XGlobal> stream(
+            wbase, wstep, per, a.n, a.wbits, XGlobal{a.xq, static_cast<uint64_t>(rows) * a.in * 4u, tk0 * 64u}, xoff,
+            smem + sg * kStage, lane);
+        stream.issue();
+        stream.run(acc);
     }
-    const uint64_t wstride = static_cast<uint64_t>(out_tiles) * nw;  // words a tile row
-    const uint32_t* wbase = w + static_cast<uint64_t>(blk) * BT * nw + tk0 * wstride;
-    gemv_stream<CB, WIDE, RB, BT, ST>(wbase, static_cast<uint32_t>(wstride) * 4u, per, n, plan, wbits, xq,
-                                      static_cast<uint64_t>(rows) * in * 4u, xoff, tk0 * 64u, smem + sg * kStage, lane,
-                                      acc);
     __syncthreads();  // every wave is done with its stage before the sums take the memory
 
     // lane holds, for activation row (lane % 16) of block r, output columns 4g..4g+3 of tile t
@@ -101,103 +240,111 @@ __global__ void __launch_bounds__(256) dense_gemv(const uint32_t* __restrict__ w
         const uint32_t row = r * 16u + (l & 15u);
         if (row >= rows) continue;
         const float4v s = ((red[0][i] + red[1][i]) + red[2][i]) + red[3][i];
-        float* dst = z + (static_cast<size_t>(ksl) * rows + row) * out + (blk * BT + t) * 16u + 4u * (l >> 4);
-        *reinterpret_cast<float4v*>(dst) = s;
-    }
-}
-
-// Grid (out / 128, rows), 64 threads: lane L finishes outputs b 128 + L and + 64.
-template <int DT>
-__device__ __forceinline__ void finish_block(const float* z, const float* xs, const uint16_t* svh, void* y,
-                                             uint32_t out, uint32_t rows, uint32_t ks, uint32_t inblk, int defer,
-                                             uint32_t row, uint32_t b, uint32_t lane) {
-    float xsum = 0.0f;
-    if (defer)
-        for (uint32_t q = 0; q < inblk; ++q) xsum += xs[static_cast<size_t>(row) * inblk + q];
-    float v[2];
+        float* dst = a.z + (static_cast<size_t>(ksl) * rows + row) * a.out + (blk * BT + t) * 16u + 4u * (l >> 4);
+        if constexpr (FUSE == kChain) {
+            *reinterpret_cast<float4v*>(dst) = s;
+        } else {
 #pragma unroll
-    for (uint32_t j = 0; j < 2u; ++j) {
-        const uint32_t o = b * 128u + lane + 64u * j;
-        float acc = z[static_cast<size_t>(row) * out + o];
-        for (uint32_t k = 1u; k < ks; ++k) acc += z[(static_cast<size_t>(k) * rows + row) * out + o];
-        if (defer) acc = __builtin_fmaf(acc, mul1_a(), mul1_b() * xsum);
-        v[j] = round_half(acc);
+            for (int c = 0; c < 4; ++c) store_coherent(dst + c, s[c]);
+        }
     }
-    h128_wave(v, lane);
-#pragma unroll
-    for (uint32_t j = 0; j < 2u; ++j) {
-        const uint32_t o = b * 128u + lane + 64u * j;
-        store_act<DT>(y, static_cast<size_t>(row) * out + o, round_half(v[j] * kHadScale * half_value(svh[o])));
+
+    if constexpr (FUSE != kChain) {
+        // The last workgroup to arrive at a 128-column block finishes it. The planes (and the one-launch form's block
+        // sums) are stored device-coherently; once every lane's stores are acknowledged the workgroup counts itself
+        // in, and the one that reads the full count sums the planes in slice order, as dense_finish does. Nothing
+        // spins, and no cache is flushed.
+        wait_stores();
+        __syncthreads();
+        if (threadIdx.x == 0u) {
+            const uint32_t before =
+                __hip_atomic_fetch_add(a.arrive + b128, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last_flag = before == a.ks * kShare - 1u;
+        }
+        __syncthreads();
+        if (last_flag) {
+            for (uint32_t row = sg; row < rows; row += 4u) {
+                const float* xs_row = a.xs + (FUSE == kOne ? (static_cast<size_t>(b128) * rows + row) * inblk
+                                                           : static_cast<size_t>(row) * inblk);
+                // arrive form: the block sums came from the prepare launch, only the planes cross workgroups
+                finish_block<true, FUSE == kOne>(a.dt, a.z, xs_row, a.svh, a.y, a.out, rows, a.ks, inblk, a.defer, row,
+                                                 b128, lane);
+            }
+            if (threadIdx.x == 0u)  // zero again for the next call
+                __hip_atomic_store(a.arrive + b128, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
 }
 
-template <int DT>
-__global__ void __launch_bounds__(64) dense_finish(const float* z, const float* xs, const uint16_t* svh, void* y,
-                                                   uint32_t out, uint32_t rows, uint32_t ks, uint32_t inblk,
-                                                   int defer) {
-    finish_block<DT>(z, xs, svh, y, out, rows, ks, inblk, defer, blockIdx.y, blockIdx.x, threadIdx.x);
-}
-
-template <int CB, bool WIDE, int RB>
-hipError_t launch_gemv_bt(const DenseLaunch& d, hipStream_t s) {
-    const dim3 block(256);
-    const uint32_t out_tiles = d.out / 16u;
-    auto go = [&](auto kern, uint32_t bt) {
-        hipLaunchKernelGGL(kern, dim3(out_tiles / bt, d.ks), block, 0, s, d.trellis, d.xq, d.z, d.in, d.out, d.rows,
-                           d.n, d.wbits, (d.in / 16u) / (4u * d.ks));
-        return hipGetLastError();
-    };
-    if (d.bt == 8u) return go(dense_gemv<CB, WIDE, RB, 8>, 8u);
-    return go(dense_gemv<CB, WIDE, RB, 4>, 4u);
+template <int CB, bool WIDE, int RB, int BT>
+hipError_t launch_gemv_fuse(const DenseLaunch& d, int fuse, hipStream_t s) {
+    GemvArgs a;
+    a.w = d.trellis;
+    a.xq = d.xq;
+    a.z = d.z;
+    a.xs = d.xs;
+    a.x = d.x;
+    a.suh = d.suh;
+    a.svh = d.svh;
+    a.y = d.y;
+    a.arrive = d.arrive;
+    a.in = d.in;
+    a.out = d.out;
+    a.rows = d.rows;
+    a.n = d.n;
+    a.wbits = d.wbits;
+    a.per = (d.in / 16u) / (4u * d.ks);
+    a.ks = d.ks;
+    a.dt = d.dtype;
+    a.defer = d.codebook == kMul1Defer;
+    const dim3 grid((d.out / 16u) / BT, d.ks), block(256);
+    if (fuse == kOne) {
+        if constexpr (RB == 1) {
+            const size_t dyn = 4u * (a.per + 1u) * (kXldsRows * 64u);
+            hipLaunchKernelGGL((dense_gemv<CB, WIDE, 1, BT, kOne>), grid, block, dyn, s, a);
+        } else {
+            return hipErrorInvalidValue;
+        }
+    } else if (fuse == kArrive) {
+        hipLaunchKernelGGL((dense_gemv<CB, WIDE, RB, BT, kArrive>), grid, block, 0, s, a);
+    } else {
+        hipLaunchKernelGGL((dense_gemv<CB, WIDE, RB, BT, kChain>), grid, block, 0, s, a);
+    }
+    return hipGetLastError();
 }
 
 template <int CB>
-hipError_t launch_gemv_cb(const DenseLaunch& d, hipStream_t s) {
+hipError_t launch_gemv_cb(const DenseLaunch& d, int fuse, hipStream_t s) {
     const bool wide = quad_needs_wide(d.n);
     const bool two = d.rows > 16u;
-    if (wide) return two ? launch_gemv_bt<CB, true, 2>(d, s) : launch_gemv_bt<CB, true, 1>(d, s);
-    return two ? launch_gemv_bt<CB, false, 2>(d, s) : launch_gemv_bt<CB, false, 1>(d, s);
+    const bool bt8 = d.bt == 8u;
+    if (wide) {
+        if (two) return bt8 ? launch_gemv_fuse<CB, true, 2, 8>(d, fuse, s) : launch_gemv_fuse<CB, true, 2, 4>(d, fuse, s);
+        return bt8 ? launch_gemv_fuse<CB, true, 1, 8>(d, fuse, s) : launch_gemv_fuse<CB, true, 1, 4>(d, fuse, s);
+    }
+    if (two) return bt8 ? launch_gemv_fuse<CB, false, 2, 8>(d, fuse, s) : launch_gemv_fuse<CB, false, 2, 4>(d, fuse, s);
+    return bt8 ? launch_gemv_fuse<CB, false, 1, 8>(d, fuse, s) : launch_gemv_fuse<CB, false, 1, 4>(d, fuse, s);
 }
 
 }  // namespace
 
 hipError_t launch_dense_prep(const DenseLaunch& d, hipStream_t s) {
-    const dim3 grid(d.in / 128u, d.rows), block(64);
-    switch (d.dtype) {
-        case kF32: hipLaunchKernelGGL(dense_prep<kF32>, grid, block, 0, s, d.x, d.suh, d.xq, d.xs, d.in); break;
-        case kF16: hipLaunchKernelGGL(dense_prep<kF16>, grid, block, 0, s, d.x, d.suh, d.xq, d.xs, d.in); break;
-        default: hipLaunchKernelGGL(dense_prep<kBf16>, grid, block, 0, s, d.x, d.suh, d.xq, d.xs, d.in); break;
-    }
+    hipLaunchKernelGGL(dense_prep, dim3(d.in / 128u, d.rows), dim3(64), 0, s, d.x, d.suh, d.xq, d.xs, d.in, d.dtype);
     return hipGetLastError();
 }
 
-hipError_t launch_dense_gemv(const DenseLaunch& d, hipStream_t s) {
+hipError_t launch_dense_gemv(const DenseLaunch& d, int fuse, hipStream_t s) {
     switch (d.codebook) {
-        case kMul1: return launch_gemv_cb<kMul1>(d, s);
-        case kMcg: return launch_gemv_cb<kMcg>(d, s);
-        case kMul1Defer: return launch_gemv_cb<kMul1Defer>(d, s);
-        default: return launch_gemv_cb<kMcgPair>(d, s);
+        case kMul1: return launch_gemv_cb<kMul1>(d, fuse, s);
+        case kMcg: return launch_gemv_cb<kMcg>(d, fuse, s);
+        case kMul1Defer: return launch_gemv_cb<kMul1Defer>(d, fuse, s);
+        default: return launch_gemv_cb<kMcgPair>(d, fuse, s);
     }
 }
 
 hipError_t launch_dense_finish(const DenseLaunch& d, hipStream_t s) {
-    const dim3 grid(d.out / 128u, d.rows), block(64);
-    const int defer = d.codebook == kMul1Defer;
-    const uint32_t inblk = d.in / 128u;
-    switch (d.dtype) {
-        case kF32:
-            hipLaunchKernelGGL(dense_finish<kF32>, grid, block, 0, s, d.z, d.xs, d.svh, d.y, d.out, d.rows, d.ks, inblk,
-                               defer);
-            break;
-        case kF16:
-            hipLaunchKernelGGL(dense_finish<kF16>, grid, block, 0, s, d.z, d.xs, d.svh, d.y, d.out, d.rows, d.ks, inblk,
-                               defer);
-            break;
-        default:
-            hipLaunchKernelGGL(dense_finish<kBf16>, grid, block, 0, s, d.z, d.xs, d.svh, d.y, d.out, d.rows, d.ks, inblk,
-                               defer);
-            break;
-    }
+    hipLaunchKernelGGL(dense_finish, dim3(d.out / 128u, d.rows), dim3(64), 0, s, d.z, d.xs, d.svh, d.y, d.out, d.rows,
+                       d.ks, d.in / 128u, static_cast<int>(d.codebook == kMul1Defer), d.dtype);
     return hipGetLastError();
 }
 

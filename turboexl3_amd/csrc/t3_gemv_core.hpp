@@ -12,6 +12,10 @@
 //
 // Sums: each MFMA output element depends on its own activation row alone, and a wave's tile rows are taken in
 // ascending order, so a row's partial sum is a function of (matrix, K part, row) only.
+//
+// Cost model (measured on MI355X): per tile a lane issues 13 vector-ALU instructions (1 v_alignbit, then v_bfe,
+// v_mul_lo, v_bitop3 a weight) and one MFMA; the MFMA holds the SIMD's issue for its 16 cycles, it does not overlap
+// vector ALU work. About 80 cycles a tile a SIMD: the kernel is instruction-bound below 6 bits a weight.
 #pragma once
 
 #include "t3_decode.hpp"
@@ -19,111 +23,176 @@
 namespace t3 {
 
 constexpr uint32_t kTileSlot = 256u;  // LDS bytes a staged tile (2n <= 256)
+constexpr uint32_t kXldsRows = 4u;    // activation rows the in-LDS form of the prepared input holds
 
-// LDS bytes one wave's stage takes: two buffers of BT tile slots
+// LDS bytes one wave's stage takes: two buffers of BT tile slots, then a dump where the lanes past a tile row's last
+// byte put their (zero) registers, so the store needs neither a branch nor a per-lane buffer offset: the dump is
+// 512 bytes plus one buffer's length, because a store to buffer 1 adds that length for every lane alike
 template <int BT>
 constexpr uint32_t gemv_stage_bytes() {
-    return 2u * BT * kTileSlot;
+    return 3u * BT * kTileSlot + 512u;
 }
 
+// Where a wave's prepared activations come from.
+struct XGlobal {            // u32 [rows][in], doubled f16 in quad order
+    const uint32_t* base;
+    uint64_t bytes;
+    uint32_t first;         // byte offset of the wave's first input tile inside a row (a tile: 64 bytes)
+};
+struct XLds {               // the wave's own [per + 1][kXldsRows][64 bytes], written by the in-kernel prepare;
+    const unsigned char* base;  // the last tile row all zeros: what a row past the wave's last multiplies by
+};
+
+// One wave's stream over `per` tile rows. Construct, `issue()` the first loads, do whatever else the kernel has to
+// do while they fly (the one-launch form prepares its activations there), then `run()`.
+//
 // wbase: the wave's first tile row (tile 0 of its BT); wstep: bytes from one tile row to the next; per: tile rows.
-// xbase/xbytes: the prepared rows (u32 [rows][in], doubled f16 in quad order); xoff[r]: the lane's byte offset of
-// block r's activation row plus its quad; xo: byte offset of the wave's first input tile inside a row (tile 64 B).
-// stage: the wave's own LDS bytes (gemv_stage_bytes<BT>()), 16-byte aligned.
-// acc[r][t] += the 16 x 16 product of activation block r and tile t, summed over the wave's tile rows in order.
-template <int CB, bool WIDE, int RB, int BT, int ST>
-__device__ __forceinline__ void gemv_stream(const uint32_t* wbase, uint32_t wstep, uint32_t per, uint32_t n,
-                                            const QuadPlan<WIDE>& plan, uint32_t wbits, const uint32_t* xbase,
-                                            uint64_t xbytes, const uint32_t (&xoff)[RB], uint32_t xo,
-                                            unsigned char* stage, uint32_t lane, float4v (&acc)[RB][BT]) {
-    const uint32_t tile_bytes = 2u * n;
-    const uint32_t chunk_bytes = static_cast<uint32_t>(BT) * tile_bytes;  // a multiple of 16: BT is 4 or 8, n even
-    // bytes from the wave's first tile row to the end of its last (the range check covers the scalar offset too)
-    const uint32_t span_bytes = (per - 1u) * wstep + chunk_bytes;
-    // a lane past the chunk asks for an offset no buffer reaches: zeros, no traffic
-    const uint32_t voff = lane * 16u < chunk_bytes ? lane * 16u : 0x40000000u;
-    // where the lane's four loaded dwords land: tile slot + offset inside the tile
-    uint32_t put[4];
-#pragma unroll
-    for (uint32_t j = 0; j < 4u; ++j) {
-        const uint32_t b = lane * 16u + 4u * j;
-        const uint32_t t = b / tile_bytes;
-        put[j] = t * kTileSlot + (b - t * tile_bytes);
-    }
-    const bool writer = lane * 16u < chunk_bytes;
-    // where the lane's quad words sit inside a tile slot
-    const uint32_t get_bp = plan.ib_prev * 4u, get_bl = plan.ib_last * 4u;
-    const uint32_t get_ap = plan.ia_prev * 4u, get_al = plan.ia_last * 4u;
+// xoff[r]: the lane's byte offset of block r's activation row plus its quad, inside a row (XGlobal) or inside a tile
+// row's kXldsRows x 64 bytes (XLds). stage: the wave's own LDS bytes (gemv_stage_bytes<BT>()), 16-byte aligned.
+// run(): acc[r][t] += the 16 x 16 product of activation block r and tile t, summed over the wave's tile rows in order.
+template <int CB, bool WIDE, int RB, int BT, int ST, typename XSrc>
+struct GemvStream {
+    static constexpr bool kXLds = __is_same(XSrc, XLds);
+    static_assert(ST % 2 == 0, "stage buffers and word sets alternate by ring slot parity");
 
-    auto load_chunk = [&](uint32_t row) -> uint4v {
-        const __amdgpu_buffer_rsrc_t res = make_rsrc(wbase, row < per ? span_bytes : 0u);
-        return buf_load_u128(res, voff, row * wstep);
-    };
-    auto load_x = [&](uint32_t row, uint4v(&dst)[RB]) {
-        const __amdgpu_buffer_rsrc_t res = make_rsrc(xbase, row < per ? xbytes : 0u);
-        const uint32_t soff = xo + row * 64u;
-#pragma unroll
-        for (int r = 0; r < RB; ++r) dst[r] = buf_load_u128(res, xoff[r], soff);
-    };
-    auto stage_chunk = [&](const uint4v& v, unsigned char* buf) {
-        if (writer) {
-#pragma unroll
-            for (uint32_t j = 0; j < 4u; ++j) *reinterpret_cast<uint32_t*>(buf + put[j]) = v[j];
-        }
-    };
-    auto consume = [&](const unsigned char* buf, const uint4v(&xv)[RB]) {
-#pragma unroll
-        for (int t = 0; t < BT; ++t) {
-            const unsigned char* slot = buf + static_cast<uint32_t>(t) * kTileSlot;
-            QuadWords<WIDE> words;
-            words.b_prev = *reinterpret_cast<const uint32_t*>(slot + get_bp);
-            words.b_last = *reinterpret_cast<const uint32_t*>(slot + get_bl);
-            if constexpr (WIDE) {
-                words.a_prev = *reinterpret_cast<const uint32_t*>(slot + get_ap);
-                words.a_last = *reinterpret_cast<const uint32_t*>(slot + get_al);
-            }
-            uint32_t cw[4];
-            quad_codewords<WIDE>(words, plan, wbits, cw);
-            uint4v a;
-#pragma unroll
-            for (int m = 0; m < 4; ++m) a[m] = weight_pair<CB>(cw[m]);
-#pragma unroll
-            for (int r = 0; r < RB; ++r)
-                acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a),
-                                                                   __builtin_bit_cast(half8, xv[r]), acc[r][t], 0, 0, 0);
-        }
-    };
-
-    // The activations ride the same ring as the codes: the load counter retires in order, so an activation load
-    // issued later than a tile row's would hold that row's wait back to the activations' shorter lead.
-    static_assert(ST % 2 == 0, "the LDS stage alternates two buffers by ring slot parity");
+    const uint32_t* wbase;
+    uint32_t wstep, per, n, wbits, lane;
+    XSrc xs;
+    uint32_t xoff[RB];
+    unsigned char* stage;
+    uint32_t span_bytes, voff;
+    // Three overlapped pipelines, all in the wave's own program order:
+    //   global -> registers   ST tile rows ahead (ring), the activations beside them: the load counter retires in
+    //                         order, so a load issued later than a row's would hold that row's wait back to its lead;
+    //   registers -> LDS -> registers   one row ahead (two stage buffers, two word sets by row parity);
+    //   decode + MFMA         the row whose words are already in registers.
     uint4v ring[ST];
     uint4v xr[ST][RB];
+
+    __device__ __forceinline__ GemvStream(const uint32_t* wbase_, uint32_t wstep_, uint32_t per_, uint32_t n_,
+                                          uint32_t wbits_, const XSrc& xs_, const uint32_t (&xoff_)[RB],
+                                          unsigned char* stage_, uint32_t lane_)
+        : wbase(wbase_), wstep(wstep_), per(per_), n(n_), wbits(wbits_), lane(lane_), xs(xs_), stage(stage_) {
 #pragma unroll
-    for (int s = 0; s < ST; ++s) {
-        load_x(static_cast<uint32_t>(s), xr[s]);
-        ring[s] = load_chunk(static_cast<uint32_t>(s));
-        __builtin_amdgcn_sched_barrier(0);  // issue order = ring order: the first row's wait must not cover the rest
+        for (int r = 0; r < RB; ++r) xoff[r] = xoff_[r];
+        const uint32_t chunk_bytes = static_cast<uint32_t>(BT) * 2u * n;  // a multiple of 16: BT is 4 or 8, n even
+        // bytes from the wave's first tile row to the end of its last (the range check covers the scalar offset too)
+        span_bytes = (per - 1u) * wstep + chunk_bytes;
+        // a lane past the chunk asks for an offset no buffer reaches: zeros, no traffic
+        voff = lane * 16u < chunk_bytes ? lane * 16u : 0x40000000u;
     }
-    for (uint32_t i = 0; i < per; i += ST) {
+
+    __device__ __forceinline__ uint4v load_chunk(uint32_t row) const {
+        const __amdgpu_buffer_rsrc_t res = make_rsrc(wbase, row < per ? span_bytes : 0u);
+        return buf_load_u128(res, voff, row * wstep);
+    }
+    __device__ __forceinline__ void load_x(uint32_t row, uint4v (&dst)[RB]) const {
+        if constexpr (!kXLds) {
+            const __amdgpu_buffer_rsrc_t res = make_rsrc(xs.base, row < per ? xs.bytes : 0u);
+            const uint32_t soff = xs.first + row * 64u;
 #pragma unroll
-        for (int s = 0; s < ST; ++s) {
-            const uint32_t row = i + static_cast<uint32_t>(s);
-            unsigned char* buf = stage + static_cast<uint32_t>(s & 1) * (BT * kTileSlot);
-            __builtin_amdgcn_sched_barrier(0);
-            if (row < per) {
-                stage_chunk(ring[s], buf);
-                uint4v xv[RB];
-#pragma unroll
-                for (int r = 0; r < RB; ++r) xv[r] = xr[s][r];
-                __builtin_amdgcn_sched_barrier(0);
-                ring[s] = load_chunk(row + ST);
-                load_x(row + ST, xr[s]);
-                __builtin_amdgcn_sched_barrier(0);
-                consume(buf, xv);
-            }
+            for (int r = 0; r < RB; ++r) dst[r] = buf_load_u128(res, xoff[r], soff);
         }
     }
-}
+
+    __device__ __forceinline__ void issue() {
+#pragma unroll
+        for (int s = 0; s < ST; ++s) {
+            ring[s] = load_chunk(static_cast<uint32_t>(s));
+            load_x(static_cast<uint32_t>(s), xr[s]);
+            __builtin_amdgcn_sched_barrier(0);  // issue order = ring order: the first row's wait must not cover the rest
+        }
+    }
+
+    __device__ __forceinline__ void run(float4v (&acc)[RB][BT]) {
+        const uint32_t tile_bytes = 2u * n;
+        const uint32_t chunk_bytes = static_cast<uint32_t>(BT) * tile_bytes;
+        // The loads are in flight; everything a lane needs to decode is worked out under their latency.
+        const QuadPlan<WIDE> plan = quad_plan<WIDE>(n, lane);
+        // where the lane's four loaded dwords land: tile slot + offset inside the tile (a lane past the chunk stores
+        // into the dump behind both buffers); b / tile_bytes by a 16-bit reciprocal, exact for b < 1024 and
+        // tile_bytes >= 32
+        const bool writer = lane * 16u < chunk_bytes;
+        const uint32_t inv_tile = (1u << 16) / tile_bytes + 1u;
+        uint32_t put[4];
+#pragma unroll
+        for (uint32_t j = 0; j < 4u; ++j) {
+            const uint32_t b = lane * 16u + 4u * j;
+            const uint32_t t = (b * inv_tile) >> 16;
+            put[j] = writer ? t * kTileSlot + (b - t * tile_bytes) : 2u * BT * kTileSlot + (lane & 31u) * 16u + 4u * j;
+        }
+        // where the lane's quad words sit inside a tile slot
+        const uint32_t get_bp = plan.ib_prev * 4u, get_bl = plan.ib_last * 4u;
+        const uint32_t get_ap = plan.ia_prev * 4u, get_al = plan.ia_last * 4u;
+
+        auto stage_chunk = [&](const uint4v& v, uint32_t parity) {
+#pragma unroll
+            for (uint32_t j = 0; j < 4u; ++j)
+                *reinterpret_cast<uint32_t*>(stage + parity * (BT * kTileSlot) + put[j]) = v[j];
+        };
+        // a tile row's words, read back from the stage into registers one row ahead of their decode
+        auto fetch = [&](uint32_t parity, uint32_t row, QuadWords<WIDE>(&wd)[BT], uint4v(&xv)[RB]) {
+            const unsigned char* buf = stage + parity * (BT * kTileSlot);
+#pragma unroll
+            for (int t = 0; t < BT; ++t) {
+                const unsigned char* slot = buf + static_cast<uint32_t>(t) * kTileSlot;
+                wd[t].b_prev = *reinterpret_cast<const uint32_t*>(slot + get_bp);
+                wd[t].b_last = *reinterpret_cast<const uint32_t*>(slot + get_bl);
+                if constexpr (WIDE) {
+                    wd[t].a_prev = *reinterpret_cast<const uint32_t*>(slot + get_ap);
+                    wd[t].a_last = *reinterpret_cast<const uint32_t*>(slot + get_al);
+                }
+            }
+            if constexpr (kXLds) {
+                const uint32_t xrow = row < per ? row : per;  // past the last: the zero row
+#pragma unroll
+                for (int r = 0; r < RB; ++r)
+                    xv[r] = *reinterpret_cast<const uint4v*>(xs.base + xrow * (kXldsRows * 64u) + xoff[r]);
+            }
+        };
+        auto consume = [&](const QuadWords<WIDE>(&wd)[BT], const uint4v(&xv)[RB]) {
+#pragma unroll
+            for (int t = 0; t < BT; ++t) {
+                uint32_t cw[4];
+                quad_codewords<WIDE>(wd[t], plan, wbits, cw);
+                uint4v a;
+#pragma unroll
+                for (int m = 0; m < 4; ++m) a[m] = weight_pair<CB>(cw[m]);
+#pragma unroll
+                for (int r = 0; r < RB; ++r)
+                    acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                        __builtin_bit_cast(half8, a), __builtin_bit_cast(half8, xv[r]), acc[r][t], 0, 0, 0);
+            }
+        };
+
+        QuadWords<WIDE> words[2][BT];
+        uint4v xw[2][RB];  // XLds: the activations of the row being decoded and of the next, read beside the words
+        stage_chunk(ring[0], 0u);
+        ring[0] = load_chunk(ST);
+        fetch(0u, 0u, words[0], xw[0]);
+        // No branch inside the ring: a row past the wave's last arrives as zeros for the codes, and multiplies zero
+        // activations (a zero-sized buffer, or the LDS form's zero row); the decoded weights of zero codes are finite,
+        // so the products add nothing. (Branches here also cost the compiler its count of the loads in flight: it
+        // then drains them all at every join.)
+        uint32_t i = 0;
+        do {
+#pragma unroll
+            for (int s = 0; s < ST; ++s) {
+                const uint32_t row = i + static_cast<uint32_t>(s);
+                const int sn = (s + 1) % ST;  // the ring slot of row + 1
+                __builtin_amdgcn_sched_barrier(0);
+                stage_chunk(ring[sn], static_cast<uint32_t>(sn & 1));
+                ring[sn] = load_chunk(row + 1u + ST);
+                fetch(static_cast<uint32_t>(sn & 1), row + 1u, words[sn & 1], xw[sn & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (kXLds) consume(words[s & 1], xw[s & 1]);
+                else consume(words[s & 1], xr[s]);
+                __builtin_amdgcn_sched_barrier(0);
+                load_x(row + ST, xr[s]);
+            }
+            i += ST;
+        } while (i < per);
+    }
+};
 
 }  // namespace t3

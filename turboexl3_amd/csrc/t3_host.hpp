@@ -67,17 +67,27 @@ constexpr uint32_t kGemvTargetWgs = 768; // three workgroups a CU
 constexpr uint32_t kGemvMinPer = 4;      // input tiles a wave at least
 
 // K slices of a GEMV over in_tiles input tiles and `groups` workgroup columns: the smallest divisor d of
-// in_tiles / 4 that reaches the target workgroup count while every wave keeps kGemvMinPer tiles.
+// in_tiles / 4 that reaches the target workgroup count while every wave keeps kGemvMinPer tiles. Splits that leave a
+// wave whole 128-blocks of the input (per % 8 == 0) are preferred: the one-launch form prepares its input by block.
 inline uint32_t gemv_slices(uint32_t in_tiles, uint32_t groups) {
     const uint32_t q = in_tiles / 4u;
-    uint32_t best = 1;
-    for (uint32_t d = 1; d <= q; ++d) {
-        if (q % d != 0) continue;
-        if (q / d < kGemvMinPer && d > 1) break;
-        best = d;
-        if (static_cast<uint64_t>(groups) * d >= kGemvTargetWgs) break;
+    for (int whole = 1; whole >= 0; --whole) {
+        uint32_t best = 0;
+        for (uint32_t d = 1; d <= q; ++d) {
+            if (q % d != 0) continue;
+            const uint32_t per = q / d;
+            if (per < kGemvMinPer && d > 1) break;
+            if (whole && per % 8u != 0u) continue;
+            best = d;
+            if (static_cast<uint64_t>(groups) * d >= kGemvTargetWgs) break;
+        }
+        if (best != 0) return best;
     }
-    return best;
+    return 1;
 }
+
+// The caller's workspace starts with the arrival counters of the fused launches, at a fixed place and size whatever
+// the call's shapes: zero when the workspace is first passed, and zero again after every call.
+constexpr size_t kCounterBytes = 65536;
 
 }  // namespace t3

@@ -26,8 +26,12 @@ struct DenseLaunch {
     uint32_t ks = 1, bt = 4;
 };
 
+// the GEMV launch's form: 0 planes only (the chain), 1 + the finish by the last workgroup to arrive at a column block,
+// 2 + the prepare inside the launch (up to 4 rows)
+enum DenseFuse : int { kFuseChain = 0, kFuseArrive = 1, kFuseOne = 2 };
+
 hipError_t launch_dense_prep(const DenseLaunch& d, hipStream_t s);
-hipError_t launch_dense_gemv(const DenseLaunch& d, hipStream_t s);
+hipError_t launch_dense_gemv(const DenseLaunch& d, int fuse, hipStream_t s);
 hipError_t launch_dense_finish(const DenseLaunch& d, hipStream_t s);
 
 // trellis [in/16][out/16][n] -> W_hat f16 [in][out], bit-exact (format.reconstructInner)

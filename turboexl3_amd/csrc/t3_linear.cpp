@@ -44,6 +44,7 @@ int32_t check_dense(const t3_array* x, const t3_array* trellis, const t3_array* 
     if (max_rows != 0 && rows > max_rows) return T3_Exl3EngineNotImplemented;
     // the kernels address one matrix, and one call's prepared rows, through 32-bit byte offsets
     if ((in / 16) * (out / 16) * n * 2 >= (1ll << 31) || rows * in * 4 >= (1ll << 31)) return T3_Exl3EngineNotImplemented;
+    if (out / 128 > static_cast<int64_t>(kCounterBytes / 4)) return T3_Exl3EngineNotImplemented;
 
     DenseLaunch& l = call->launch;
     l.x = x->data;
@@ -63,14 +64,16 @@ int32_t check_dense(const t3_array* x, const t3_array* trellis, const t3_array* 
     return T3_OK;
 }
 
-// xq u32 [rows][in], xs f32 [rows][in / 128], z f32 [ks][rows][out], arrival counters u32 [out / 128]
+// arrival counters u32 [out / 128] (fixed place), xq u32 [rows][in], xs f32 [rows][in / 128], z f32 [ks][rows][out]
 void carve_dense(DenseCall* call, void* workspace) {
     DenseLaunch& l = call->launch;
     Carver c(workspace);
+    l.arrive = c.take<uint32_t>(kCounterBytes);
     l.xq = c.take<uint32_t>(static_cast<size_t>(l.rows) * l.in * 4u);
-    l.xs = c.take<float>(static_cast<size_t>(l.rows) * (l.in / 128u) * 4u);
+    // the one-launch form keeps a copy of the block sums a 128-column block (up to 4 rows)
+    const size_t xs_copies = l.rows <= 4u ? l.out / 128u : 1u;
+    l.xs = c.take<float>(xs_copies * l.rows * (l.in / 128u) * 4u);
     l.z = c.take<float>(static_cast<size_t>(l.ks) * l.rows * l.out * 4u);
-    l.arrive = c.take<uint32_t>(static_cast<size_t>(l.out / 128u) * 4u);
     call->workspace = c.used;
 }
 
@@ -78,9 +81,22 @@ int32_t run_chain(const DenseCall& call, hipStream_t s, uint32_t stages) {
     if (stages & T3_STAGE_PREPARE)
         if (const int32_t st = hip_status(launch_dense_prep(call.launch, s)); st != T3_OK) return st;
     if (stages & T3_STAGE_GEMV)
-        if (const int32_t st = hip_status(launch_dense_gemv(call.launch, s)); st != T3_OK) return st;
+        if (const int32_t st = hip_status(launch_dense_gemv(call.launch, kFuseChain, s)); st != T3_OK) return st;
     if (stages & T3_STAGE_FINISH) return hip_status(launch_dense_finish(call.launch, s));
     return T3_OK;
+}
+
+// The served form (src/core/dense.zig:1229-1242 takes DEC-ONE up to 4 rows the same way). Up to 4 rows: one launch
+// where a wave's K part is whole 128-blocks and small enough to prepare in LDS, else the prepare launch and the
+// arriving GEMV. More rows: the chain (measured: with 16 and 32 rows the planes' coherent traffic costs the arriving
+// form more than the finish launch it saves).
+int32_t run_fused(const DenseCall& call, hipStream_t s) {
+    const DenseLaunch& l = call.launch;
+    const uint32_t per = (l.in / 16u) / (4u * l.ks);
+    if (l.rows > 4u) return run_chain(call, s, 7u);
+    if (per % 8u == 0u && per <= 16u) return hip_status(launch_dense_gemv(l, kFuseOne, s));
+    if (const int32_t st = hip_status(launch_dense_prep(l, s)); st != T3_OK) return st;
+    return hip_status(launch_dense_gemv(l, kFuseArrive, s));
 }
 
 }  // namespace
@@ -118,7 +134,14 @@ int32_t t3_linear_stages(t3_stream stream, const t3_array* x, const t3_array* tr
 
 int32_t t3_linear(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
                   const t3_array* svh, t3_decode dec, t3_array* y, void* workspace, size_t workspace_bytes) {
-    return t3_linear_chain(stream, x, trellis, suh, svh, dec, y, workspace, workspace_bytes);
+    if (!suh || !svh || !y) return T3_BadArgs;
+    t3::DenseCall call;
+    if (const int32_t st = t3::check_dense(x, trellis, suh, svh, dec, y, 32, &call); st != T3_OK) return st;
+    if (!workspace) return T3_BadArgs;
+    t3::carve_dense(&call, workspace);
+    if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
+    if (!t3::config().dec_one) return t3::run_chain(call, static_cast<hipStream_t>(stream), 7u);
+    return t3::run_fused(call, static_cast<hipStream_t>(stream));
 }
 
 int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_array* w_hat) {
