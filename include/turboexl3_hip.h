@@ -140,7 +140,10 @@ int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_
 /* ---- routed experts (src/root.zig:822-904,976-1004) ------------------------------------------------------- */
 
 /* x [B, S, D]; inds (U32/I32) and scores (F32/BF16/F16) [B, S, K], K <= 32; y [B, S, D] in x's dtype.
- * `verify_rows` is accepted and ignored, as in the reference (src/root.zig:822-825). */
+ * `verify_rows` is accepted and ignored, as in the reference (src/root.zig:822-825). Up to 16 rows: the split-K GEMV
+ * chain, four launches (five under decode_form 3, the same bytes). A routed id outside [0, E) is skipped. Gate and up
+ * must share a rate (T3_Exl3GateUpRateMismatch); the down's rate may differ (the reference refuses that,
+ * src/root.zig:841; this library's kernels take a rate a launch). */
 int32_t t3_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
                const t3_array* scores, t3_decode dec, int32_t verify_rows, t3_array* y, void* workspace,
                size_t workspace_bytes);
@@ -154,7 +157,17 @@ int32_t t3_moe_clamped(t3_stream stream, const t3_array* x, const t3_bank* bank,
 int32_t t3_moe_with_shared(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
                            const t3_array* scores, t3_decode dec, int32_t verify_rows, const t3_array* shared,
                            t3_array* y, void* workspace, size_t workspace_bytes);
-int32_t t3_moe_workspace_bytes(const t3_array* x, const t3_bank* bank, const t3_array* inds, size_t* bytes);
+/* The routed experts with a shared expert inside the same launches: every row also runs each expert of `shared_bank`
+ * (same widths and rates as `bank`) at weight 1, summed after the row's routed slots in f32 before the output
+ * rounding. limit 0: no clamp; 1..128: `t3_moe_clamped`'s. The role of Qwen3.8's fused shared expert
+ * (src/models/qwen38/api.zig:305-312) with the gate left to the caller; the reference's own `moeWithShared` adds a
+ * finished tensor instead. */
+int32_t t3_moe_shared_expert(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
+                             const t3_array* scores, t3_decode dec, int32_t limit, const t3_bank* shared_bank,
+                             t3_array* y, void* workspace, size_t workspace_bytes);
+/* shared_bank: NULL, or the bank `t3_moe_shared_expert` will take (its slots need scratch too). */
+int32_t t3_moe_workspace_bytes(const t3_array* x, const t3_bank* bank, const t3_array* inds,
+                               const t3_bank* shared_bank, size_t* bytes);
 
 /* ---- pack contract (src/core/spec.zig) ------------------------------------------------------------------- */
 

@@ -1,0 +1,230 @@
+"""The routed-expert decode chain against ref.moeRowClamped (the CPU oracle): the cases and bars of turboexl3
+src/hip_tests.zig:444-504,885-928 (f32 5e-3, bf16 1.5e-2 of rms per row; a row alone == the row among others, byte for
+byte; the four-launch form == the five-launch form, byte for byte), plus the clamp, skipped slots, mixed rates and the
+shared expert."""
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_util import MCG, MUL1, bytes_of, dev_f16_bits, dev_u16, make_x, to_f32
+
+pytestmark = pytest.mark.gpu
+
+F32_BAR = 5e-3
+BF16_BAR = 1.5e-2
+
+
+@pytest.fixture(scope="module")
+def t3():
+    from turboexl3_amd import api
+    return api
+
+
+def dev_bank(t3, b):
+    def proj(t, suh, svh):
+        return t3.Proj(dev_u16(t), dev_f16_bits(suh), dev_f16_bits(svh))
+    return t3.Bank(proj(b.gate_t, b.gate_suh, b.gate_svh), proj(b.up_t, b.up_suh, b.up_svh),
+                   proj(b.down_t, b.down_suh, b.down_svh))
+
+
+class RefBank:
+    """ref.moeRowClamped composed from the oracle's `project` stages on W_hat decoded once per expert (the bits of
+    format.project; tests/test_oracle_pins.py holds the composition to the C moe_row)."""
+
+    def __init__(self, oracle, bank, codebook, mask):
+        self.o, self.b, self.cb, self.mask = oracle, bank, codebook, mask
+        self.cache = {}
+
+    def _what(self, which, e):
+        key = (which, e)
+        if key not in self.cache:
+            b = self.b
+            t, in_f, out_f, n = {"gate": (b.gate_t, b.hidden, b.inter, b.n_gu), "up": (b.up_t, b.hidden, b.inter, b.n_gu),
+                                 "down": (b.down_t, b.inter, b.hidden, b.n_dn)}[which]
+            self.cache[key] = self.o.reconstruct_inner(t[e], in_f, out_f, n, self.cb, self.mask)
+        return self.cache[key]
+
+    def project(self, which, e, x):
+        b = self.b
+        t, suh, svh, in_f, out_f, n = {
+            "gate": (b.gate_t, b.gate_suh, b.gate_svh, b.hidden, b.inter, b.n_gu),
+            "up": (b.up_t, b.up_suh, b.up_svh, b.hidden, b.inter, b.n_gu),
+            "down": (b.down_t, b.down_suh, b.down_svh, b.inter, b.hidden, b.n_dn)}[which]
+        return self.o.project_rows(x[None, :], t[e], suh[e], svh[e], in_f, out_f, n, self.cb, self.mask, threads=8,
+                                   w_hat=self._what(which, e))[0]
+
+    def slot(self, e, x, limit):
+        g, u = self.project("gate", e, x), self.project("up", e, x)
+        if limit > 0:
+            g = np.minimum(g, np.float32(limit))
+            u = np.clip(u, -limit, limit).astype(np.float32)
+        h = ((g / (np.float32(1) + np.exp(-g).astype(np.float32))).astype(np.float32) * u).astype(np.float32)
+        return self.project("down", e, h)
+
+    def row(self, x, slots, scores, limit=0.0):
+        acc = np.zeros(self.b.hidden, dtype=np.float32)
+        for e, w in zip(slots, scores):
+            if 0 <= e < self.b.experts:
+                acc = (acc + (np.float32(w) * self.slot(int(e), x, limit)).astype(np.float32)).astype(np.float32)
+        return acc
+
+
+def routing(rng, rows, topk, experts):
+    slots = np.stack([rng.permutation(experts)[:topk] for _ in range(rows)]).astype(np.int32)
+    scores = (0.05 + rng.random((rows, topk)) * 0.2).astype(np.float32)
+    return slots, scores
+
+
+CASES = [
+    # (hidden, inter, experts, topk, n, codebook, wbits, dtype): src/hip_tests.zig:451-458's list
+    (512, 256, 12, 4, 64, MCG, 16, torch.float32),
+    (512, 256, 12, 4, 64, MUL1, 16, torch.float32),
+    (512, 256, 12, 8, 36, MCG, 16, torch.float32),
+    (512, 384, 12, 4, 128, MUL1, 12, torch.float32),
+    (2560, 640, 16, 10, 48, MUL1, 16, torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("hidden,inter,experts,topk,n,codebook,wbits,dtype", CASES)
+def test_moe_decode_rows_1_to_16(oracle, t3, hidden, inter, experts, topk, n, codebook, wbits, dtype):
+    rng = np.random.default_rng(0xF03 + hidden + n)
+    bank = oracle.synth_bank(rng, experts, hidden, inter, n)
+    dbank = dev_bank(t3, bank)
+    ref = RefBank(oracle, bank, codebook, (1 << wbits) - 1)
+    dec = t3.Decode(codebook, wbits)
+    max_rows = 16
+    x_dev, x_f32 = make_x(rng, max_rows, hidden, dtype)
+    slots, scores = routing(rng, max_rows, topk, experts)
+    d_slots, d_scores = torch.from_numpy(slots).cuda(), torch.from_numpy(scores).cuda()
+    yref = np.stack([ref.row(x_f32[r], slots[r], scores[r]) for r in range(max_rows)])
+    bar = F32_BAR if dtype == torch.float32 else BF16_BAR
+    worst = 0.0
+    for rows in (1, 2, 3, 4, 5, 8, 16):
+        y = t3.moe(x_dev[:rows].reshape(1, rows, hidden), dbank, d_slots[:rows].reshape(1, rows, topk),
+                   d_scores[:rows].reshape(1, rows, topk), dec)
+        assert y.shape == (1, rows, hidden) and y.dtype == dtype
+        got = to_f32(y).reshape(rows, hidden)
+        for r in range(rows):
+            e = oracle.compare(got[r], yref[r])
+            worst = max(worst, e)
+            assert e <= bar, f"rows {rows} row {r}: {e:.3e} over the bar {bar}"
+        if rows > 1:
+            for r in (0, rows - 1):
+                alone = t3.moe(x_dev[r:r + 1].reshape(1, 1, hidden), dbank, d_slots[r:r + 1].reshape(1, 1, topk),
+                               d_scores[r:r + 1].reshape(1, 1, topk), dec)
+                assert bytes_of(alone) == bytes_of(y[0, r]), f"rows {rows}: row {r} differs from the row alone"
+    print(f"moe decode {hidden}x{inter} n={n} cb={codebook} {dtype}: worst {worst:.3e} (bar {bar})")
+
+
+def test_four_launch_form_equals_five_launch_form(oracle, t3):
+    # src/hip_tests.zig:885-928: form 9's bytes are form 3's
+    rng = np.random.default_rng(9)
+    for codebook, n in ((MCG, 64), (MUL1, 48)):
+        bank = oracle.synth_bank(rng, 8, 512, 256, n)
+        dbank = dev_bank(t3, bank)
+        x_dev, _ = make_x(rng, 5, 512, torch.bfloat16)
+        slots, scores = routing(rng, 5, 4, 8)
+        args = (x_dev.reshape(1, 5, 512), dbank, torch.from_numpy(slots).cuda().reshape(1, 5, 4),
+                torch.from_numpy(scores).cuda().reshape(1, 5, 4), t3.Decode(codebook, 16))
+        nine = t3.moe(*args)
+        t3.configure(decode_form=3)
+        try:
+            three = t3.moe(*args)
+        finally:
+            t3.configure()
+        assert bytes_of(nine) == bytes_of(three)
+
+
+def test_clamp_skipped_slots_and_score_dtypes(oracle, t3):
+    rng = np.random.default_rng(21)
+    hidden, inter, experts, topk, n = 512, 256, 6, 4, 64
+    bank = oracle.synth_bank(rng, experts, hidden, inter, n)
+    dbank = dev_bank(t3, bank)
+    ref = RefBank(oracle, bank, MCG, 0xFFFF)
+    x_dev, x_f32 = make_x(rng, 3, hidden, torch.float32)
+    slots, scores = routing(rng, 3, topk, experts)
+    slots[1, 2] = -1          # skipped
+    slots[2, 0] = experts     # out of range: skipped
+    d_slots = torch.from_numpy(slots).cuda().reshape(1, 3, topk)
+    d_scores = torch.from_numpy(scores).cuda().reshape(1, 3, topk)
+    x3 = x_dev.reshape(1, 3, hidden)
+    limit = 1  # gate and up are O(1): a limit of 1 clamps a good share of them
+    y = to_f32(t3.moe_clamped(x3, dbank, d_slots, d_scores, t3.Decode.mcg, limit)).reshape(3, hidden)
+    unclamped = to_f32(t3.moe(x3, dbank, d_slots, d_scores, t3.Decode.mcg)).reshape(3, hidden)
+    for r in range(3):
+        want = ref.row(x_f32[r], slots[r], scores[r], float(limit))
+        assert oracle.compare(y[r], want) <= F32_BAR
+        assert oracle.compare(unclamped[r], ref.row(x_f32[r], slots[r], scores[r])) <= F32_BAR
+        assert oracle.compare(y[r], unclamped[r]) > 0.05, "the clamp should change this case"
+        _, hits = oracle.moe_row(bank, x_f32[r], slots[r], scores[r], MCG, limit=float(limit))
+        assert hits[0] > 0 and hits[1] > 0
+    # a limit no value reaches gives the unclamped bytes (the reference's clamped == unclamped at limit 128)
+    small = oracle.synth_bank(rng, experts, hidden, inter, n)
+    dsmall = dev_bank(t3, small)
+    a = t3.moe_clamped(x3, dsmall, d_slots, d_scores, t3.Decode.mcg, 128)
+    b = t3.moe(x3, dsmall, d_slots, d_scores, t3.Decode.mcg)
+    assert bytes_of(a) == bytes_of(b)
+    # scores arrive in bf16 / f16 and are widened exactly; ids as uint32
+    for sdt in (torch.bfloat16, torch.float16):
+        s16 = d_scores.to(sdt)
+        got = t3.moe(x3, dsmall, d_slots, s16, t3.Decode.mcg)
+        want = t3.moe(x3, dsmall, d_slots, s16.to(torch.float32), t3.Decode.mcg)
+        assert bytes_of(got) == bytes_of(want)
+
+
+def test_mixed_rates_and_shared_expert(oracle, t3):
+    # gate|up at K2, down at K3 (the reference refuses mixed rates; these kernels take a rate a launch), and a shared
+    # expert as one more slot of every row at weight 1
+    rng = np.random.default_rng(33)
+    hidden, inter, experts, topk = 512, 256, 8, 3
+    bank = oracle.synth_bank(rng, experts, hidden, inter, 32, 48)
+    shared = oracle.synth_bank(rng, 1, hidden, inter, 32, 48)
+    dbank, dshared = dev_bank(t3, bank), dev_bank(t3, shared)
+    ref, sref = RefBank(oracle, bank, MUL1, 0xFFFF), RefBank(oracle, shared, MUL1, 0xFFFF)
+    x_dev, x_f32 = make_x(rng, 4, hidden, torch.float16)
+    slots, scores = routing(rng, 4, topk, experts)
+    d_slots = torch.from_numpy(slots).cuda().reshape(2, 2, topk)
+    d_scores = torch.from_numpy(scores).cuda().reshape(2, 2, topk)
+    x3 = x_dev.reshape(2, 2, hidden)
+    half_ulp = 2.0 ** -11
+    y = to_f32(t3.moe(x3, dbank, d_slots, d_scores, t3.Decode.mul1)).reshape(4, hidden)
+    ys = to_f32(t3.moe_shared_expert(x3, dbank, d_slots, d_scores, t3.Decode.mul1, 0, dshared)).reshape(4, hidden)
+    for r in range(4):
+        routed = ref.row(x_f32[r], slots[r], scores[r])
+        assert oracle.compare(y[r], routed, half_ulp) <= F32_BAR
+        both = (routed + sref.slot(0, x_f32[r], 0.0)).astype(np.float32)
+        assert oracle.compare(ys[r], both, half_ulp) <= F32_BAR
+    # moeWithShared: the routed output rounded to x's dtype, plus a finished shared tensor, rounded again
+    sh = (rng.standard_normal((2, 2, hidden)) * 0.1).astype(np.float16)
+    yw = t3.moe_with_shared(x3, dbank, d_slots, d_scores, t3.Decode.mul1, False, torch.from_numpy(sh).cuda())
+    want = (t3.moe(x3, dbank, d_slots, d_scores, t3.Decode.mul1).to(torch.float32) + torch.from_numpy(sh).cuda().to(torch.float32)).to(torch.float16)
+    assert bytes_of(yw) == bytes_of(want)
+
+
+def test_moe_refusals(oracle, t3):
+    rng = np.random.default_rng(1)
+    bank = oracle.synth_bank(rng, 4, 256, 128, 32)
+    dbank = dev_bank(t3, bank)
+    x = torch.zeros(1, 1, 256, dtype=torch.float16, device="cuda")
+    inds = torch.zeros(1, 1, 2, dtype=torch.int32, device="cuda")
+    scores = torch.ones(1, 1, 2, dtype=torch.float32, device="cuda")
+
+    def name(fn):
+        with pytest.raises(t3.T3Error) as e:
+            fn()
+        return e.value.name
+
+    assert name(lambda: t3.moe_clamped(x, dbank, inds, scores, t3.Decode.mcg, 0)) == "InvalidExl3Clamp"
+    assert name(lambda: t3.moe_clamped(x, dbank, inds, scores, t3.Decode.mcg, 129)) == "InvalidExl3Clamp"
+    assert name(lambda: t3.moe(x[0], dbank, inds, scores, t3.Decode.mcg)) == "BadExl3Shape"
+    assert name(lambda: t3.moe(x, dbank, inds, scores[:, :, :1], t3.Decode.mcg)) == "BadExl3Shape"
+    big = torch.zeros(1, 1, 33, dtype=torch.int32, device="cuda")
+    assert name(lambda: t3.moe(x, dbank, big, torch.ones(1, 1, 33, device="cuda"), t3.Decode.mcg)) == "BadExl3Shape"
+    assert name(lambda: t3.moe(x, dbank, inds.to(torch.int16), scores, t3.Decode.mcg)) == "BadExl3Dtype"
+    assert name(lambda: t3.moe(x, dbank, inds, scores.to(torch.int32), t3.Decode.mcg)) == "BadExl3Dtype"
+    mism = oracle.synth_bank(rng, 4, 256, 128, 32)
+    mism.up_t = rng.integers(0, 65536, (4, 16, 8, 48), dtype=np.uint16)
+    assert name(lambda: t3.moe(x, dev_bank(t3, mism), inds, scores, t3.Decode.mcg)) == "Exl3GateUpRateMismatch"
+    bad = oracle.synth_bank(rng, 4, 256, 128, 32)
+    bad.down_svh = bad.down_svh[:, :128]
+    assert name(lambda: t3.moe(x, dev_bank(t3, bad), inds, scores, t3.Decode.mcg)) == "BadExl3Shape"

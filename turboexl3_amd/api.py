@@ -166,9 +166,10 @@ def _cbank(bank: Bank):
     return CBank(proj(bank.gate), proj(bank.up), proj(bank.down)), keep
 
 
-def _moe_workspace(L, ax, cb, ai, device):
+def _moe_workspace(L, ax, cb, ai, device, shared=None):
     need = C.c_size_t(0)
-    _check(L.t3_moe_workspace_bytes(C.byref(ax), C.byref(cb), C.byref(ai), C.byref(need)))
+    _check(L.t3_moe_workspace_bytes(C.byref(ax), C.byref(cb), C.byref(ai), C.byref(shared) if shared is not None else None,
+                                    C.byref(need)))
     return _workspace(device, need.value)
 
 
@@ -210,6 +211,20 @@ def moe_with_shared(x, bank: Bank, inds, scores, dec: Decode, verify_rows: bool,
     ay = _arr(y)
     _check(L.t3_moe_with_shared(_stream_ptr(stream), C.byref(ax), C.byref(cb), C.byref(ai), C.byref(asc), dec.c(),
                                 int(verify_rows), C.byref(ash), C.byref(ay), ws.data_ptr(), ws.numel()))
+    return y
+
+
+def moe_shared_expert(x, bank: Bank, inds, scores, dec: Decode, limit: int, shared_bank: Bank, stream=None) -> torch.Tensor:
+    """The routed experts with every expert of `shared_bank` as extra slots of each row at weight 1 (limit 0: no clamp)."""
+    L = _lib.lib()
+    ax, ai, asc = _arr(x), _arr(inds), _arr(scores)
+    cb, _keep = _cbank(bank)
+    sb, _keep2 = _cbank(shared_bank)
+    ws = _moe_workspace(L, ax, cb, ai, x.device, sb)
+    y = torch.empty_like(x)
+    ay = _arr(y)
+    _check(L.t3_moe_shared_expert(_stream_ptr(stream), C.byref(ax), C.byref(cb), C.byref(ai), C.byref(asc), dec.c(),
+                                  int(limit), C.byref(sb), C.byref(ay), ws.data_ptr(), ws.numel()))
     return y
 
 

@@ -21,43 +21,12 @@
 
 #include "t3_gemv_core.hpp"
 #include "t3_kernels.hpp"
+#include "t3_stages.hpp"
 
 namespace t3 {
 namespace {
 
 enum Fuse : int { kChain = 0, kArrive = 1, kOne = 2 };
-
-__device__ __forceinline__ float load_act_rt(int dt, const void* p, size_t i) {
-    if (dt == kF32) return load_act<kF32>(p, i);
-    if (dt == kF16) return load_act<kF16>(p, i);
-    return load_act<kBf16>(p, i);
-}
-__device__ __forceinline__ void store_act_rt(int dt, void* p, size_t i, float v) {
-    if (dt == kF32) store_act<kF32>(p, i, v);
-    else if (dt == kF16) store_act<kF16>(p, i, v);
-    else store_act<kBf16>(p, i, v);
-}
-
-// One 128-block of one row, one wave: lane L owns elements L and L + 64. Returns the lane's two prepared f16 values
-// (bits) and the block's sum of them (the same in every lane).
-__device__ __forceinline__ void prep_values(int dt, const void* x, const uint16_t* suh, uint32_t in, uint32_t row,
-                                            uint32_t b, uint32_t lane, uint32_t (&hv)[2], float& sum) {
-    float v[2];
-#pragma unroll
-    for (uint32_t j = 0; j < 2u; ++j) {
-        const uint32_t i = b * 128u + lane + 64u * j;
-        v[j] = round_half(load_act_rt(dt, x, static_cast<size_t>(row) * in + i)) * half_value(suh[i]);
-    }
-    h128_wave(v, lane);
-    sum = 0.0f;
-#pragma unroll
-    for (uint32_t j = 0; j < 2u; ++j) {
-        hv[j] = half_bits(v[j] * kHadScale);
-        sum += half_value(hv[j]);
-    }
-#pragma unroll
-    for (int m = 32; m > 0; m >>= 1) sum += __shfl_xor(sum, m, 64);
-}
 
 // Grid (in / 128, rows), 64 threads. xq: uint32 [rows][in], word (tk 16 + quad_slot(r)) = the f16 value of input
 // tk 16 + r in both halves. xs: f32 [rows][in / 128].

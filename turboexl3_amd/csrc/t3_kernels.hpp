@@ -34,6 +34,49 @@ hipError_t launch_dense_prep(const DenseLaunch& d, hipStream_t s);
 hipError_t launch_dense_gemv(const DenseLaunch& d, int fuse, hipStream_t s);
 hipError_t launch_dense_finish(const DenseLaunch& d, hipStream_t s);
 
+// A bank of experts, expert e on axis 0 (turboexl3 src/root.zig:73-76): trellis [E][in/16][out/16][n] as u32 words,
+// suh f16 [E][in], svh f16 [E][out]; gate, up: hidden -> inter; down: inter -> hidden.
+struct RoutedBank {
+    const uint32_t* gate_t = nullptr;
+    const uint32_t* up_t = nullptr;
+    const uint32_t* down_t = nullptr;
+    const uint16_t* gate_suh = nullptr;
+    const uint16_t* up_suh = nullptr;
+    const uint16_t* down_suh = nullptr;
+    const uint16_t* gate_svh = nullptr;
+    const uint16_t* up_svh = nullptr;
+    const uint16_t* down_svh = nullptr;
+    uint32_t experts = 0;
+};
+
+// One routed call at decode rows. Scratch by the reference's role names (src/hip/plan.zig:29-39).
+struct MoeLaunch {
+    RoutedBank bank, shared;     // shared: the bank the shared slots read (shared_slots of its experts, in order)
+    const void* x = nullptr;     // [rows][hidden] in dtype
+    const int32_t* slots = nullptr;  // [rows][topk] expert ids
+    const void* scores = nullptr;    // [rows][topk] in score_dt
+    const void* shared_add = nullptr;  // moeWithShared: [rows][hidden] in dtype, or null
+    void* y = nullptr;
+    uint32_t* xg = nullptr;      // u32 [RKT][hidden]
+    uint32_t* xu = nullptr;
+    uint32_t* hd = nullptr;      // u32 [RKT][inter]
+    float* sg = nullptr;         // f32 [RKT][hidden / 128]
+    float* su = nullptr;
+    float* hs = nullptr;         // f32 [RKT][inter / 128]
+    float* zg = nullptr;         // f32 [ks_gu][RKT][inter]
+    float* zu = nullptr;
+    float* zd = nullptr;         // f32 [ks_dn][RKT][hidden]
+    uint32_t hidden = 0, inter = 0, rows = 0, topk = 0, shared_slots = 0;
+    uint32_t n_gu = 0, n_dn = 0, wbits = 16;
+    uint32_t per_gu = 8, per_dn = 4, parts_gu = 0, parts_dn = 0, ks_gu = 1, ks_dn = 1, bt_gu = 8, bt_dn = 8;
+    int codebook = 0, dtype = 0, score_dt = 0, defer = 0;
+    float limit = 0.0f;
+};
+
+// prepare_apart: five launches (prepare, gate|up, mid, down, combine); else four (each gate|up wave prepares its own
+// 128-block in LDS). The same bytes.
+hipError_t launch_moe_decode(const MoeLaunch& a, bool prepare_apart, hipStream_t s);
+
 // trellis [in/16][out/16][n] -> W_hat f16 [in][out], bit-exact (format.reconstructInner)
 hipError_t launch_dequant(const uint32_t* trellis, uint16_t* w_hat, uint32_t in, uint32_t out, uint32_t n,
                           uint32_t wbits, int codebook, hipStream_t s);

@@ -1,26 +1,215 @@
-// Routed experts: `moe`, `moeClamped`, `moeWithShared` (turboexl3 src/root.zig:822-904,976-1004).
+// Routed experts: `moe`, `moeClamped`, `moeWithShared` (turboexl3 src/root.zig:822-904,976-1004) and the fused
+// shared-expert form, over the decode-row chain of t3_moe.hip.
 
 #include "t3_host.hpp"
 
+namespace t3 {
+namespace {
+
+struct MoeCall {
+    MoeLaunch launch;
+    size_t workspace = 0;
+    int64_t rows = 0;
+};
+
+// One projection's arrays against the geometry (src/root.zig:87-102).
+int32_t check_proj(const t3_proj& p, int64_t experts, int64_t in, int64_t out, int64_t* n) {
+    if (!array_ok(&p.trellis) || !array_ok(&p.suh) || !array_ok(&p.svh)) return T3_BadArgs;
+    const t3_array& t = p.trellis;
+    if (in <= 0 || out <= 0 || in % 128 != 0 || out % 128 != 0 || t.ndim != 4 || t.shape[0] != experts ||
+        t.shape[1] != in / 16 || t.shape[2] != out / 16 || !rate_ok(t.shape[3]) || p.suh.ndim != 2 ||
+        p.suh.shape[0] != experts || p.suh.shape[1] != in || p.svh.ndim != 2 || p.svh.shape[0] != experts ||
+        p.svh.shape[1] != out)
+        return T3_BadExl3Shape;
+    if ((t.dtype != T3_U16 && t.dtype != T3_I16) || p.suh.dtype != T3_F16 || p.svh.dtype != T3_F16) return T3_BadExl3Dtype;
+    *n = t.shape[3];
+    return T3_OK;
+}
+
+// root.bankGeometry (src/root.zig:104-126): every projection validated; gate and up share a rate.
+int32_t check_bank(const t3_bank* bank, int64_t hidden, RoutedBank* out, int64_t* inter, int64_t* n_gu, int64_t* n_dn) {
+    if (!bank || !array_ok(&bank->gate.trellis)) return T3_BadArgs;
+    const t3_array& g = bank->gate.trellis;
+    if (g.ndim != 4 || g.shape[0] <= 0 || g.shape[2] <= 0 || g.shape[2] > (1 << 26)) return T3_BadExl3Shape;
+    const int64_t experts = g.shape[0], width = g.shape[2] * 16;
+    int64_t ng = 0, nu = 0, nd = 0;
+    if (const int32_t st = check_proj(bank->gate, experts, hidden, width, &ng); st != T3_OK) return st;
+    if (const int32_t st = check_proj(bank->up, experts, hidden, width, &nu); st != T3_OK) return st;
+    if (const int32_t st = check_proj(bank->down, experts, width, hidden, &nd); st != T3_OK) return st;
+    if (nu != ng) return T3_Exl3GateUpRateMismatch;
+    // one expert's matrix is addressed through 32-bit byte offsets
+    if ((hidden / 16) * (width / 16) * (ng > nd ? ng : nd) * 2 >= (1ll << 31)) return T3_Exl3EngineNotImplemented;
+    out->gate_t = static_cast<const uint32_t*>(bank->gate.trellis.data);
+    out->up_t = static_cast<const uint32_t*>(bank->up.trellis.data);
+    out->down_t = static_cast<const uint32_t*>(bank->down.trellis.data);
+    out->gate_suh = static_cast<const uint16_t*>(bank->gate.suh.data);
+    out->up_suh = static_cast<const uint16_t*>(bank->up.suh.data);
+    out->down_suh = static_cast<const uint16_t*>(bank->down.suh.data);
+    out->gate_svh = static_cast<const uint16_t*>(bank->gate.svh.data);
+    out->up_svh = static_cast<const uint16_t*>(bank->up.svh.data);
+    out->down_svh = static_cast<const uint16_t*>(bank->down.svh.data);
+    out->experts = static_cast<uint32_t>(experts);
+    *inter = width;
+    *n_gu = ng;
+    *n_dn = nd;
+    return T3_OK;
+}
+
+// root.validateCall (src/root.zig:128-141) and the partition of the decode chain.
+int32_t check_moe(const t3_array* x, const t3_bank* bank, const t3_array* inds, const t3_array* scores,
+                  const t3_bank* shared_bank, const t3_array* shared_add, t3_decode dec, int32_t limit,
+                  const t3_array* y, MoeCall* call) {
+    if (!array_ok(x) || !array_ok(inds) || (scores && !array_ok(scores)) || (y && !array_ok(y)) ||
+        (shared_add && !array_ok(shared_add)))
+        return T3_BadArgs;
+    if (x->ndim != 3 || inds->ndim != 3 || x->shape[0] <= 0 || x->shape[1] <= 0 || x->shape[0] != inds->shape[0] ||
+        x->shape[1] != inds->shape[1] || inds->shape[2] <= 0 || inds->shape[2] > T3_REDUCE_MAX_TOPK)
+        return T3_BadExl3Shape;
+    if (x->shape[2] <= 0 || x->shape[2] % 128 != 0) return T3_BadExl3Shape;
+    if (scores) {
+        if (scores->ndim != 3) return T3_BadExl3Shape;
+        for (int i = 0; i < 3; ++i)
+            if (scores->shape[i] != inds->shape[i]) return T3_BadExl3Shape;
+        if (!is_act_dtype(scores->dtype)) return T3_BadExl3Dtype;
+    }
+    if (!is_act_dtype(x->dtype) || (inds->dtype != T3_U32 && inds->dtype != T3_I32)) return T3_BadExl3Dtype;
+    const int64_t rows = x->shape[0] * x->shape[1], topk = inds->shape[2], hidden = x->shape[2];
+    if (rows > (1ll << 24) || rows * topk > (1ll << 28)) return T3_BadExl3Shape;
+    MoeLaunch& l = call->launch;
+    int64_t inter = 0, n_gu = 0, n_dn = 0;
+    if (const int32_t st = check_bank(bank, hidden, &l.bank, &inter, &n_gu, &n_dn); st != T3_OK) return st;
+    if (shared_bank) {
+        int64_t s_inter = 0, s_gu = 0, s_dn = 0;
+        if (const int32_t st = check_bank(shared_bank, hidden, &l.shared, &s_inter, &s_gu, &s_dn); st != T3_OK) return st;
+        // the shared slots ride the routed launches: the same widths and rates
+        if (s_inter != inter || s_gu != n_gu || s_dn != n_dn) return T3_Exl3EngineNotImplemented;
+        if (topk + l.shared.experts > 64) return T3_BadExl3Shape;
+        l.shared_slots = l.shared.experts;
+    }
+    if (shared_add) {
+        if (shared_add->dtype != x->dtype) return T3_BadExl3Shape;  // src/root.zig:977
+        int64_t count = 1;
+        for (int i = 0; i < shared_add->ndim; ++i) count *= shared_add->shape[i];
+        if (count != rows * hidden) return T3_BadExl3Shape;
+    }
+    if (y) {
+        if (y->ndim != 3 || y->shape[0] != x->shape[0] || y->shape[1] != x->shape[1] || y->shape[2] != hidden)
+            return T3_BadExl3Shape;
+        if (y->dtype != x->dtype) return T3_BadExl3Dtype;
+    }
+    Dec d;
+    if (const int32_t st = resolve_decode(dec, &d); st != T3_OK) return st;
+    if (limit < 0 || limit > 128) return T3_InvalidExl3Clamp;
+    call->rows = rows;
+    l.x = x->data;
+    l.slots = static_cast<const int32_t*>(inds->data);
+    l.scores = scores ? scores->data : nullptr;
+    l.score_dt = scores ? scores->dtype : T3_F32;
+    l.shared_add = shared_add ? shared_add->data : nullptr;
+    l.y = y ? y->data : nullptr;
+    l.hidden = static_cast<uint32_t>(hidden);
+    l.inter = static_cast<uint32_t>(inter);
+    l.rows = static_cast<uint32_t>(rows);
+    l.topk = static_cast<uint32_t>(topk);
+    l.n_gu = static_cast<uint32_t>(n_gu);
+    l.n_dn = static_cast<uint32_t>(n_dn);
+    l.wbits = d.wbits;
+    l.codebook = d.gemv_form;
+    l.defer = d.gemv_form == 2;
+    l.dtype = x->dtype;
+    l.limit = static_cast<float>(limit);
+    // Partitions: functions of the bank's shapes alone. gate|up: a part is one 128-block of the input (8 tiles), so a
+    // wave can prepare its own block; down: 4 tiles a part, its input being prepared by the mid launch.
+    l.bt_gu = gemv_bt(l.n_gu);
+    l.bt_dn = gemv_bt(l.n_dn);
+    l.per_gu = 8;
+    l.parts_gu = (l.hidden / 16u) / l.per_gu;
+    l.ks_gu = (l.parts_gu + 3u) / 4u;
+    l.per_dn = 4;
+    l.parts_dn = (l.inter / 16u) / l.per_dn;
+    l.ks_dn = (l.parts_dn + 3u) / 4u;
+    return T3_OK;
+}
+
+void carve_moe(MoeCall* call, void* workspace) {
+    MoeLaunch& l = call->launch;
+    const size_t rkt = static_cast<size_t>(l.rows) * (l.topk + l.shared_slots);
+    Carver c(workspace);
+    c.take<uint32_t>(kCounterBytes);
+    l.xg = c.take<uint32_t>(rkt * l.hidden * 4u);
+    l.xu = c.take<uint32_t>(rkt * l.hidden * 4u);
+    l.hd = c.take<uint32_t>(rkt * l.inter * 4u);
+    l.sg = c.take<float>(rkt * (l.hidden / 128u) * 4u);
+    l.su = c.take<float>(rkt * (l.hidden / 128u) * 4u);
+    l.hs = c.take<float>(rkt * (l.inter / 128u) * 4u);
+    l.zg = c.take<float>(static_cast<size_t>(l.ks_gu) * rkt * l.inter * 4u);
+    l.zu = c.take<float>(static_cast<size_t>(l.ks_gu) * rkt * l.inter * 4u);
+    l.zd = c.take<float>(static_cast<size_t>(l.ks_dn) * rkt * l.hidden * 4u);
+    call->workspace = c.used;
+}
+
+int32_t run_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
+                const t3_array* scores, const t3_bank* shared_bank, const t3_array* shared_add, t3_decode dec,
+                int32_t limit, t3_array* y, void* workspace, size_t workspace_bytes) {
+    if (!scores || !y) return T3_BadArgs;
+    MoeCall call;
+    if (const int32_t st = check_moe(x, bank, inds, scores, shared_bank, shared_add, dec, limit, y, &call); st != T3_OK)
+        return st;
+    // rows above the decode chain's take the prefill GEMM chain (src/root.zig:850-853)
+    if (call.rows > T3_DECODE_ROWS_MAX) return T3_Exl3EngineNotImplemented;
+    if (!workspace) return T3_BadArgs;
+    carve_moe(&call, workspace);
+    if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
+    const bool prepare_apart = config().decode_form == 3;
+    return hip_status(launch_moe_decode(call.launch, prepare_apart, static_cast<hipStream_t>(stream)));
+}
+
+}  // namespace
+}  // namespace t3
+
 extern "C" {
 
-int32_t t3_moe_workspace_bytes(const t3_array*, const t3_bank*, const t3_array*, size_t*) {
-    return T3_Exl3EngineNotImplemented;
+int32_t t3_moe_workspace_bytes(const t3_array* x, const t3_bank* bank, const t3_array* inds,
+                               const t3_bank* shared_bank, size_t* bytes) {
+    if (!bytes) return T3_BadArgs;
+    t3::MoeCall call;
+    const t3_decode dec = {0, 16};
+    if (const int32_t st = t3::check_moe(x, bank, inds, nullptr, shared_bank, nullptr, dec, 0, nullptr, &call);
+        st != T3_OK)
+        return st;
+    if (call.rows > T3_DECODE_ROWS_MAX) return T3_Exl3EngineNotImplemented;
+    t3::carve_moe(&call, nullptr);
+    *bytes = call.workspace;
+    return T3_OK;
 }
 
-int32_t t3_moe(t3_stream, const t3_array*, const t3_bank*, const t3_array*, const t3_array*, t3_decode, int32_t,
-               t3_array*, void*, size_t) {
-    return T3_Exl3EngineNotImplemented;
+int32_t t3_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
+               const t3_array* scores, t3_decode dec, int32_t verify_rows, t3_array* y, void* workspace,
+               size_t workspace_bytes) {
+    (void)verify_rows;
+    return t3::run_moe(stream, x, bank, inds, scores, nullptr, nullptr, dec, 0, y, workspace, workspace_bytes);
 }
 
-int32_t t3_moe_clamped(t3_stream, const t3_array*, const t3_bank*, const t3_array*, const t3_array*, t3_decode,
-                       int32_t, t3_array*, void*, size_t) {
-    return T3_Exl3EngineNotImplemented;
+int32_t t3_moe_clamped(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
+                       const t3_array* scores, t3_decode dec, int32_t limit, t3_array* y, void* workspace,
+                       size_t workspace_bytes) {
+    if (limit <= 0 || limit > 128) return T3_InvalidExl3Clamp;
+    return t3::run_moe(stream, x, bank, inds, scores, nullptr, nullptr, dec, limit, y, workspace, workspace_bytes);
 }
 
-int32_t t3_moe_with_shared(t3_stream, const t3_array*, const t3_bank*, const t3_array*, const t3_array*, t3_decode,
-                           int32_t, const t3_array*, t3_array*, void*, size_t) {
-    return T3_Exl3EngineNotImplemented;
+int32_t t3_moe_with_shared(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
+                           const t3_array* scores, t3_decode dec, int32_t verify_rows, const t3_array* shared,
+                           t3_array* y, void* workspace, size_t workspace_bytes) {
+    (void)verify_rows;
+    if (!shared) return T3_BadArgs;
+    return t3::run_moe(stream, x, bank, inds, scores, nullptr, shared, dec, 0, y, workspace, workspace_bytes);
+}
+
+int32_t t3_moe_shared_expert(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
+                             const t3_array* scores, t3_decode dec, int32_t limit, const t3_bank* shared_bank,
+                             t3_array* y, void* workspace, size_t workspace_bytes) {
+    if (!shared_bank) return T3_BadArgs;
+    return t3::run_moe(stream, x, bank, inds, scores, shared_bank, nullptr, dec, limit, y, workspace, workspace_bytes);
 }
 
 }  // extern "C"

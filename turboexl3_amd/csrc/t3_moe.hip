@@ -1,0 +1,301 @@
+// Routed experts at decode rows on gfx950: the split-K GEMV chain over gathered top-k experts, no decoded weight
+// written anywhere (turboexl3 src/core/decode.zig:274-517 form 3 / form 9; roles of src/hip/plan.zig:294-364).
+//
+// Per routed pair ("row-slot") rk = row * KT + k, expert e (profile "exl3": format.project's rounding points, the
+// reference's src/core/ref.zig:154-190):
+//   prepare   xg, xu = f16(H128(f16(x) * suh_e) / sqrt(128)) with the gate's and the up's own suh;
+//   gate|up   zg, zu = xg * Wg_e, xu * Wu_e, split over K parts, planes summed in part order;
+//   mid       g, u = finish(zg), finish(zu) -> clamp (gate from above, up both ways) -> h = f16(silu(g) * u)
+//             -> the down's prepare of h with down_suh_e;
+//   down      zd = hd * Wd_e;
+//   combine   per row: acc = fma(score_k, finish(zd_k), acc) in slot order, then y's dtype.
+// A shared expert rides the same launches as slots K..KT-1 of every row, read from its own bank at weight 1.
+// One wave serves one row-slot's K part with the dense path's streaming core; the matrix core runs one live row of 16.
+// Launch forms: five launches (prepare apart) or four (each gate|up wave prepares its own 128-block in LDS): the same
+// statements in the same order, so the same bytes.
+
+#include "t3_gemv_core.hpp"
+#include "t3_kernels.hpp"
+#include "t3_stages.hpp"
+
+namespace t3 {
+namespace {
+
+struct SlotRef {
+    uint32_t row, e;
+    bool live, shared;
+};
+
+// Row-slot rk of KT = topk + shared slots a row. A routed id outside [0, experts) is skipped, as the reference skips it
+// (src/kernels/hip/decode/decode.hip:26-28).
+__device__ __forceinline__ SlotRef resolve_slot(const MoeLaunch& a, uint32_t rk) {
+    SlotRef s;
+    const uint32_t kt = a.topk + a.shared_slots;
+    s.row = rk / kt;
+    const uint32_t k = rk - s.row * kt;
+    s.shared = k >= a.topk;
+    if (s.shared) {
+        s.e = k - a.topk;
+        s.live = true;
+    } else {
+        const int32_t es = a.slots[s.row * a.topk + k];
+        s.live = es >= 0 && static_cast<uint32_t>(es) < a.bank.experts;
+        s.e = static_cast<uint32_t>(es);
+    }
+    return s;
+}
+
+__device__ __forceinline__ float score_of(const MoeLaunch& a, uint32_t row, uint32_t k) {
+    const size_t i = static_cast<size_t>(row) * a.topk + k;
+    if (a.score_dt == kF32) return static_cast<const float*>(a.scores)[i];
+    if (a.score_dt == kF16) return half_value(static_cast<const uint16_t*>(a.scores)[i]);
+    return bf16_value(static_cast<const uint16_t*>(a.scores)[i]);
+}
+
+// Grid (hidden / 128, RKT), 64 threads: the five-launch form's prepare. xg, xu: u32 [RKT][hidden] (quad order, doubled);
+// sg, su: f32 [RKT][hidden / 128].
+__global__ void __launch_bounds__(64) moe_prep(const MoeLaunch a) {
+    const uint32_t b = blockIdx.x, rk = blockIdx.y, lane = threadIdx.x;
+    const SlotRef s = resolve_slot(a, rk);
+    if (!s.live) return;
+    const RoutedBank& bank = s.shared ? a.shared : a.bank;
+    const uint32_t nb = a.hidden / 128u;
+#pragma unroll
+    for (uint32_t proj = 0; proj < 2u; ++proj) {
+        const uint16_t* suh = (proj ? bank.up_suh : bank.gate_suh) + static_cast<size_t>(s.e) * a.hidden;
+        uint32_t hv[2];
+        float sum;
+        prep_values(a.dtype, a.x, suh, a.hidden, s.row, b, lane, hv, sum);
+        uint32_t* xq = proj ? a.xu : a.xg;
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j) {
+            const uint32_t i = b * 128u + lane + 64u * j;
+            xq[static_cast<size_t>(rk) * a.hidden + (i & ~15u) + quad_slot(i & 15u)] = hv[j] | (hv[j] << 16);
+        }
+        if (lane == 0u) (proj ? a.su : a.sg)[static_cast<size_t>(rk) * nb + b] = sum;
+    }
+}
+
+// Grid (out / 16 / BT, RKT * NPROJ, KS), 256 threads. NPROJ 2: gate (proj 0) and up (proj 1), hidden -> inter;
+// NPROJ 1: down, inter -> hidden. Wave sg of slice blockIdx.z takes K part 4 z + sg of `parts` (a part: `per` input
+// tiles). z[proj]: f32 [KS][RKT][out], the four waves' sums, wave 0 first. XLDS (gate|up only, per == 8): the wave
+// prepares its own 128-block of x in LDS.
+template <int CB, bool WIDE, int BT, int NPROJ, bool XLDS>
+__global__ void __launch_bounds__(256) moe_gemv(const MoeLaunch a) {
+    constexpr int ST = 2;
+    constexpr uint32_t kStage = gemv_stage_bytes<BT>();
+    constexpr uint32_t kRed = 4u * BT * 64u * 16u;
+    constexpr uint32_t kMain = kRed > 4u * kStage ? kRed : 4u * kStage;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[kMain];
+    float4v(*red)[BT * 64] = reinterpret_cast<float4v(*)[BT * 64]>(smem);
+    const uint32_t blk = blockIdx.x, rk = blockIdx.y / NPROJ, proj = blockIdx.y % NPROJ, ksl = blockIdx.z;
+    const uint32_t sg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
+    const SlotRef s = resolve_slot(a, rk);
+    if (!s.live) return;  // uniform over the workgroup
+    const RoutedBank& bank = s.shared ? a.shared : a.bank;
+    const uint32_t in = NPROJ == 2 ? a.hidden : a.inter, out = NPROJ == 2 ? a.inter : a.hidden;
+    const uint32_t n = NPROJ == 2 ? a.n_gu : a.n_dn;
+    const uint32_t per = NPROJ == 2 ? a.per_gu : a.per_dn, parts = NPROJ == 2 ? a.parts_gu : a.parts_dn;
+    const uint32_t in_tiles = in >> 4, out_tiles = out >> 4, nw = n >> 1;
+    const uint32_t* wmat = (NPROJ == 1 ? bank.down_t : (proj ? bank.up_t : bank.gate_t)) +
+                           static_cast<size_t>(s.e) * in_tiles * out_tiles * nw;
+    const uint32_t part = ksl * 4u + sg;
+    const uint32_t tk0 = part * per;
+    const uint64_t wstride = static_cast<uint64_t>(out_tiles) * nw;
+    const uint32_t* wbase = wmat + static_cast<uint64_t>(blk) * BT * nw + tk0 * wstride;
+    const uint32_t wstep = static_cast<uint32_t>(wstride) * 4u;
+    const uint32_t rkt = a.rows * (a.topk + a.shared_slots);
+
+    float4v acc[1][BT];
+#pragma unroll
+    for (int t = 0; t < BT; ++t) acc[0][t] = float4v{0.f, 0.f, 0.f, 0.f};
+
+    if (part < parts) {  // uniform over the wave; a wave past the last part adds zeros below
+        uint32_t xoff[1];
+        if constexpr (XLDS) {
+            extern __shared__ __attribute__((aligned(16))) unsigned char xdyn[];
+            unsigned char* xst = xdyn + sg * ((per + 1u) * (kXldsRows * 64u));
+            xoff[0] = (lane >> 4) * 16u;  // every activation row of the fragment is the slot's one row
+            GemvStream<CB, WIDE, 1, BT, ST, XLds> stream(wbase, wstep, per, n, a.wbits, XLds{xst}, xoff,
+                                                         smem + sg * kStage, lane);
+            stream.issue();
+            const uint16_t* suh = (proj ? bank.up_suh : bank.gate_suh) + static_cast<size_t>(s.e) * a.hidden;
+            const uint32_t blocks = per >> 3;
+            for (uint32_t b = 0; b < blocks; ++b) {
+                uint32_t hv[2];
+                float sum;
+                prep_values(a.dtype, a.x, suh, a.hidden, s.row, (tk0 >> 3) + b, lane, hv, sum);
+#pragma unroll
+                for (uint32_t j = 0; j < 2u; ++j) {
+                    const uint32_t i = lane + 64u * j;
+                    const uint32_t at = ((b * 8u + (i >> 4)) * kXldsRows) * 64u + quad_slot(i & 15u) * 4u;
+                    *reinterpret_cast<uint32_t*>(xst + at) = hv[j] | (hv[j] << 16);
+                }
+                // every column workgroup of the slot stores the same sum: a handful of plain stores, read by the
+                // next launch
+                if (a.defer && lane == 0u)
+                    (proj ? a.su : a.sg)[static_cast<size_t>(rk) * (a.hidden / 128u) + (tk0 >> 3) + b] = sum;
+            }
+            for (uint32_t i = lane; i < kXldsRows * 16u; i += 64u)
+                *reinterpret_cast<uint32_t*>(xst + per * (kXldsRows * 64u) + i * 4u) = 0u;
+            stream.run(acc);
+        } else {
+            const uint32_t* xq = NPROJ == 1 ? a.hd : (proj ? a.xu : a.xg);
+            xoff[0] = (rk * in + 4u * (lane >> 4)) * 4u;
+            GemvStream<CB, WIDE, 1, BT, ST, XGlobal> stream(
+                wbase, wstep, per, n, a.wbits, XGlobal{xq, static_cast<uint64_t>(rkt) * in * 4u, tk0 * 64u}, xoff,
+                smem + sg * kStage, lane);
+            stream.issue();
+            stream.run(acc);
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < BT; ++t) red[sg][t * 64 + lane] = acc[0][t];
+    __syncthreads();
+    // activation row 0 of the fragment is the slot's row: lanes with lane % 16 == 0 hold its sums
+    float* z = NPROJ == 1 ? a.zd : (proj ? a.zu : a.zg);
+    for (uint32_t i = threadIdx.x; i < static_cast<uint32_t>(BT * 64); i += 256u) {
+        const uint32_t l = i & 63u, t = i >> 6;
+        if ((l & 15u) != 0u) continue;
+        const float4v v = ((red[0][i] + red[1][i]) + red[2][i]) + red[3][i];
+        float* dst = z + (static_cast<size_t>(ksl) * rkt + rk) * out + (blk * BT + t) * 16u + 4u * (l >> 4);
+        *reinterpret_cast<float4v*>(dst) = v;
+    }
+}
+
+// One block's sums over the K slices (slice order; the first plane starts the sum) and the deferred MUL1 map.
+__device__ __forceinline__ void plane_sums(const float* z, size_t planes_stride, uint32_t ks, const float* bsum,
+                                           uint32_t nb, int defer, uint32_t lane, float (&s)[2]) {
+#pragma unroll
+    for (uint32_t j = 0; j < 2u; ++j) s[j] = z[lane + 64u * j];
+    for (uint32_t k = 1; k < ks; ++k)
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j) s[j] += z[k * planes_stride + lane + 64u * j];
+    if (defer) {
+        float xsum = 0.0f;
+        for (uint32_t q = 0; q < nb; ++q) xsum += bsum[q];
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j) s[j] = __builtin_fmaf(s[j], mul1_a(), mul1_b() * xsum);
+    }
+}
+
+// Grid (inter / 128, RKT), 64 threads: gate and up finishes, the (clamped) SwiGLU in f32 on their f16 values, and the
+// down's prepare: hd u32 [RKT][inter] (quad order, doubled), hs f32 [RKT][inter / 128].
+__global__ void __launch_bounds__(64) moe_mid(const MoeLaunch a) {
+    const uint32_t b = blockIdx.x, rk = blockIdx.y, lane = threadIdx.x;
+    const SlotRef s = resolve_slot(a, rk);
+    if (!s.live) return;
+    const RoutedBank& bank = s.shared ? a.shared : a.bank;
+    const uint32_t rkt = a.rows * (a.topk + a.shared_slots), nb = a.hidden / 128u;
+    const size_t plane = static_cast<size_t>(rkt) * a.inter, at = static_cast<size_t>(rk) * a.inter + b * 128u;
+    float g[2], u[2];
+    plane_sums(a.zg + at, plane, a.ks_gu, a.sg + static_cast<size_t>(rk) * nb, nb, a.defer, lane, g);
+    plane_sums(a.zu + at, plane, a.ks_gu, a.su + static_cast<size_t>(rk) * nb, nb, a.defer, lane, u);
+    finish_values(g, bank.gate_svh + static_cast<size_t>(s.e) * a.inter, b, lane);
+    finish_values(u, bank.up_svh + static_cast<size_t>(s.e) * a.inter, b, lane);
+    float d[2];
+#pragma unroll
+    for (uint32_t j = 0; j < 2u; ++j) {
+        float gv = g[j], uv = u[j];
+        if (a.limit > 0.0f) {  // comparisons: a NaN passes through (ref.zig:132-140)
+            gv = gv > a.limit ? a.limit : gv;
+            uv = uv > a.limit ? a.limit : (uv < -a.limit ? -a.limit : uv);
+        }
+        const float hv = round_half((gv / (1.0f + expf(-gv))) * uv);
+        d[j] = hv * half_value(bank.down_suh[static_cast<size_t>(s.e) * a.inter + b * 128u + lane + 64u * j]);
+    }
+    h128_wave(d, lane);
+    float sum = 0.0f;
+#pragma unroll
+    for (uint32_t j = 0; j < 2u; ++j) {
+        const uint32_t i = b * 128u + lane + 64u * j;
+        const uint32_t hh = half_bits(d[j] * kHadScale);
+        a.hd[static_cast<size_t>(rk) * a.inter + (i & ~15u) + quad_slot(i & 15u)] = hh | (hh << 16);
+        sum += half_value(hh);
+    }
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) sum += __shfl_xor(sum, m, 64);
+    if (lane == 0u) a.hs[static_cast<size_t>(rk) * (a.inter / 128u) + b] = sum;
+}
+
+// Grid (hidden / 128, rows), 64 threads: every slot's down finish, then the score-weighted sum in slot order.
+__global__ void __launch_bounds__(64) moe_combine(const MoeLaunch a) {
+    const uint32_t b = blockIdx.x, row = blockIdx.y, lane = threadIdx.x;
+    const uint32_t kt = a.topk + a.shared_slots, rkt = a.rows * kt, nbi = a.inter / 128u;
+    const size_t plane = static_cast<size_t>(rkt) * a.hidden;
+    float acc[2] = {0.0f, 0.0f};
+    for (uint32_t k = 0; k < kt; ++k) {
+        const uint32_t rk = row * kt + k;
+        const SlotRef s = resolve_slot(a, rk);
+        if (!s.live) continue;  // uniform over the wave
+        const RoutedBank& bank = s.shared ? a.shared : a.bank;
+        float v[2];
+        plane_sums(a.zd + static_cast<size_t>(rk) * a.hidden + b * 128u, plane, a.ks_dn,
+                   a.hs + static_cast<size_t>(rk) * nbi, nbi, a.defer, lane, v);
+        finish_values(v, bank.down_svh + static_cast<size_t>(s.e) * a.hidden, b, lane);
+        const float w = s.shared ? 1.0f : score_of(a, row, k);
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j) acc[j] = __builtin_fmaf(w, v[j], acc[j]);
+    }
+#pragma unroll
+    for (uint32_t j = 0; j < 2u; ++j) {
+        const size_t o = static_cast<size_t>(row) * a.hidden + b * 128u + lane + 64u * j;
+        if (a.shared_add) {
+            // `moeWithShared`: the routed output rounds to x's dtype, then the add rounds again (src/root.zig:976-984)
+            float r = acc[j];
+            if (a.dtype == kF16) r = round_half(r);
+            else if (a.dtype == kBf16) r = bf16_value(bf16_bits(r));
+            store_act_rt(a.dtype, a.y, o, r + load_act_rt(a.dtype, a.shared_add, o));
+        } else {
+            store_act_rt(a.dtype, a.y, o, acc[j]);
+        }
+    }
+}
+
+template <int CB, bool WIDE, int NPROJ, bool XLDS>
+hipError_t launch_gemv_bt(const MoeLaunch& a, hipStream_t s) {
+    const uint32_t out = NPROJ == 2 ? a.inter : a.hidden;
+    const uint32_t bt = NPROJ == 2 ? a.bt_gu : a.bt_dn, ks = NPROJ == 2 ? a.ks_gu : a.ks_dn;
+    const uint32_t rkt = a.rows * (a.topk + a.shared_slots);
+    const dim3 grid((out / 16u) / bt, rkt * NPROJ, ks), block(256);
+    const size_t dyn = XLDS ? 4u * (a.per_gu + 1u) * (kXldsRows * 64u) : 0u;
+    if (bt == 8u) hipLaunchKernelGGL((moe_gemv<CB, WIDE, 8, NPROJ, XLDS>), grid, block, dyn, s, a);
+    else hipLaunchKernelGGL((moe_gemv<CB, WIDE, 4, NPROJ, XLDS>), grid, block, dyn, s, a);
+    return hipGetLastError();
+}
+
+template <int NPROJ, bool XLDS>
+hipError_t launch_gemv_cb(const MoeLaunch& a, hipStream_t s) {
+    const bool wide = quad_needs_wide(NPROJ == 2 ? a.n_gu : a.n_dn);
+    switch (a.codebook) {
+        case kMul1: return wide ? launch_gemv_bt<kMul1, true, NPROJ, XLDS>(a, s) : launch_gemv_bt<kMul1, false, NPROJ, XLDS>(a, s);
+        case kMcg: return wide ? launch_gemv_bt<kMcg, true, NPROJ, XLDS>(a, s) : launch_gemv_bt<kMcg, false, NPROJ, XLDS>(a, s);
+        case kMul1Defer:
+            return wide ? launch_gemv_bt<kMul1Defer, true, NPROJ, XLDS>(a, s)
+                        : launch_gemv_bt<kMul1Defer, false, NPROJ, XLDS>(a, s);
+        default:
+            return wide ? launch_gemv_bt<kMcgPair, true, NPROJ, XLDS>(a, s) : launch_gemv_bt<kMcgPair, false, NPROJ, XLDS>(a, s);
+    }
+}
+
+}  // namespace
+
+hipError_t launch_moe_decode(const MoeLaunch& a, bool prepare_apart, hipStream_t s) {
+    const uint32_t rkt = a.rows * (a.topk + a.shared_slots);
+    hipError_t e;
+    if (prepare_apart) {
+        hipLaunchKernelGGL(moe_prep, dim3(a.hidden / 128u, rkt), dim3(64), 0, s, a);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        if ((e = launch_gemv_cb<2, false>(a, s)) != hipSuccess) return e;
+    } else {
+        if ((e = launch_gemv_cb<2, true>(a, s)) != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(moe_mid, dim3(a.inter / 128u, rkt), dim3(64), 0, s, a);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+    if ((e = launch_gemv_cb<1, false>(a, s)) != hipSuccess) return e;
+    hipLaunchKernelGGL(moe_combine, dim3(a.hidden / 128u, a.rows), dim3(64), 0, s, a);
+    return hipGetLastError();
+}
+
+}  // namespace t3
