@@ -115,6 +115,72 @@ class DenseRunner:
         return e0.elapsed_time(e1) * 1e-3 / steps
 
 
+class MoeRunner:
+    """BASELINE config 3: 512 experts, hidden 2048, inter 512, K3, top-10, clamp 7, one shared expert (inter 512) in the
+    same launches. Every call routes to a fresh set of experts (a rotation of disjoint routings) so the codes come from
+    HBM: the bank alone is 604 MB."""
+
+    E, HIDDEN, INTER, K, TOPK, LIMIT = 512, 2048, 512, 3, 10, 7
+
+    def __init__(self, torch, api, tokens: int, seed: int = 5):
+        import ctypes as C
+
+        from turboexl3_amd import _lib
+        self.C, self.L, self.torch, self.api = C, _lib.lib(), torch, api
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+        n = 16 * self.K
+
+        def proj(experts, in_f, out_f):
+            t = torch.randint(-32768, 32768, (experts, in_f // 16, out_f // 16, n), dtype=torch.int16, device="cuda",
+                              generator=g)
+            suh = (0.5 + torch.rand(experts, in_f, device="cuda", generator=g)).to(torch.float16)
+            svh = ((0.5 + torch.rand(experts, out_f, device="cuda", generator=g)) / in_f ** 0.5).to(torch.float16)
+            return api.Proj(t, suh, svh)
+
+        def bank(experts):
+            return api.Bank(proj(experts, self.HIDDEN, self.INTER), proj(experts, self.HIDDEN, self.INTER),
+                            proj(experts, self.INTER, self.HIDDEN))
+
+        self.bank, self.shared = bank(self.E), bank(1)
+        self.tokens = tokens
+        self.x = torch.randn(1, tokens, self.HIDDEN, device="cuda", generator=g).to(torch.bfloat16)
+        # router logits ~ N(0,1) -> top-k -> softmax over the selected (harness side, as in the reference's benches)
+        self.sets = 24
+        logits = torch.randn(self.sets, tokens, self.E, device="cuda", generator=g)
+        top = torch.topk(logits, self.TOPK, dim=-1)
+        self.inds = top.indices.to(torch.int32).contiguous()
+        self.scores = torch.softmax(top.values, dim=-1).to(torch.float32).contiguous()
+        self.cb, self._k1 = api._cbank(self.bank)
+        self.sb, self._k2 = api._cbank(self.shared)
+        self.ax = api._arr(self.x)
+        self.ai = [api._arr(self.inds[i:i + 1]) for i in range(self.sets)]
+        self.asc = [api._arr(self.scores[i:i + 1]) for i in range(self.sets)]
+        self.y = torch.empty_like(self.x)
+        self.ay = api._arr(self.y)
+        need = C.c_size_t(0)
+        st = self.L.t3_moe_workspace_bytes(C.byref(self.ax), C.byref(self.cb), C.byref(self.ai[0]), C.byref(self.sb),
+                                           C.byref(need))
+        assert st == 0, _lib.error_name(st)
+        self.ws = torch.zeros(need.value, dtype=torch.uint8, device="cuda")
+        self.dec = api.Decode.mcg.c()
+        self.stream = torch.cuda.current_stream().cuda_stream
+        per_expert = 3 * (self.HIDDEN // 16) * (self.INTER // 16) * n * 2
+        distinct = [len(set(self.inds[i].flatten().tolist())) for i in range(self.sets)]
+        self.code_bytes = (sum(distinct) / self.sets + 1) * per_expert  # + the shared expert
+
+    def call(self, i: int, stages: int = 0):
+        C = self.C
+        j = i % self.sets
+        st = self.L.t3_moe_shared_expert(self.stream, C.byref(self.ax), C.byref(self.cb), C.byref(self.ai[j]),
+                                         C.byref(self.asc[j]), self.dec, self.LIMIT, C.byref(self.sb), C.byref(self.ay),
+                                         self.ws.data_ptr(), self.ws.numel())
+        if st != 0:
+            raise RuntimeError(self.L.t3_error_name(st).decode())
+
+    time = DenseRunner.time
+
+
 def cpu_baseline(n: int, seed: int, budget_s: float = 20.0):
     """format.project (the C oracle) on the host: the same shape and seeded distributions, one row, one thread,
     re-decoding every tile as the reference does. A bounded sample: whole calls until ~budget_s is spent."""
@@ -154,6 +220,7 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--k", type=int, default=4)
     ap.add_argument("--rows", type=int, default=1)
+    ap.add_argument("--moe", action="store_true", help="also time the routed-expert decode chain (config 3)")
     ap.add_argument("--in-f", type=int, default=4096)
     ap.add_argument("--out-f", type=int, default=12288)
     args = ap.parse_args()
@@ -199,6 +266,14 @@ def main() -> int:
                      "frac": head["gemv_frac_of_hbm"], "traffic": None, "kernel": "t3::dense_gemv",
                      "us_per_launch": head["gemv_us"], "algorithmic_bytes_per_launch": head["code_bytes"]},
     }
+    if args.moe:
+        out["moe_decode"] = []
+        for tokens in (1, 8):
+            run = MoeRunner(torch, api, tokens)
+            t = run.time(max(50, args.steps // 2), 10)
+            out["moe_decode"].append({"tokens": tokens, "us_per_call": t * 1e6, "code_bytes": run.code_bytes,
+                                      "gbps": run.code_bytes / t / 1e9, "frac_of_hbm": run.code_bytes / t / HBM_PEAK})
+            del run
     if args.sweep:
         out["sweep"] = [measure(k, r, max(50, args.steps // 4), 10) for k in (3, 4, 5) for r in (1, 4, 16, 32)]
     if not args.no_cpu:
