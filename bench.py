@@ -29,6 +29,9 @@ sys.path.insert(0, ROOT)
 IN_F, OUT_F = 4096, 12288
 HBM_PEAK = 8.0e12
 MIN_ROTATION_BYTES = 512 << 20
+# HBM bytes one chain-GEMV launch moves, from the profiler's FETCH_SIZE and WRITE_SIZE counters scaled by a 256 MiB
+# copy (profiles/dense_gemv_in4096_out12288_k4_rows1.txt): keyed by (in, out, K, rows); other workloads report null
+MEASURED_TRAFFIC = {(4096, 12288, 4, 1): 25_762_406}
 
 
 def code_bytes(in_f: int, out_f: int, n: int) -> int:
@@ -221,6 +224,9 @@ def main() -> int:
     ap.add_argument("--k", type=int, default=4)
     ap.add_argument("--rows", type=int, default=1)
     ap.add_argument("--moe", action="store_true", help="also time the routed-expert decode chain (config 3)")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="also run one 256 MiB device copy, the known-size kernel that scales the profiler's "
+                         "FETCH_SIZE / WRITE_SIZE readings")
     ap.add_argument("--in-f", type=int, default=4096)
     ap.add_argument("--out-f", type=int, default=12288)
     args = ap.parse_args()
@@ -253,6 +259,12 @@ def main() -> int:
                 "call_gbps": cb / t_call / 1e9, "gemv_us": t_gemv * 1e6, "gemv_gbps": cb / t_gemv / 1e9,
                 "gemv_frac_of_hbm": cb / t_gemv / HBM_PEAK}
 
+    if args.traffic_probe:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     head = measure(args.k, args.rows, args.steps, args.warmup)
     out = {
         "metric": "EXL3 GEMV HBM GB/s (% of 8 TB/s) at decode rows; MoE prefill GEMM TFLOP/s",
@@ -263,7 +275,8 @@ def main() -> int:
                                f"f16 activations, {head['copies']} rotating weight copies",
                    "pct_of_8TBps": 100.0 * head["call_gbps"] * 1e9 / HBM_PEAK},
         "roofline": {"bound": "hbm", "achieved": head["gemv_gbps"], "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": head["gemv_frac_of_hbm"], "traffic": None, "kernel": "t3::dense_gemv",
+                     "frac": head["gemv_frac_of_hbm"],
+                     "traffic": MEASURED_TRAFFIC.get((IN_F, OUT_F, args.k, args.rows)), "kernel": "t3::dense_gemv",
                      "us_per_launch": head["gemv_us"], "algorithmic_bytes_per_launch": head["code_bytes"]},
     }
     if args.moe:
