@@ -71,11 +71,26 @@ struct MoeLaunch {
     uint32_t per_gu = 8, per_dn = 4, parts_gu = 0, parts_dn = 0, ks_gu = 1, ks_dn = 1, bt_gu = 8, bt_dn = 8;
     int codebook = 0, dtype = 0, score_dt = 0, defer = 0;
     float limit = 0.0f;
+    // prefill only (the route's roles, src/hip/plan.zig:40-45): row-slots sorted by expert. order [P] position ->
+    // row-slot, inv [P] row-slot -> position (~0: skipped), items [max_items] {expert, first position, rows, 0},
+    // counts [E + S + 4]: per-expert counts, then the item count and the placed total; cursor [E + S].
+    uint32_t* order = nullptr;
+    uint32_t* inv = nullptr;
+    uint32_t* items = nullptr;
+    uint32_t* counts = nullptr;
+    uint32_t* cursor = nullptr;
+    uint32_t max_items = 0, item_rows = 64;
 };
 
 // prepare_apart: five launches (prepare, gate|up, mid, down, combine); else four (each gate|up wave prepares its own
 // 128-block in LDS). The same bytes.
 hipError_t launch_moe_decode(const MoeLaunch& a, bool prepare_apart, hipStream_t s);
+
+// The same call above the decode rows: route, prepare, gate|up GEMM, mid, down GEMM, combine. xg, xu, hd hold plain f16
+// here (quad order), zg, zu, zd one plane each, all by sorted position.
+hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s);
+// One dense projection above 32 rows: prepare (f16, quad order), the trellis GEMM, finish. xq holds plain f16; ks = 1.
+hipError_t launch_dense_prefill(const DenseLaunch& d, hipStream_t s);
 
 // trellis [in/16][out/16][n] -> W_hat f16 [in][out], bit-exact (format.reconstructInner)
 hipError_t launch_dequant(const uint32_t* trellis, uint16_t* w_hat, uint32_t in, uint32_t out, uint32_t n,

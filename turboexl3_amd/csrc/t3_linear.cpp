@@ -77,6 +77,20 @@ void carve_dense(DenseCall* call, void* workspace) {
     call->workspace = c.used;
 }
 
+// Above 32 rows: xq plain f16 [rows][in], xs f32 [rows][in / 128], z one f32 plane [rows][out].
+void carve_dense_prefill(DenseCall* call, void* workspace) {
+    DenseLaunch& l = call->launch;
+    l.ks = 1;
+    Carver c(workspace);
+    l.arrive = c.take<uint32_t>(kCounterBytes);
+    l.xq = c.take<uint32_t>(static_cast<size_t>(l.rows) * l.in * 2u);
+    l.xs = c.take<float>(static_cast<size_t>(l.rows) * (l.in / 128u) * 4u);
+    l.z = c.take<float>(static_cast<size_t>(l.rows) * l.out * 4u);
+    call->workspace = c.used;
+}
+
+constexpr uint32_t kGemvRowsMax = 32;
+
 int32_t run_chain(const DenseCall& call, hipStream_t s, uint32_t stages) {
     if (stages & T3_STAGE_PREPARE)
         if (const int32_t st = hip_status(launch_dense_prep(call.launch, s)); st != T3_OK) return st;
@@ -107,8 +121,9 @@ extern "C" {
 int32_t t3_linear_workspace_bytes(const t3_array* x, const t3_array* trellis, t3_decode dec, size_t* bytes) {
     if (!bytes) return T3_BadArgs;
     t3::DenseCall call;
-    if (const int32_t st = t3::check_dense(x, trellis, nullptr, nullptr, dec, nullptr, 32, &call); st != T3_OK) return st;
-    t3::carve_dense(&call, nullptr);
+    if (const int32_t st = t3::check_dense(x, trellis, nullptr, nullptr, dec, nullptr, 0, &call); st != T3_OK) return st;
+    if (call.launch.rows > t3::kGemvRowsMax) t3::carve_dense_prefill(&call, nullptr);
+    else t3::carve_dense(&call, nullptr);
     *bytes = call.workspace;
     return T3_OK;
 }
@@ -136,8 +151,15 @@ int32_t t3_linear(t3_stream stream, const t3_array* x, const t3_array* trellis, 
                   const t3_array* svh, t3_decode dec, t3_array* y, void* workspace, size_t workspace_bytes) {
     if (!suh || !svh || !y) return T3_BadArgs;
     t3::DenseCall call;
-    if (const int32_t st = t3::check_dense(x, trellis, suh, svh, dec, y, 32, &call); st != T3_OK) return st;
+    if (const int32_t st = t3::check_dense(x, trellis, suh, svh, dec, y, 0, &call); st != T3_OK) return st;
     if (!workspace) return T3_BadArgs;
+    if (call.launch.rows > t3::kGemvRowsMax) {
+        if (!t3::config().prefill || call.launch.rows > 65535u) return T3_Exl3EngineNotImplemented;
+        // the trellis GEMM (the role of src/core/dense.zig:978-1034 and of dequant + matmul + finish, :909-922)
+        t3::carve_dense_prefill(&call, workspace);
+        if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
+        return t3::hip_status(t3::launch_dense_prefill(call.launch, static_cast<hipStream_t>(stream)));
+    }
     t3::carve_dense(&call, workspace);
     if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
     if (!t3::config().dec_one) return t3::run_chain(call, static_cast<hipStream_t>(stream), 7u);

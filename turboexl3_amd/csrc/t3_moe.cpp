@@ -148,6 +148,45 @@ void carve_moe(MoeCall* call, void* workspace) {
     call->workspace = c.used;
 }
 
+// Above the decode rows every buffer is indexed by sorted position, the prepared activations are plain f16 and each
+// projection has one plane; the route's arrays follow (src/hip/plan.zig:417-432 sizes the same roles).
+void carve_moe_prefill(MoeCall* call, void* workspace) {
+    MoeLaunch& l = call->launch;
+    const size_t p = static_cast<size_t>(l.rows) * (l.topk + l.shared_slots);
+    const size_t et = static_cast<size_t>(l.bank.experts) + l.shared_slots;
+    // items of 64 rows unless the experts see few rows each: a short item still pays its whole decode
+    l.item_rows = p / et <= 32u ? 32u : 64u;
+    l.max_items = static_cast<uint32_t>((p < et ? p : et) + p / l.item_rows);
+    Carver c(workspace);
+    c.take<uint32_t>(kCounterBytes);
+    l.xg = c.take<uint32_t>(p * l.hidden * 2u);
+    l.xu = c.take<uint32_t>(p * l.hidden * 2u);
+    l.hd = c.take<uint32_t>(p * l.inter * 2u);
+    l.sg = c.take<float>(p * (l.hidden / 128u) * 4u);
+    l.su = c.take<float>(p * (l.hidden / 128u) * 4u);
+    l.hs = c.take<float>(p * (l.inter / 128u) * 4u);
+    l.zg = c.take<float>(p * l.inter * 4u);
+    l.zu = c.take<float>(p * l.inter * 4u);
+    l.zd = c.take<float>(p * l.hidden * 4u);
+    l.order = c.take<uint32_t>(p * 4u);
+    l.inv = c.take<uint32_t>(p * 4u);
+    l.items = c.take<uint32_t>(static_cast<size_t>(l.max_items) * 16u);
+    l.counts = c.take<uint32_t>((et + 4u) * 4u);
+    l.cursor = c.take<uint32_t>(et * 4u);
+    call->workspace = c.used;
+}
+
+// the rows a routed call takes through the GEMM chain, or the refusal (src/root.zig:850-853)
+int32_t admit_prefill(const MoeCall& call) {
+    if (!config().prefill) return T3_Exl3EngineNotImplemented;
+    const MoeLaunch& l = call.launch;
+    const int64_t p = static_cast<int64_t>(l.rows) * (l.topk + l.shared_slots);
+    const int64_t widest = l.hidden > l.inter ? l.hidden : l.inter;
+    // the GEMM addresses a projection's prepared rows through 32-bit byte offsets
+    if (p * widest * 2 >= (1ll << 31)) return T3_Exl3EngineNotImplemented;
+    return T3_OK;
+}
+
 int32_t run_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
                 const t3_array* scores, const t3_bank* shared_bank, const t3_array* shared_add, t3_decode dec,
                 int32_t limit, t3_array* y, void* workspace, size_t workspace_bytes) {
@@ -155,9 +194,14 @@ int32_t run_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const 
     MoeCall call;
     if (const int32_t st = check_moe(x, bank, inds, scores, shared_bank, shared_add, dec, limit, y, &call); st != T3_OK)
         return st;
-    // rows above the decode chain's take the prefill GEMM chain (src/root.zig:850-853)
-    if (call.rows > T3_DECODE_ROWS_MAX) return T3_Exl3EngineNotImplemented;
     if (!workspace) return T3_BadArgs;
+    // rows above the decode chain's take the prefill GEMM chain (src/root.zig:850-853)
+    if (call.rows > T3_DECODE_ROWS_MAX) {
+        if (const int32_t st = admit_prefill(call); st != T3_OK) return st;
+        carve_moe_prefill(&call, workspace);
+        if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
+        return hip_status(launch_moe_prefill(call.launch, static_cast<hipStream_t>(stream)));
+    }
     carve_moe(&call, workspace);
     if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
     const bool prepare_apart = config().decode_form == 3;
@@ -177,8 +221,12 @@ int32_t t3_moe_workspace_bytes(const t3_array* x, const t3_bank* bank, const t3_
     if (const int32_t st = t3::check_moe(x, bank, inds, nullptr, shared_bank, nullptr, dec, 0, nullptr, &call);
         st != T3_OK)
         return st;
-    if (call.rows > T3_DECODE_ROWS_MAX) return T3_Exl3EngineNotImplemented;
-    t3::carve_moe(&call, nullptr);
+    if (call.rows > T3_DECODE_ROWS_MAX) {
+        if (const int32_t st = t3::admit_prefill(call); st != T3_OK) return st;
+        t3::carve_moe_prefill(&call, nullptr);
+    } else {
+        t3::carve_moe(&call, nullptr);
+    }
     *bytes = call.workspace;
     return T3_OK;
 }

@@ -16,64 +16,15 @@
 
 #include "t3_gemv_core.hpp"
 #include "t3_kernels.hpp"
+#include "t3_routed.hpp"
 #include "t3_stages.hpp"
 
 namespace t3 {
 namespace {
 
-struct SlotRef {
-    uint32_t row, e;
-    bool live, shared;
-};
-
-// Row-slot rk of KT = topk + shared slots a row. A routed id outside [0, experts) is skipped, as the reference skips it
-// (src/kernels/hip/decode/decode.hip:26-28).
-__device__ __forceinline__ SlotRef resolve_slot(const MoeLaunch& a, uint32_t rk) {
-    SlotRef s;
-    const uint32_t kt = a.topk + a.shared_slots;
-    s.row = rk / kt;
-    const uint32_t k = rk - s.row * kt;
-    s.shared = k >= a.topk;
-    if (s.shared) {
-        s.e = k - a.topk;
-        s.live = true;
-    } else {
-        const int32_t es = a.slots[s.row * a.topk + k];
-        s.live = es >= 0 && static_cast<uint32_t>(es) < a.bank.experts;
-        s.e = static_cast<uint32_t>(es);
-    }
-    return s;
-}
-
-__device__ __forceinline__ float score_of(const MoeLaunch& a, uint32_t row, uint32_t k) {
-    const size_t i = static_cast<size_t>(row) * a.topk + k;
-    if (a.score_dt == kF32) return static_cast<const float*>(a.scores)[i];
-    if (a.score_dt == kF16) return half_value(static_cast<const uint16_t*>(a.scores)[i]);
-    return bf16_value(static_cast<const uint16_t*>(a.scores)[i]);
-}
-
-// Grid (hidden / 128, RKT), 64 threads: the five-launch form's prepare. xg, xu: u32 [RKT][hidden] (quad order, doubled);
-// sg, su: f32 [RKT][hidden / 128].
+// Grid (hidden / 128, RKT), 64 threads: the five-launch form's prepare.
 __global__ void __launch_bounds__(64) moe_prep(const MoeLaunch a) {
-    const uint32_t b = blockIdx.x, rk = blockIdx.y, lane = threadIdx.x;
-    const SlotRef s = resolve_slot(a, rk);
-    if (!s.live) return;
-    const RoutedBank& bank = s.shared ? a.shared : a.bank;
-    const uint32_t nb = a.hidden / 128u;
-#pragma unroll
-    for (uint32_t proj = 0; proj < 2u; ++proj) {
-        const uint16_t* suh = (proj ? bank.up_suh : bank.gate_suh) + static_cast<size_t>(s.e) * a.hidden;
-        uint32_t hv[2];
-        float sum;
-        prep_values(a.dtype, a.x, suh, a.hidden, s.row, b, lane, hv, sum);
-        uint32_t* xq = proj ? a.xu : a.xg;
-#pragma unroll
-        for (uint32_t j = 0; j < 2u; ++j) {
-            const uint32_t i = b * 128u + lane + 64u * j;
-            xq[static_cast<size_t>(rk) * a.hidden + (i & ~15u) + quad_slot(i & 15u)] = hv[j] | (hv[j] << 16);
-        }
-        if (lane == 0u) (proj ? a.su : a.sg)[static_cast<size_t>(rk) * nb + b] = sum;
-    }
+    routed_prep_block<false>(a, blockIdx.y, blockIdx.y, blockIdx.x, threadIdx.x);
 }
 
 // Grid (out / 16 / BT, RKT * NPROJ, KS), 256 threads. NPROJ 2: gate (proj 0) and up (proj 1), hidden -> inter;
@@ -164,93 +115,14 @@ __global__ void __launch_bounds__(256) moe_gemv(const MoeLaunch a) {
     }
 }
 
-// One block's sums over the K slices (slice order; the first plane starts the sum) and the deferred MUL1 map.
-__device__ __forceinline__ void plane_sums(const float* z, size_t planes_stride, uint32_t ks, const float* bsum,
-                                           uint32_t nb, int defer, uint32_t lane, float (&s)[2]) {
-#pragma unroll
-    for (uint32_t j = 0; j < 2u; ++j) s[j] = z[lane + 64u * j];
-    for (uint32_t k = 1; k < ks; ++k)
-#pragma unroll
-        for (uint32_t j = 0; j < 2u; ++j) s[j] += z[k * planes_stride + lane + 64u * j];
-    if (defer) {
-        float xsum = 0.0f;
-        for (uint32_t q = 0; q < nb; ++q) xsum += bsum[q];
-#pragma unroll
-        for (uint32_t j = 0; j < 2u; ++j) s[j] = __builtin_fmaf(s[j], mul1_a(), mul1_b() * xsum);
-    }
-}
-
-// Grid (inter / 128, RKT), 64 threads: gate and up finishes, the (clamped) SwiGLU in f32 on their f16 values, and the
-// down's prepare: hd u32 [RKT][inter] (quad order, doubled), hs f32 [RKT][inter / 128].
+// Grid (inter / 128, RKT), 64 threads.
 __global__ void __launch_bounds__(64) moe_mid(const MoeLaunch a) {
-    const uint32_t b = blockIdx.x, rk = blockIdx.y, lane = threadIdx.x;
-    const SlotRef s = resolve_slot(a, rk);
-    if (!s.live) return;
-    const RoutedBank& bank = s.shared ? a.shared : a.bank;
-    const uint32_t rkt = a.rows * (a.topk + a.shared_slots), nb = a.hidden / 128u;
-    const size_t plane = static_cast<size_t>(rkt) * a.inter, at = static_cast<size_t>(rk) * a.inter + b * 128u;
-    float g[2], u[2];
-    plane_sums(a.zg + at, plane, a.ks_gu, a.sg + static_cast<size_t>(rk) * nb, nb, a.defer, lane, g);
-    plane_sums(a.zu + at, plane, a.ks_gu, a.su + static_cast<size_t>(rk) * nb, nb, a.defer, lane, u);
-    finish_values(g, bank.gate_svh + static_cast<size_t>(s.e) * a.inter, b, lane);
-    finish_values(u, bank.up_svh + static_cast<size_t>(s.e) * a.inter, b, lane);
-    float d[2];
-#pragma unroll
-    for (uint32_t j = 0; j < 2u; ++j) {
-        float gv = g[j], uv = u[j];
-        if (a.limit > 0.0f) {  // comparisons: a NaN passes through (ref.zig:132-140)
-            gv = gv > a.limit ? a.limit : gv;
-            uv = uv > a.limit ? a.limit : (uv < -a.limit ? -a.limit : uv);
-        }
-        const float hv = round_half((gv / (1.0f + expf(-gv))) * uv);
-        d[j] = hv * half_value(bank.down_suh[static_cast<size_t>(s.e) * a.inter + b * 128u + lane + 64u * j]);
-    }
-    h128_wave(d, lane);
-    float sum = 0.0f;
-#pragma unroll
-    for (uint32_t j = 0; j < 2u; ++j) {
-        const uint32_t i = b * 128u + lane + 64u * j;
-        const uint32_t hh = half_bits(d[j] * kHadScale);
-        a.hd[static_cast<size_t>(rk) * a.inter + (i & ~15u) + quad_slot(i & 15u)] = hh | (hh << 16);
-        sum += half_value(hh);
-    }
-#pragma unroll
-    for (int m = 32; m > 0; m >>= 1) sum += __shfl_xor(sum, m, 64);
-    if (lane == 0u) a.hs[static_cast<size_t>(rk) * (a.inter / 128u) + b] = sum;
+    routed_mid_block<false>(a, blockIdx.y, blockIdx.y, blockIdx.x, threadIdx.x);
 }
 
-// Grid (hidden / 128, rows), 64 threads: every slot's down finish, then the score-weighted sum in slot order.
+// Grid (hidden / 128, rows), 64 threads.
 __global__ void __launch_bounds__(64) moe_combine(const MoeLaunch a) {
-    const uint32_t b = blockIdx.x, row = blockIdx.y, lane = threadIdx.x;
-    const uint32_t kt = a.topk + a.shared_slots, rkt = a.rows * kt, nbi = a.inter / 128u;
-    const size_t plane = static_cast<size_t>(rkt) * a.hidden;
-    float acc[2] = {0.0f, 0.0f};
-    for (uint32_t k = 0; k < kt; ++k) {
-        const uint32_t rk = row * kt + k;
-        const SlotRef s = resolve_slot(a, rk);
-        if (!s.live) continue;  // uniform over the wave
-        const RoutedBank& bank = s.shared ? a.shared : a.bank;
-        float v[2];
-        plane_sums(a.zd + static_cast<size_t>(rk) * a.hidden + b * 128u, plane, a.ks_dn,
-                   a.hs + static_cast<size_t>(rk) * nbi, nbi, a.defer, lane, v);
-        finish_values(v, bank.down_svh + static_cast<size_t>(s.e) * a.hidden, b, lane);
-        const float w = s.shared ? 1.0f : score_of(a, row, k);
-#pragma unroll
-        for (uint32_t j = 0; j < 2u; ++j) acc[j] = __builtin_fmaf(w, v[j], acc[j]);
-    }
-#pragma unroll
-    for (uint32_t j = 0; j < 2u; ++j) {
-        const size_t o = static_cast<size_t>(row) * a.hidden + b * 128u + lane + 64u * j;
-        if (a.shared_add) {
-            // `moeWithShared`: the routed output rounds to x's dtype, then the add rounds again (src/root.zig:976-984)
-            float r = acc[j];
-            if (a.dtype == kF16) r = round_half(r);
-            else if (a.dtype == kBf16) r = bf16_value(bf16_bits(r));
-            store_act_rt(a.dtype, a.y, o, r + load_act_rt(a.dtype, a.shared_add, o));
-        } else {
-            store_act_rt(a.dtype, a.y, o, acc[j]);
-        }
-    }
+    routed_combine_block<false>(a, blockIdx.y, blockIdx.x, threadIdx.x);
 }
 
 template <int CB, bool WIDE, int NPROJ, bool XLDS>

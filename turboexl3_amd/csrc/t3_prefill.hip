@@ -1,0 +1,454 @@
+// Above the decode rows on gfx950: the grouped trellis GEMM on the matrix cores, the route that feeds it, and the two
+// chains it serves: routed experts beyond 16 rows (turboexl3 src/core/prefill.zig:1-24; roles of src/hip/plan.zig:
+// 380-520) and one dense projection beyond 32 rows (src/core/dense.zig:978-1034).
+//
+// The GEMM. An item is up to RB * 16 activation rows that share one weight matrix (one expert's rows after the route,
+// or a block of a dense call's rows). A workgroup takes one item and 256 output columns; each of its four waves owns
+// four adjacent 16 x 16 tiles a tile row and decodes them EXACTLY (the f16 bits of format.decodeTile), a quad of
+// weights a lane, two tile rows a step: 8 f16 = the A fragment of v_mfma_f32_16x16x32_f16 over K = 32, with no shuffle
+// and no LDS round trip for the decoded weights. The item's prepared activations (f16, quad order) go through LDS once
+// a step for all four waves and are read back as B fragments, 16 bytes a lane. Every decoded weight feeds RB MFMAs.
+// A row's sums depend on (matrix, K order) alone: not on the item it landed in, nor on the rows beside it.
+//
+// Cost (measured beside the GEMV): the exact decode is ~5 vector-ALU operations a weight and the matrix core does not
+// overlap them, so at 64 rows an item the kernel is bound by the decode, not by MFMA.
+
+#include "t3_decode.hpp"
+#include "t3_kernels.hpp"
+#include "t3_routed.hpp"
+#include "t3_stages.hpp"
+
+namespace t3 {
+namespace {
+
+constexpr uint32_t kPfTiles = 4;           // adjacent tiles a wave (a tile row's chunk: 4 * 2n <= 1 KB)
+constexpr uint32_t kPfSlot = 256;          // LDS bytes a staged tile
+constexpr uint32_t kPfRowStride = 80;      // LDS bytes an activation row a step: 64 + 16 so 16 rows hit 16 bank groups
+constexpr uint32_t kPfWStage = 2u * kPfTiles * kPfSlot + 1024u;  // two tile rows, then the dump of the idle lanes
+
+struct PfGemm {
+    const uint32_t* w[2];    // the bank's trellis a projection (gate, up) or (down, -)
+    const uint32_t* ws[2];   // the shared bank's: experts numbered from `experts` up
+    const uint16_t* xq[2];   // prepared activations f16 [positions][in], quad order
+    float* z[2];             // f32 [positions][out]
+    const uint32_t* items;   // {expert, first position, rows, 0} an item; null: dense, item i = rows i RB 16 ...
+    const uint32_t* n_items; // the route's item count (device)
+    uint32_t in, out, n, wbits, positions, experts, nblk;
+};
+
+// The weight a GEMM feeds the matrix core as one f16: exact, or MUL1's h = 1024 + t when its map is deferred.
+template <int CB>
+__device__ __forceinline__ uint32_t weight_half(uint32_t cw) {
+    if constexpr (CB == kMul1Defer) return mul1_h(cw);
+    else return static_cast<uint32_t>(decode_exact<CB>(cw));
+}
+
+// Grid (8 * nblk * ceil(max_items / 8), projections), 256 threads. Consecutive workgroup ids go round the eight dies,
+// so the workgroups that share an item's activations (its nblk column blocks) are given ids 8 apart: one die's L2
+// serves them all.
+template <int CB, bool WIDE, int RB>
+__global__ void __launch_bounds__(256) pf_gemm(const PfGemm a) {
+    constexpr uint32_t BM = RB * 16u;
+    constexpr uint32_t kABuf = BM * kPfRowStride;
+    constexpr uint32_t kPieces = BM * 4u;                      // 16-byte pieces of an item's rows a step
+    constexpr uint32_t kALoads = (kPieces + 255u) / 256u;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[2u * kABuf + 4u * kPfWStage];
+
+    const uint32_t id = blockIdx.x, proj = blockIdx.y;
+    const uint32_t j = id >> 3, blk = j % a.nblk, item_i = (j / a.nblk) * 8u + (id & 7u);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u, tid = threadIdx.x;
+    uint32_t e = 0, first, count;
+    if (a.items) {
+        if (item_i >= a.n_items[0]) return;
+        e = a.items[item_i * 4u];
+        first = a.items[item_i * 4u + 1u];
+        count = a.items[item_i * 4u + 2u];
+    } else {
+        first = item_i * BM;
+        if (first >= a.positions) return;
+        count = a.positions - first < BM ? a.positions - first : BM;
+    }
+    const uint32_t in_tiles = a.in >> 4, out_tiles = a.out >> 4, nw = a.n >> 1;
+    const bool from_shared = e >= a.experts;
+    const uint32_t* wmat = (from_shared ? a.ws[proj] : a.w[proj]) +
+                           static_cast<size_t>(from_shared ? e - a.experts : e) * in_tiles * out_tiles * nw;
+    const uint32_t col0 = blk * 16u + wave * kPfTiles;  // the wave's first tile column
+    const bool active = col0 < out_tiles;               // uniform over the wave (out is a multiple of 128, not of 256)
+    const uint32_t wstep = out_tiles * nw * 4u;
+    const uint32_t tile_bytes = 2u * a.n, chunk_bytes = kPfTiles * tile_bytes;
+    // the wave's window of the matrix: a tile row past the last one falls outside it and reads as zeros
+    const __amdgpu_buffer_rsrc_t wres =
+        make_rsrc(wmat + static_cast<size_t>(col0) * nw, active ? (in_tiles - 1u) * wstep + chunk_bytes : 0u);
+    const uint32_t wvoff = lane * 16u < chunk_bytes ? lane * 16u : 0x40000000u;
+    const __amdgpu_buffer_rsrc_t xres = make_rsrc(a.xq[proj], static_cast<uint64_t>(a.positions) * a.in * 2u);
+
+    unsigned char* abuf = smem;
+    unsigned char* stage = smem + 2u * kABuf + wave * kPfWStage;
+
+    // where this thread's pieces of the item's rows come from and go
+    uint32_t a_voff[kALoads], a_put[kALoads];
+    bool a_live[kALoads];
+#pragma unroll
+    for (uint32_t i = 0; i < kALoads; ++i) {
+        const uint32_t idx = tid + 256u * i, row = idx >> 2, piece = idx & 3u;
+        a_live[i] = idx < kPieces;
+        a_voff[i] = a_live[i] && row < count ? ((first + row) * a.in + piece * 8u) * 2u : 0x80000000u;
+        // 8 halves = tile piece / 2, quads 2 (piece % 2) and + 1: row, then quad, then tile, 8 bytes each
+        a_put[i] = row * kPfRowStride + (piece & 1u) * 32u + (piece >> 1) * 8u;
+    }
+    auto load_a = [&](uint32_t step, uint4v(&dst)[kALoads]) {
+#pragma unroll
+        for (uint32_t i = 0; i < kALoads; ++i) dst[i] = buf_load_u128(xres, a_voff[i], step * 64u);
+    };
+    auto put_a = [&](const uint4v(&src)[kALoads], uint32_t parity) {
+#pragma unroll
+        for (uint32_t i = 0; i < kALoads; ++i)
+            if (a_live[i]) {
+                unsigned char* p = abuf + parity * kABuf + a_put[i];
+                *reinterpret_cast<uint2*>(p) = make_uint2(src[i][0], src[i][1]);
+                *reinterpret_cast<uint2*>(p + 16u) = make_uint2(src[i][2], src[i][3]);
+            }
+    };
+
+    const QuadPlan<WIDE> plan = quad_plan<WIDE>(a.n, lane);
+    const uint32_t inv_tile = (1u << 16) / tile_bytes + 1u;
+    const bool writer = lane * 16u < chunk_bytes;
+    uint32_t put[4];
+#pragma unroll
+    for (uint32_t jj = 0; jj < 4u; ++jj) {
+        const uint32_t b = lane * 16u + 4u * jj;
+        const uint32_t t = (b * inv_tile) >> 16;
+        put[jj] = writer ? t * kPfSlot + (b - t * tile_bytes) : 2u * kPfTiles * kPfSlot + lane * 16u + 4u * jj;
+    }
+    const uint32_t get_bp = plan.ib_prev * 4u, get_bl = plan.ib_last * 4u;
+    const uint32_t get_ap = plan.ia_prev * 4u, get_al = plan.ia_last * 4u;
+
+    auto load_w = [&](uint32_t step, uint4v(&dst)[2]) {
+        dst[0] = buf_load_u128(wres, wvoff, (2u * step) * wstep);
+        dst[1] = buf_load_u128(wres, wvoff, (2u * step + 1u) * wstep);
+    };
+    auto stage_w = [&](const uint4v(&src)[2]) {
+#pragma unroll
+        for (uint32_t r = 0; r < 2u; ++r)
+#pragma unroll
+            for (uint32_t jj = 0; jj < 4u; ++jj)
+                *reinterpret_cast<uint32_t*>(stage + (writer ? r * (kPfTiles * kPfSlot) : 0u) + put[jj]) = src[r][jj];
+    };
+    auto fetch_w = [&](QuadWords<WIDE>(&wd)[2][kPfTiles]) {
+#pragma unroll
+        for (uint32_t r = 0; r < 2u; ++r)
+#pragma unroll
+            for (uint32_t t = 0; t < kPfTiles; ++t) {
+                const unsigned char* slot = stage + (r * kPfTiles + t) * kPfSlot;
+                wd[r][t].b_prev = *reinterpret_cast<const uint32_t*>(slot + get_bp);
+                wd[r][t].b_last = *reinterpret_cast<const uint32_t*>(slot + get_bl);
+                if constexpr (WIDE) {
+                    wd[r][t].a_prev = *reinterpret_cast<const uint32_t*>(slot + get_ap);
+                    wd[r][t].a_last = *reinterpret_cast<const uint32_t*>(slot + get_al);
+                }
+            }
+    };
+
+    float4v acc[RB][kPfTiles];
+#pragma unroll
+    for (int mb = 0; mb < RB; ++mb)
+#pragma unroll
+        for (uint32_t t = 0; t < kPfTiles; ++t) acc[mb][t] = float4v{0.f, 0.f, 0.f, 0.f};
+
+    // one step: K = 32 = tile rows 2 step and 2 step + 1
+    auto compute = [&](const QuadWords<WIDE>(&wd)[2][kPfTiles], uint32_t parity) {
+        uint4v bf[RB];
+#pragma unroll
+        for (int mb = 0; mb < RB; ++mb)
+            bf[mb] = *reinterpret_cast<const uint4v*>(abuf + parity * kABuf +
+                                                      (static_cast<uint32_t>(mb) * 16u + (lane & 15u)) * kPfRowStride +
+                                                      (lane >> 4) * 16u);
+#pragma unroll
+        for (uint32_t t = 0; t < kPfTiles; ++t) {
+            uint32_t c0[4], c1[4];
+            quad_codewords<WIDE>(wd[0][t], plan, a.wbits, c0);
+            quad_codewords<WIDE>(wd[1][t], plan, a.wbits, c1);
+            uint4v af;
+            af[0] = weight_half<CB>(c0[0]) | (weight_half<CB>(c0[1]) << 16);
+            af[1] = weight_half<CB>(c0[2]) | (weight_half<CB>(c0[3]) << 16);
+            af[2] = weight_half<CB>(c1[0]) | (weight_half<CB>(c1[1]) << 16);
+            af[3] = weight_half<CB>(c1[2]) | (weight_half<CB>(c1[3]) << 16);
+#pragma unroll
+            for (int mb = 0; mb < RB; ++mb)
+                acc[mb][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, af),
+                                                                    __builtin_bit_cast(half8, bf[mb]), acc[mb][t], 0, 0, 0);
+        }
+    };
+
+    const uint32_t steps = in_tiles >> 1;  // even: in is a multiple of 128
+    uint4v wreg[2], areg[kALoads];
+    QuadWords<WIDE> wd0[2][kPfTiles], wd1[2][kPfTiles];
+    load_w(0u, wreg);
+    load_a(0u, areg);
+    put_a(areg, 0u);
+    stage_w(wreg);
+    fetch_w(wd0);
+    load_w(1u, wreg);
+    load_a(1u, areg);
+    __syncthreads();
+    for (uint32_t s = 0; s < steps; s += 2u) {
+        // even step: words in wd0, activations in buffer 0; wreg / areg hold step s + 1
+        stage_w(wreg);
+        load_w(s + 2u, wreg);
+        fetch_w(wd1);
+        compute(wd0, 0u);
+        put_a(areg, 1u);
+        load_a(s + 2u, areg);
+        __syncthreads();
+        // odd step
+        stage_w(wreg);
+        load_w(s + 3u, wreg);
+        fetch_w(wd0);
+        compute(wd1, 1u);
+        put_a(areg, 0u);
+        load_a(s + 3u, areg);
+        __syncthreads();
+    }
+
+    if (!active) return;
+    // D[i][j]: i = the weight's column inside its tile (this lane: 4 (lane / 16) .. + 3), j = activation row lane % 16
+    float* z = a.z[proj];
+#pragma unroll
+    for (int mb = 0; mb < RB; ++mb) {
+        const uint32_t row = static_cast<uint32_t>(mb) * 16u + (lane & 15u);
+        if (row >= count) continue;
+#pragma unroll
+        for (uint32_t t = 0; t < kPfTiles; ++t)
+            *reinterpret_cast<float4v*>(z + static_cast<size_t>(first + row) * a.out + (col0 + t) * 16u + 4u * (lane >> 4)) =
+                acc[mb][t];
+    }
+}
+
+// ---- the route (src/hip/plan.zig:40-45,412-415: order, inv, items, counts) -------------------------------------
+
+// expert number of a row-slot in [0, experts + shared slots), or ~0 for a skipped id
+__device__ __forceinline__ uint32_t slot_expert(const MoeLaunch& a, uint32_t rk) {
+    const SlotRef s = resolve_slot(a, rk);
+    if (!s.live) return ~0u;
+    return s.shared ? a.bank.experts + s.e : s.e;
+}
+
+__global__ void __launch_bounds__(256) pf_clear(uint32_t* counts, uint32_t len) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i < len) counts[i] = 0u;
+}
+
+__global__ void __launch_bounds__(256) pf_hist(const MoeLaunch a) {
+    const uint32_t rk = blockIdx.x * 256u + threadIdx.x;
+    if (rk >= a.rows * (a.topk + a.shared_slots)) return;
+    const uint32_t e = slot_expert(a, rk);
+    if (e != ~0u) atomicAdd(a.counts + e, 1u);
+}
+
+// One workgroup of 1024: exclusive sums of the experts' counts (positions) and of their item counts; every expert
+// writes its own items. counts[E]: items in all; counts[E + 1]: positions placed.
+__global__ void __launch_bounds__(1024) pf_scan(const MoeLaunch a) {
+    __shared__ uint32_t wave_pos[16], wave_items[16], carry[2];
+    const uint32_t et = a.bank.experts + a.shared_slots, tid = threadIdx.x, lane = tid & 63u, wv = tid >> 6;
+    if (tid == 0u) carry[0] = carry[1] = 0u;
+    __syncthreads();
+    for (uint32_t base = 0; base < et; base += 1024u) {
+        const uint32_t e = base + tid;
+        const uint32_t c = e < et ? a.counts[e] : 0u;
+        const uint32_t ni = (c + a.item_rows - 1u) / a.item_rows;
+        uint32_t pos = c, it = ni;  // inclusive sums inside the wave
+#pragma unroll
+        for (uint32_t d = 1; d < 64u; d <<= 1) {
+            const uint32_t p = __shfl_up(pos, d, 64), q = __shfl_up(it, d, 64);
+            if (lane >= d) {
+                pos += p;
+                it += q;
+            }
+        }
+        if (lane == 63u) {
+            wave_pos[wv] = pos;
+            wave_items[wv] = it;
+        }
+        __syncthreads();
+        uint32_t pos0 = carry[0], it0 = carry[1];
+        for (uint32_t w = 0; w < wv; ++w) {
+            pos0 += wave_pos[w];
+            it0 += wave_items[w];
+        }
+        pos0 += pos - c;  // exclusive
+        it0 += it - ni;
+        if (e < et) {
+            a.cursor[e] = pos0;
+            for (uint32_t i = 0; i < ni; ++i) {
+                uint32_t* item = a.items + static_cast<size_t>(it0 + i) * 4u;
+                const uint32_t left = c - i * a.item_rows;
+                item[0] = e;
+                item[1] = pos0 + i * a.item_rows;
+                item[2] = left < a.item_rows ? left : a.item_rows;
+                item[3] = 0u;
+            }
+        }
+        __syncthreads();
+        if (tid == 1023u) {
+            carry[0] = pos0 + c;
+            carry[1] = it0 + ni;
+        }
+        __syncthreads();
+    }
+    if (tid == 0u) {
+        a.counts[et] = carry[1];
+        a.counts[et + 1u] = carry[0];
+    }
+}
+
+// Where a row-slot lands inside its expert's run does not matter to any sum, so the runs are filled in arrival order.
+__global__ void __launch_bounds__(256) pf_place(const MoeLaunch a) {
+    const uint32_t rk = blockIdx.x * 256u + threadIdx.x;
+    if (rk >= a.rows * (a.topk + a.shared_slots)) return;
+    const uint32_t e = slot_expert(a, rk);
+    if (e == ~0u) {
+        a.inv[rk] = ~0u;
+        return;
+    }
+    const uint32_t q = atomicAdd(a.cursor + e, 1u);
+    a.order[q] = rk;
+    a.inv[rk] = q;
+}
+
+// ---- the routed chain's stages by sorted position: grid (blocks * positions), 64 threads -------------------------
+
+__global__ void __launch_bounds__(64) pf_prep(const MoeLaunch a) {
+    const uint32_t nb = a.hidden / 128u, q = blockIdx.x / nb, b = blockIdx.x % nb;
+    if (q >= a.counts[a.bank.experts + a.shared_slots + 1u]) return;
+    routed_prep_block<true>(a, a.order[q], q, b, threadIdx.x);
+}
+
+__global__ void __launch_bounds__(64) pf_mid(const MoeLaunch a) {
+    const uint32_t nb = a.inter / 128u, q = blockIdx.x / nb, b = blockIdx.x % nb;
+    if (q >= a.counts[a.bank.experts + a.shared_slots + 1u]) return;
+    routed_mid_block<true>(a, a.order[q], q, b, threadIdx.x);
+}
+
+__global__ void __launch_bounds__(64) pf_combine(const MoeLaunch a) {
+    const uint32_t nb = a.hidden / 128u;
+    routed_combine_block<true>(a, blockIdx.x / nb, blockIdx.x % nb, threadIdx.x);
+}
+
+// ---- dense prepare: grid (in / 128 * rows), 64 threads: plain f16 in quad order, block sums ----------------------
+
+__global__ void __launch_bounds__(64) pf_dense_prep(const void* x, const uint16_t* suh, uint16_t* xq, float* xs,
+                                                    uint32_t in, int dt) {
+    const uint32_t nb = in / 128u, row = blockIdx.x / nb, b = blockIdx.x % nb, lane = threadIdx.x;
+    uint32_t hv[2];
+    float sum;
+    prep_values(dt, x, suh, in, row, b, lane, hv, sum);
+#pragma unroll
+    for (uint32_t j = 0; j < 2u; ++j) {
+        const uint32_t i = b * 128u + lane + 64u * j;
+        xq[static_cast<size_t>(row) * in + (i & ~15u) + quad_slot(i & 15u)] = static_cast<uint16_t>(hv[j]);
+    }
+    if (lane == 0u) xs[static_cast<size_t>(row) * nb + b] = sum;
+}
+
+template <int CB, bool WIDE>
+hipError_t launch_gemm_rb(const PfGemm& g, uint32_t max_items, uint32_t nproj, uint32_t item_rows, hipStream_t s) {
+    const dim3 grid(8u * g.nblk * ((max_items + 7u) / 8u), nproj), block(256);
+    if (item_rows == 32u) hipLaunchKernelGGL((pf_gemm<CB, WIDE, 2>), grid, block, 0, s, g);
+    else hipLaunchKernelGGL((pf_gemm<CB, WIDE, 4>), grid, block, 0, s, g);
+    return hipGetLastError();
+}
+
+// The GEMM decodes exactly whatever form the GEMV runs: MCG's pair form has no use here (it would double K).
+hipError_t launch_gemm(const PfGemm& g, int codebook, uint32_t max_items, uint32_t nproj, uint32_t item_rows,
+                       hipStream_t s) {
+    const bool wide = quad_needs_wide(g.n);
+    switch (codebook) {
+        case kMul1:
+            return wide ? launch_gemm_rb<kMul1, true>(g, max_items, nproj, item_rows, s)
+                        : launch_gemm_rb<kMul1, false>(g, max_items, nproj, item_rows, s);
+        case kMul1Defer:
+            return wide ? launch_gemm_rb<kMul1Defer, true>(g, max_items, nproj, item_rows, s)
+                        : launch_gemm_rb<kMul1Defer, false>(g, max_items, nproj, item_rows, s);
+        default:
+            return wide ? launch_gemm_rb<kMcg, true>(g, max_items, nproj, item_rows, s)
+                        : launch_gemm_rb<kMcg, false>(g, max_items, nproj, item_rows, s);
+    }
+}
+
+}  // namespace
+
+hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s) {
+    const uint32_t kt = a.topk + a.shared_slots, p = a.rows * kt, et = a.bank.experts + a.shared_slots;
+    hipError_t e;
+    hipLaunchKernelGGL(pf_clear, dim3((et + 2u + 255u) / 256u), dim3(256), 0, s, a.counts, et + 2u);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+    hipLaunchKernelGGL(pf_hist, dim3((p + 255u) / 256u), dim3(256), 0, s, a);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+    hipLaunchKernelGGL(pf_scan, dim3(1), dim3(1024), 0, s, a);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+    hipLaunchKernelGGL(pf_place, dim3((p + 255u) / 256u), dim3(256), 0, s, a);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+    hipLaunchKernelGGL(pf_prep, dim3(p * (a.hidden / 128u)), dim3(64), 0, s, a);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+
+    PfGemm g{};
+    g.w[0] = a.bank.gate_t;
+    g.w[1] = a.bank.up_t;
+    g.ws[0] = a.shared.gate_t;
+    g.ws[1] = a.shared.up_t;
+    g.xq[0] = reinterpret_cast<const uint16_t*>(a.xg);
+    g.xq[1] = reinterpret_cast<const uint16_t*>(a.xu);
+    g.z[0] = a.zg;
+    g.z[1] = a.zu;
+    g.items = a.items;
+    g.n_items = a.counts + et;
+    g.in = a.hidden;
+    g.out = a.inter;
+    g.n = a.n_gu;
+    g.wbits = a.wbits;
+    g.positions = p;
+    g.experts = a.bank.experts;
+    g.nblk = (a.inter + 255u) / 256u;
+    if ((e = launch_gemm(g, a.codebook, a.max_items, 2u, a.item_rows, s)) != hipSuccess) return e;
+
+    hipLaunchKernelGGL(pf_mid, dim3(p * (a.inter / 128u)), dim3(64), 0, s, a);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+
+    g.w[0] = a.bank.down_t;
+    g.ws[0] = a.shared.down_t;
+    g.w[1] = g.ws[1] = nullptr;
+    g.xq[0] = reinterpret_cast<const uint16_t*>(a.hd);
+    g.xq[1] = nullptr;
+    g.z[0] = a.zd;
+    g.z[1] = nullptr;
+    g.in = a.inter;
+    g.out = a.hidden;
+    g.n = a.n_dn;
+    g.nblk = (a.hidden + 255u) / 256u;
+    if ((e = launch_gemm(g, a.codebook, a.max_items, 1u, a.item_rows, s)) != hipSuccess) return e;
+
+    hipLaunchKernelGGL(pf_combine, dim3(a.rows * (a.hidden / 128u)), dim3(64), 0, s, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_dense_prefill(const DenseLaunch& d, hipStream_t s) {
+    hipError_t e;
+    hipLaunchKernelGGL(pf_dense_prep, dim3(d.rows * (d.in / 128u)), dim3(64), 0, s, d.x, d.suh,
+                       reinterpret_cast<uint16_t*>(d.xq), d.xs, d.in, d.dtype);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+    PfGemm g{};
+    g.w[0] = d.trellis;
+    g.xq[0] = reinterpret_cast<const uint16_t*>(d.xq);
+    g.z[0] = d.z;
+    g.in = d.in;
+    g.out = d.out;
+    g.n = d.n;
+    g.wbits = d.wbits;
+    g.positions = d.rows;
+    g.experts = 1u;
+    g.nblk = (d.out + 255u) / 256u;
+    if ((e = launch_gemm(g, d.codebook, (d.rows + 63u) / 64u, 1u, 64u, s)) != hipSuccess) return e;
+    return launch_dense_finish(d, s);
+}
+
+}  // namespace t3
