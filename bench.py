@@ -184,6 +184,58 @@ class MoeRunner:
     time = DenseRunner.time
 
 
+class PrefillRunner:
+    """BASELINE config 4: 2048 tokens, 256 experts, top-8, hidden 7168, inter 2048, gate|up K2, down K3, bf16, clamp 7.
+    flops = tokens * topk * 3 * 2 * hidden * inter. `scale` shrinks experts and tokens together (same rows an expert)."""
+
+    def __init__(self, torch, api, tokens=2048, experts=256, topk=8, hidden=7168, inter=2048, k_gu=2, k_dn=3, seed=9):
+        import ctypes as C
+
+        from turboexl3_amd import _lib
+        self.C, self.L, self.torch, self.api = C, _lib.lib(), torch, api
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+
+        def proj(in_f, out_f, k):
+            t = torch.randint(-32768, 32768, (experts, in_f // 16, out_f // 16, 16 * k), dtype=torch.int16,
+                              device="cuda", generator=g)
+            suh = (0.5 + torch.rand(experts, in_f, device="cuda", generator=g)).to(torch.float16)
+            svh = ((0.5 + torch.rand(experts, out_f, device="cuda", generator=g)) / in_f ** 0.5).to(torch.float16)
+            return api.Proj(t, suh, svh)
+
+        self.bank = api.Bank(proj(hidden, inter, k_gu), proj(hidden, inter, k_gu), proj(inter, hidden, k_dn))
+        self.x = torch.randn(1, tokens, hidden, device="cuda", generator=g).to(torch.bfloat16)
+        logits = torch.randn(tokens, experts, device="cuda", generator=g)
+        top = torch.topk(logits, topk, dim=-1)
+        self.inds = top.indices.to(torch.int32).reshape(1, tokens, topk).contiguous()
+        self.scores = torch.softmax(top.values, dim=-1).to(torch.float32).reshape(1, tokens, topk).contiguous()
+        self.cb, self._k1 = api._cbank(self.bank)
+        self.ax, self.ai, self.asc = api._arr(self.x), api._arr(self.inds), api._arr(self.scores)
+        self.y = torch.empty_like(self.x)
+        self.ay = api._arr(self.y)
+        need = C.c_size_t(0)
+        st = self.L.t3_moe_workspace_bytes(C.byref(self.ax), C.byref(self.cb), C.byref(self.ai), None, C.byref(need))
+        assert st == 0, _lib.error_name(st)
+        self.ws = torch.zeros(need.value, dtype=torch.uint8, device="cuda")
+        self.dec = api.Decode.mcg.c()
+        self.stream = torch.cuda.current_stream().cuda_stream
+        self.flops = tokens * topk * 3 * 2 * hidden * inter
+        self.code_bytes = experts * (2 * code_bytes_of(hidden, inter, 16 * k_gu) + code_bytes_of(inter, hidden, 16 * k_dn))
+
+    def call(self, i: int, stages: int = 0):
+        C = self.C
+        st = self.L.t3_moe_clamped(self.stream, C.byref(self.ax), C.byref(self.cb), C.byref(self.ai), C.byref(self.asc),
+                                   self.dec, 7, C.byref(self.ay), self.ws.data_ptr(), self.ws.numel())
+        if st != 0:
+            raise RuntimeError(self.L.t3_error_name(st).decode())
+
+    time = DenseRunner.time
+
+
+def code_bytes_of(in_f: int, out_f: int, n: int) -> int:
+    return (in_f // 16) * (out_f // 16) * n * 2
+
+
 def cpu_baseline(n: int, seed: int, budget_s: float = 20.0):
     """format.project (the C oracle) on the host: the same shape and seeded distributions, one row, one thread,
     re-decoding every tile as the reference does. A bounded sample: whole calls until ~budget_s is spent."""
@@ -224,6 +276,8 @@ def main() -> int:
     ap.add_argument("--k", type=int, default=4)
     ap.add_argument("--rows", type=int, default=1)
     ap.add_argument("--moe", action="store_true", help="also time the routed-expert decode chain (config 3)")
+    ap.add_argument("--prefill", action="store_true",
+                    help="also time the routed prefill chain (config 4) and the dense 4096-row projection (config 5)")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run one 256 MiB device copy, the known-size kernel that scales the profiler's "
                          "FETCH_SIZE / WRITE_SIZE readings")
@@ -287,6 +341,33 @@ def main() -> int:
             out["moe_decode"].append({"tokens": tokens, "us_per_call": t * 1e6, "code_bytes": run.code_bytes,
                                       "gbps": run.code_bytes / t / 1e9, "frac_of_hbm": run.code_bytes / t / HBM_PEAK})
             del run
+    if args.prefill:
+        run = PrefillRunner(torch, api)
+        t = run.time(5, 2)
+        out["moe_prefill"] = {"workload": "2048 tokens, E256 top-8, 7168/2048, gate|up K2, down K3, bf16, clamp 7",
+                              "ms_per_call": t * 1e3, "tflops": run.flops / t / 1e12,
+                              "frac_of_f16_mfma_peak": run.flops / t / 2.5e15, "code_gbps": run.code_bytes / t / 1e9}
+        del run
+        torch.cuda.empty_cache()
+        rows, in_f, out_f, k = 4096, 4096, 14336, 4
+        g = torch.Generator(device="cuda")
+        g.manual_seed(3)
+        tr = torch.randint(-32768, 32768, (in_f // 16, out_f // 16, 16 * k), dtype=torch.int16, device="cuda", generator=g)
+        suh = (0.5 + torch.rand(in_f, device="cuda", generator=g)).to(torch.float16)
+        svh = ((0.5 + torch.rand(out_f, device="cuda", generator=g)) / in_f ** 0.5).to(torch.float16)
+        x = torch.randn(rows, in_f, device="cuda", generator=g).to(torch.bfloat16)
+        api.linear(x, tr, suh, svh, dec)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(5):
+            api.linear(x, tr, suh, svh, dec)
+        e1.record()
+        torch.cuda.synchronize()
+        t = e0.elapsed_time(e1) * 1e-3 / 5
+        out["dense_prefill"] = {"workload": "4096 rows x (4096 -> 14336) K4 bf16", "ms_per_call": t * 1e3,
+                                "tflops": 2 * rows * in_f * out_f / t / 1e12,
+                                "frac_of_f16_mfma_peak": 2 * rows * in_f * out_f / t / 2.5e15}
     if args.sweep:
         out["sweep"] = [measure(k, r, max(50, args.steps // 4), 10) for k in (3, 4, 5) for r in (1, 4, 16, 32)]
     if not args.no_cpu:

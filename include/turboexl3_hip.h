@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define T3_ABI_VERSION 1
+#define T3_ABI_VERSION 2
 #define T3_WORKSPACE_COUNTER_BYTES 65536
 
 typedef void* t3_stream; /* hipStream_t */
@@ -91,11 +91,14 @@ typedef struct t3_bank {
 /* ---- configuration (src/core/config.zig; only the fields this path reads) --------------------------------- */
 
 typedef struct t3_config {
-    int32_t decode_form;   /* 3: the five-launch chain; 9 (default): the fused form; others refused */
+    int32_t decode_form;   /* 3: the five-launch chain; 4: four launches (prepare inside gate|up); 9 (default): two
+                            * launches (mid and combine run by the last workgroup to arrive); others refused */
     int32_t dec_one;       /* 1 (default): dense decode rows in one launch; 0: the three-launch chain */
     int32_t prefill;       /* 1 (default); 0: routed calls above 16 rows refuse Exl3EngineNotImplemented */
     int32_t mcg_pair;      /* 1 (default): MCG's GEMV feeds the hashed pair to the matrix core unrounded; 0: the f16 weight */
     int32_t mul1_defer;    /* 1 (default): MUL1's affine map applied once an output (src/core/dense.zig deferFor); 0: per weight */
+    int32_t dense_gemm_rows; /* dense calls of this many rows or more decode W_hat once into the workspace and run a plain
+                              * f16 GEMM (rocBLAS, opened at run time; absent: the trellis GEMM serves). Default 512; 0: never */
 } t3_config;
 
 /* The served configuration. */
@@ -110,7 +113,8 @@ void t3_release_engines(void);
 /* ---- dense projection (src/root.zig:309-351 `linear`) ------------------------------------------------------- */
 
 /* y [..., out] in x's dtype for x [..., in]. Rows = the product of x's leading dims.
- * 1..32 rows: the trellis GEMV on the matrix cores; more: W_hat decode + f16 GEMM. `y` is the caller's, shaped as x
+ * 1..32 rows: the trellis GEMV on the matrix cores; more: the trellis GEMM (weights decoded in registers), and from
+ * t3_config.dense_gemm_rows rows: W_hat decoded once + a plain f16 GEMM. `y` is the caller's, shaped as x
  * with the last dim `out`. Status as root.linearOn's checks. */
 int32_t t3_linear(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
                   const t3_array* svh, t3_decode dec, t3_array* y, void* workspace, size_t workspace_bytes);
@@ -141,7 +145,7 @@ int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_
 
 /* x [B, S, D]; inds (U32/I32) and scores (F32/BF16/F16) [B, S, K], K <= 32; y [B, S, D] in x's dtype.
  * `verify_rows` is accepted and ignored, as in the reference (src/root.zig:822-825). Up to 16 rows: the split-K GEMV
- * chain, four launches (five under decode_form 3, the same bytes). A routed id outside [0, E) is skipped. Gate and up
+ * chain, two launches (four or five under decode_form 4 or 3, the same bytes). A routed id outside [0, E) is skipped. Gate and up
  * must share a rate (T3_Exl3GateUpRateMismatch); the down's rate may differ (the reference refuses that,
  * src/root.zig:841; this library's kernels take a rate a launch). */
 int32_t t3_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,

@@ -54,9 +54,12 @@ def test_configure_refuses_unserved_values(lib):
     from turboexl3_amd._lib import Config
     cfg = Config()
     lib.t3_config_default(C.byref(cfg))
-    assert (cfg.decode_form, cfg.dec_one, cfg.prefill, cfg.mcg_pair, cfg.mul1_defer) == (9, 1, 1, 1, 1)
-    cfg.decode_form = 4
+    assert (cfg.decode_form, cfg.dec_one, cfg.prefill, cfg.mcg_pair, cfg.mul1_defer, cfg.dense_gemm_rows) == (9, 1, 1, 1, 1, 512)
+    cfg.decode_form = 5
     assert lib.t3_error_name(lib.t3_configure(C.byref(cfg))).decode() == "InvalidTurboexl3Config"
+    cfg.decode_form, cfg.dense_gemm_rows = 9, -1
+    assert lib.t3_error_name(lib.t3_configure(C.byref(cfg))).decode() == "InvalidTurboexl3Config"
+    cfg.dense_gemm_rows = 512
     cfg.decode_form = 3
     assert lib.t3_configure(C.byref(cfg)) == 0
     cfg.decode_form = 9

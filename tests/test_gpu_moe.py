@@ -116,23 +116,34 @@ def test_moe_decode_rows_1_to_16(oracle, t3, hidden, inter, experts, topk, n, co
     print(f"moe decode {hidden}x{inter} n={n} cb={codebook} {dtype}: worst {worst:.3e} (bar {bar})")
 
 
-def test_four_launch_form_equals_five_launch_form(oracle, t3):
-    # src/hip_tests.zig:885-928: form 9's bytes are form 3's
+def test_launch_forms_give_the_same_bytes(oracle, t3):
+    # src/hip_tests.zig:885-928: form 9's bytes are form 3's. Here: two launches (default), four, five; twice in a row
+    # (the arrival counters go back to zero), with skipped slots, a clamp and a shared expert in the same launches
     rng = np.random.default_rng(9)
-    for codebook, n in ((MCG, 64), (MUL1, 48)):
+    for codebook, n, rows, topk in ((MCG, 64, 5, 4), (MUL1, 48, 16, 4), (MUL1, 96, 3, 2)):
         bank = oracle.synth_bank(rng, 8, 512, 256, n)
-        dbank = dev_bank(t3, bank)
-        x_dev, _ = make_x(rng, 5, 512, torch.bfloat16)
-        slots, scores = routing(rng, 5, 4, 8)
-        args = (x_dev.reshape(1, 5, 512), dbank, torch.from_numpy(slots).cuda().reshape(1, 5, 4),
-                torch.from_numpy(scores).cuda().reshape(1, 5, 4), t3.Decode(codebook, 16))
-        nine = t3.moe(*args)
-        t3.configure(decode_form=3)
-        try:
-            three = t3.moe(*args)
-        finally:
-            t3.configure()
-        assert bytes_of(nine) == bytes_of(three)
+        shared = oracle.synth_bank(rng, 1, 512, 256, n)
+        dbank, dshared = dev_bank(t3, bank), dev_bank(t3, shared)
+        x_dev, _ = make_x(rng, rows, 512, torch.bfloat16)
+        slots, scores = routing(rng, rows, topk, 8)
+        slots[0, 1] = -1
+        slots[rows - 1, 0] = 8
+        d_slots = torch.from_numpy(slots).cuda().reshape(1, rows, topk)
+        d_scores = torch.from_numpy(scores).cuda().reshape(1, rows, topk)
+        dec = t3.Decode(codebook, 16)
+        calls = (lambda: t3.moe(x_dev.reshape(1, rows, 512), dbank, d_slots, d_scores, dec),
+                 lambda: t3.moe_shared_expert(x_dev.reshape(1, rows, 512), dbank, d_slots, d_scores, dec, 1, dshared))
+        for call in calls:
+            nine = call()
+            again = call()
+            assert bytes_of(nine) == bytes_of(again)
+            for form in (3, 4):
+                t3.configure(decode_form=form)
+                try:
+                    other = call()
+                finally:
+                    t3.configure()
+                assert bytes_of(nine) == bytes_of(other), f"form 9 differs from form {form}"
 
 
 def test_clamp_skipped_slots_and_score_dtypes(oracle, t3):

@@ -161,3 +161,32 @@ def test_routed_prefill_clamp_skips_mixed_rates_shared(oracle, t3):
         assert err.value.name == "Exl3EngineNotImplemented"
     finally:
         t3.configure()
+
+
+@pytest.mark.parametrize("in_f,out_f,n,codebook,dtype", [
+    (512, 384, 64, MCG, torch.float32),
+    (1024, 512, 48, MUL1, torch.float16),
+    (2560, 640, 80, MUL1, torch.bfloat16),
+])
+def test_dense_w_hat_form_from_512_rows(oracle, t3, in_f, out_f, n, codebook, dtype):
+    """From t3_config.dense_gemm_rows rows a dense call decodes W_hat once and multiplies with the library's f16 GEMM
+    (the reference's dequant + matmul + finish, src/core/dense.zig:909-922,1290-1302; held to the same bars, as its
+    Metal form is in src/core/gpu_test.zig:394-438). Without rocBLAS the call stays on the trellis GEMM: same bars."""
+    case = DenseCase(oracle, t3, 0xA11 + in_f + n, in_f, out_f, n, codebook)
+    rows = 530
+    x_dev, x_f32 = make_x(case.rng, rows, in_f, dtype, outliers=True)
+    yref = case.ref(x_f32)
+    bar = F32_BAR if dtype == torch.float32 else BF16_DENSE_BAR
+    got = to_f32(t3.linear(x_dev, case.d_trellis, case.d_suh, case.d_svh, case.dec))
+    t3.configure(dense_gemm_rows=0)
+    try:
+        fused = to_f32(t3.linear(x_dev, case.d_trellis, case.d_suh, case.d_svh, case.dec))
+    finally:
+        t3.configure()
+    worst = 0.0
+    for r in range(rows):
+        for name, y in (("w_hat", got), ("trellis", fused)):
+            e = oracle.compare(y[r], yref[r])
+            worst = max(worst, e)
+            assert e <= bar, f"{name} form row {r}: {e:.3e} over the bar {bar}"
+    print(f"dense W_hat form {in_f}x{out_f} n={n} {dtype}: worst {worst:.3e} (bar {bar})")

@@ -57,6 +57,7 @@ struct MoeLaunch {
     const void* scores = nullptr;    // [rows][topk] in score_dt
     const void* shared_add = nullptr;  // moeWithShared: [rows][hidden] in dtype, or null
     void* y = nullptr;
+    uint32_t* arrive = nullptr;  // the two-launch form's arrival counters
     uint32_t* xg = nullptr;      // u32 [RKT][hidden]
     uint32_t* xu = nullptr;
     uint32_t* hd = nullptr;      // u32 [RKT][inter]
@@ -82,15 +83,21 @@ struct MoeLaunch {
     uint32_t max_items = 0, item_rows = 64;
 };
 
-// prepare_apart: five launches (prepare, gate|up, mid, down, combine); else four (each gate|up wave prepares its own
-// 128-block in LDS). The same bytes.
-hipError_t launch_moe_decode(const MoeLaunch& a, bool prepare_apart, hipStream_t s);
+// Five launches (prepare, gate|up, mid, down, combine); four (each gate|up wave prepares its own 128-block in LDS);
+// or two (gate|up + mid, down + combine: the last workgroup to arrive at a block runs the next stage). The same bytes.
+enum MoeForm : int { kMoeFiveLaunches = 0, kMoeFourLaunches = 1, kMoeTwoLaunches = 2 };
+hipError_t launch_moe_decode(const MoeLaunch& a, int form, hipStream_t s);
 
 // The same call above the decode rows: route, prepare, gate|up GEMM, mid, down GEMM, combine. xg, xu, hd hold plain f16
 // here (quad order), zg, zu, zd one plane each, all by sorted position.
 hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s);
 // One dense projection above 32 rows: prepare (f16, quad order), the trellis GEMM, finish. xq holds plain f16; ks = 1.
 hipError_t launch_dense_prefill(const DenseLaunch& d, hipStream_t s);
+
+// The W_hat form's own stages: the prepare in natural order (plain f16 [rows][in], what a plain GEMM multiplies), and the
+// finish of an f16 z [rows][out].
+hipError_t launch_dense_prep_natural(const DenseLaunch& d, uint16_t* xp, hipStream_t s);
+hipError_t launch_dense_finish_half(const DenseLaunch& d, const uint16_t* z, hipStream_t s);
 
 // trellis [in/16][out/16][n] -> W_hat f16 [in][out], bit-exact (format.reconstructInner)
 hipError_t launch_dequant(const uint32_t* trellis, uint16_t* w_hat, uint32_t in, uint32_t out, uint32_t n,

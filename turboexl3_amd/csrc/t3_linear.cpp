@@ -91,6 +91,41 @@ void carve_dense_prefill(DenseCall* call, void* workspace) {
 
 constexpr uint32_t kGemvRowsMax = 32;
 
+// From dense_gemm_rows rows up (and with rocBLAS present) a dense call decodes W_hat once and multiplies plainly
+// (src/core/dense.zig:909-922,1290-1302): the decode is paid once a call, not once a 64-row item.
+bool takes_w_hat(const DenseLaunch& l) {
+    const int32_t from = config().dense_gemm_rows;
+    return from > 0 && l.rows >= static_cast<uint32_t>(from) && blas_available();
+}
+
+struct WhatScratch {
+    uint16_t* w_hat;  // f16 [in][out]
+    uint16_t* xp;     // f16 [rows][in], natural order
+    uint16_t* z;      // f16 [rows][out]
+};
+
+WhatScratch carve_dense_w_hat(DenseCall* call, void* workspace) {
+    DenseLaunch& l = call->launch;
+    Carver c(workspace);
+    l.arrive = c.take<uint32_t>(kCounterBytes);
+    WhatScratch w;
+    w.w_hat = c.take<uint16_t>(static_cast<size_t>(l.in) * l.out * 2u);
+    w.xp = c.take<uint16_t>(static_cast<size_t>(l.rows) * l.in * 2u);
+    w.z = c.take<uint16_t>(static_cast<size_t>(l.rows) * l.out * 2u);
+    call->workspace = c.used;
+    return w;
+}
+
+int32_t run_w_hat(const DenseCall& call, const WhatScratch& w, int codebook, hipStream_t s) {
+    const DenseLaunch& l = call.launch;
+    if (const int32_t st = hip_status(launch_dequant(l.trellis, w.w_hat, l.in, l.out, l.n, l.wbits, codebook, s));
+        st != T3_OK)
+        return st;
+    if (const int32_t st = hip_status(launch_dense_prep_natural(l, w.xp, s)); st != T3_OK) return st;
+    if (const int32_t st = blas_gemm_f16(s, w.xp, w.w_hat, w.z, l.rows, l.in, l.out); st != T3_OK) return st;
+    return hip_status(launch_dense_finish_half(l, w.z, s));
+}
+
 int32_t run_chain(const DenseCall& call, hipStream_t s, uint32_t stages) {
     if (stages & T3_STAGE_PREPARE)
         if (const int32_t st = hip_status(launch_dense_prep(call.launch, s)); st != T3_OK) return st;
@@ -122,7 +157,8 @@ int32_t t3_linear_workspace_bytes(const t3_array* x, const t3_array* trellis, t3
     if (!bytes) return T3_BadArgs;
     t3::DenseCall call;
     if (const int32_t st = t3::check_dense(x, trellis, nullptr, nullptr, dec, nullptr, 0, &call); st != T3_OK) return st;
-    if (call.launch.rows > t3::kGemvRowsMax) t3::carve_dense_prefill(&call, nullptr);
+    if (call.launch.rows > t3::kGemvRowsMax && t3::takes_w_hat(call.launch)) t3::carve_dense_w_hat(&call, nullptr);
+    else if (call.launch.rows > t3::kGemvRowsMax) t3::carve_dense_prefill(&call, nullptr);
     else t3::carve_dense(&call, nullptr);
     *bytes = call.workspace;
     return T3_OK;
@@ -155,6 +191,11 @@ int32_t t3_linear(t3_stream stream, const t3_array* x, const t3_array* trellis, 
     if (!workspace) return T3_BadArgs;
     if (call.launch.rows > t3::kGemvRowsMax) {
         if (!t3::config().prefill || call.launch.rows > 65535u) return T3_Exl3EngineNotImplemented;
+        if (t3::takes_w_hat(call.launch)) {
+            const t3::WhatScratch w = t3::carve_dense_w_hat(&call, workspace);
+            if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
+            return t3::run_w_hat(call, w, dec.codebook, static_cast<hipStream_t>(stream));
+        }
         // the trellis GEMM (the role of src/core/dense.zig:978-1034 and of dequant + matmul + finish, :909-922)
         t3::carve_dense_prefill(&call, workspace);
         if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;

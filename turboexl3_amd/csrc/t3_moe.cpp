@@ -135,7 +135,7 @@ void carve_moe(MoeCall* call, void* workspace) {
     MoeLaunch& l = call->launch;
     const size_t rkt = static_cast<size_t>(l.rows) * (l.topk + l.shared_slots);
     Carver c(workspace);
-    c.take<uint32_t>(kCounterBytes);
+    l.arrive = c.take<uint32_t>(kCounterBytes);
     l.xg = c.take<uint32_t>(rkt * l.hidden * 4u);
     l.xu = c.take<uint32_t>(rkt * l.hidden * 4u);
     l.hd = c.take<uint32_t>(rkt * l.inter * 4u);
@@ -204,8 +204,15 @@ int32_t run_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const 
     }
     carve_moe(&call, workspace);
     if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
-    const bool prepare_apart = config().decode_form == 3;
-    return hip_status(launch_moe_decode(call.launch, prepare_apart, static_cast<hipStream_t>(stream)));
+    // decode_form 3: the five-launch chain; 9: two launches while a counter a (row-slot, 128-block) fits the
+    // workspace's counter area, else four
+    const MoeLaunch& l = call.launch;
+    const size_t widest = (l.hidden > l.inter ? l.hidden : l.inter) / 128u;
+    const size_t counters = static_cast<size_t>(l.rows) * (l.topk + l.shared_slots) * widest;
+    const int form = config().decode_form == 3 ? kMoeFiveLaunches
+                     : config().decode_form == 4 || counters * 4u > kCounterBytes ? kMoeFourLaunches
+                                                                                   : kMoeTwoLaunches;
+    return hip_status(launch_moe_decode(l, form, static_cast<hipStream_t>(stream)));
 }
 
 }  // namespace

@@ -31,18 +31,27 @@ __global__ void __launch_bounds__(64) moe_prep(const MoeLaunch a) {
 // NPROJ 1: down, inter -> hidden. Wave sg of slice blockIdx.z takes K part 4 z + sg of `parts` (a part: `per` input
 // tiles). z[proj]: f32 [KS][RKT][out], the four waves' sums, wave 0 first. XLDS (gate|up only, per == 8): the wave
 // prepares its own 128-block of x in LDS.
-template <int CB, bool WIDE, int BT, int NPROJ, bool XLDS>
+//
+// ARRIVE: the launch also runs the stage after it. The planes are stored device-coherently, every workgroup counts
+// itself in at its 128-column block, and the last to arrive runs that block's next stage on the complete planes:
+// gate|up -> the slot's mid block (counter a (row-slot, block of inter)); down -> the row's combine block (counter a
+// (row, block of hidden); skipped slots count themselves in too). The statements are the chain's, so are the bytes.
+template <int CB, bool WIDE, int BT, int NPROJ, bool XLDS, bool ARRIVE>
 __global__ void __launch_bounds__(256) moe_gemv(const MoeLaunch a) {
+    // Two tile rows in flight a wave (measured: all 8 in flight is no faster; a call's time is its chain of dependent
+    // round trips, not the depth of one wave's ring)
     constexpr int ST = 2;
     constexpr uint32_t kStage = gemv_stage_bytes<BT>();
     constexpr uint32_t kRed = 4u * BT * 64u * 16u;
     constexpr uint32_t kMain = kRed > 4u * kStage ? kRed : 4u * kStage;
     __shared__ __attribute__((aligned(16))) unsigned char smem[kMain];
+    __shared__ uint32_t last_flag;
     float4v(*red)[BT * 64] = reinterpret_cast<float4v(*)[BT * 64]>(smem);
     const uint32_t blk = blockIdx.x, rk = blockIdx.y / NPROJ, proj = blockIdx.y % NPROJ, ksl = blockIdx.z;
     const uint32_t sg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
     const SlotRef s = resolve_slot(a, rk);
-    if (!s.live) return;  // uniform over the workgroup
+    // uniform over the workgroup; the down launch's arriving form still has to count a skipped slot in
+    if (!s.live && !(ARRIVE && NPROJ == 1)) return;
     const RoutedBank& bank = s.shared ? a.shared : a.bank;
     const uint32_t in = NPROJ == 2 ? a.hidden : a.inter, out = NPROJ == 2 ? a.inter : a.hidden;
     const uint32_t n = NPROJ == 2 ? a.n_gu : a.n_dn;
@@ -61,7 +70,7 @@ __global__ void __launch_bounds__(256) moe_gemv(const MoeLaunch a) {
 #pragma unroll
     for (int t = 0; t < BT; ++t) acc[0][t] = float4v{0.f, 0.f, 0.f, 0.f};
 
-    if (part < parts) {  // uniform over the wave; a wave past the last part adds zeros below
+    if (part < parts && s.live) {  // uniform over the wave; a wave past the last part adds zeros below
         uint32_t xoff[1];
         if constexpr (XLDS) {
             extern __shared__ __attribute__((aligned(16))) unsigned char xdyn[];
@@ -84,8 +93,11 @@ __global__ void __launch_bounds__(256) moe_gemv(const MoeLaunch a) {
                 }
                 // every column workgroup of the slot stores the same sum: a handful of plain stores, read by the
                 // next launch
-                if (a.defer && lane == 0u)
-                    (proj ? a.su : a.sg)[static_cast<size_t>(rk) * (a.hidden / 128u) + (tk0 >> 3) + b] = sum;
+                if (a.defer && lane == 0u) {
+                    float* at = (proj ? a.su : a.sg) + static_cast<size_t>(rk) * (a.hidden / 128u) + (tk0 >> 3) + b;
+                    if constexpr (ARRIVE) store_coherent(at, sum);
+                    else *at = sum;
+                }
             }
             for (uint32_t i = lane; i < kXldsRows * 16u; i += 64u)
                 *reinterpret_cast<uint32_t*>(xst + per * (kXldsRows * 64u) + i * 4u) = 0u;
@@ -111,7 +123,60 @@ __global__ void __launch_bounds__(256) moe_gemv(const MoeLaunch a) {
         if ((l & 15u) != 0u) continue;
         const float4v v = ((red[0][i] + red[1][i]) + red[2][i]) + red[3][i];
         float* dst = z + (static_cast<size_t>(ksl) * rkt + rk) * out + (blk * BT + t) * 16u + 4u * (l >> 4);
-        *reinterpret_cast<float4v*>(dst) = v;
+        if constexpr (ARRIVE) {
+            if (s.live)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) store_coherent(dst + c, v[c]);
+        } else {
+            *reinterpret_cast<float4v*>(dst) = v;
+        }
+    }
+
+    if constexpr (ARRIVE) {
+        constexpr uint32_t kShare = 8u / BT;  // workgroup columns a 128-column block
+        const uint32_t b128 = blk / kShare, kt = a.topk + a.shared_slots;
+        const uint32_t ks = NPROJ == 2 ? a.ks_gu : a.ks_dn;
+        const uint32_t counter = NPROJ == 2 ? rk * (a.inter / 128u) + b128 : s.row * (a.hidden / 128u) + b128;
+        const uint32_t full = NPROJ == 2 ? 2u * ks * kShare : kt * ks * kShare;
+        wait_stores();
+        __syncthreads();
+        if (threadIdx.x == 0u) {
+            const uint32_t before =
+                __hip_atomic_fetch_add(a.arrive + counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last_flag = before == full - 1u;
+        }
+        __syncthreads();
+        if (!last_flag) return;
+        if (threadIdx.x == 0u)  // zero again for the next call
+            __hip_atomic_store(a.arrive + counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if constexpr (NPROJ == 2) {
+            if (sg == 0u) routed_mid_block<false, true>(a, rk, rk, b128, lane);
+        } else {
+            // the slots' finishes four at a time, one a wave; wave 0 adds them in slot order
+            float(*fin)[128] = reinterpret_cast<float(*)[128]>(smem);
+            float acc2[2] = {0.0f, 0.0f};
+            for (uint32_t k0 = 0; k0 < kt; k0 += 4u) {
+                const uint32_t k = k0 + sg;
+                if (k < kt) {
+                    float v[2];
+                    if (routed_down_finish<true>(a, s.row * kt + k, s.row * kt + k, b128, lane, v, ks)) {
+                        fin[sg][lane] = v[0];
+                        fin[sg][lane + 64u] = v[1];
+                    }
+                }
+                __syncthreads();
+                if (sg == 0u)
+                    for (uint32_t w = 0; w < 4u && k0 + w < kt; ++w) {
+                        const SlotRef sw = resolve_slot(a, s.row * kt + k0 + w);
+                        if (!sw.live) continue;
+                        const float wgt = sw.shared ? 1.0f : score_of(a, s.row, k0 + w);
+                        acc2[0] = __builtin_fmaf(wgt, fin[w][lane], acc2[0]);
+                        acc2[1] = __builtin_fmaf(wgt, fin[w][lane + 64u], acc2[1]);
+                    }
+                __syncthreads();
+            }
+            if (sg == 0u) routed_store_row(a, s.row, b128, lane, acc2);
+        }
     }
 }
 
@@ -125,47 +190,56 @@ __global__ void __launch_bounds__(64) moe_combine(const MoeLaunch a) {
     routed_combine_block<false>(a, blockIdx.y, blockIdx.x, threadIdx.x);
 }
 
-template <int CB, bool WIDE, int NPROJ, bool XLDS>
+template <int CB, bool WIDE, int NPROJ, bool XLDS, bool ARRIVE>
 hipError_t launch_gemv_bt(const MoeLaunch& a, hipStream_t s) {
     const uint32_t out = NPROJ == 2 ? a.inter : a.hidden;
     const uint32_t bt = NPROJ == 2 ? a.bt_gu : a.bt_dn, ks = NPROJ == 2 ? a.ks_gu : a.ks_dn;
     const uint32_t rkt = a.rows * (a.topk + a.shared_slots);
     const dim3 grid((out / 16u) / bt, rkt * NPROJ, ks), block(256);
     const size_t dyn = XLDS ? 4u * (a.per_gu + 1u) * (kXldsRows * 64u) : 0u;
-    if (bt == 8u) hipLaunchKernelGGL((moe_gemv<CB, WIDE, 8, NPROJ, XLDS>), grid, block, dyn, s, a);
-    else hipLaunchKernelGGL((moe_gemv<CB, WIDE, 4, NPROJ, XLDS>), grid, block, dyn, s, a);
+    if (bt == 8u) hipLaunchKernelGGL((moe_gemv<CB, WIDE, 8, NPROJ, XLDS, ARRIVE>), grid, block, dyn, s, a);
+    else hipLaunchKernelGGL((moe_gemv<CB, WIDE, 4, NPROJ, XLDS, ARRIVE>), grid, block, dyn, s, a);
     return hipGetLastError();
 }
 
-template <int NPROJ, bool XLDS>
+template <int NPROJ, bool XLDS, bool ARRIVE>
 hipError_t launch_gemv_cb(const MoeLaunch& a, hipStream_t s) {
     const bool wide = quad_needs_wide(NPROJ == 2 ? a.n_gu : a.n_dn);
     switch (a.codebook) {
-        case kMul1: return wide ? launch_gemv_bt<kMul1, true, NPROJ, XLDS>(a, s) : launch_gemv_bt<kMul1, false, NPROJ, XLDS>(a, s);
-        case kMcg: return wide ? launch_gemv_bt<kMcg, true, NPROJ, XLDS>(a, s) : launch_gemv_bt<kMcg, false, NPROJ, XLDS>(a, s);
+        case kMul1:
+            return wide ? launch_gemv_bt<kMul1, true, NPROJ, XLDS, ARRIVE>(a, s)
+                        : launch_gemv_bt<kMul1, false, NPROJ, XLDS, ARRIVE>(a, s);
+        case kMcg:
+            return wide ? launch_gemv_bt<kMcg, true, NPROJ, XLDS, ARRIVE>(a, s)
+                        : launch_gemv_bt<kMcg, false, NPROJ, XLDS, ARRIVE>(a, s);
         case kMul1Defer:
-            return wide ? launch_gemv_bt<kMul1Defer, true, NPROJ, XLDS>(a, s)
-                        : launch_gemv_bt<kMul1Defer, false, NPROJ, XLDS>(a, s);
+            return wide ? launch_gemv_bt<kMul1Defer, true, NPROJ, XLDS, ARRIVE>(a, s)
+                        : launch_gemv_bt<kMul1Defer, false, NPROJ, XLDS, ARRIVE>(a, s);
         default:
-            return wide ? launch_gemv_bt<kMcgPair, true, NPROJ, XLDS>(a, s) : launch_gemv_bt<kMcgPair, false, NPROJ, XLDS>(a, s);
+            return wide ? launch_gemv_bt<kMcgPair, true, NPROJ, XLDS, ARRIVE>(a, s)
+                        : launch_gemv_bt<kMcgPair, false, NPROJ, XLDS, ARRIVE>(a, s);
     }
 }
 
 }  // namespace
 
-hipError_t launch_moe_decode(const MoeLaunch& a, bool prepare_apart, hipStream_t s) {
+hipError_t launch_moe_decode(const MoeLaunch& a, int form, hipStream_t s) {
     const uint32_t rkt = a.rows * (a.topk + a.shared_slots);
     hipError_t e;
-    if (prepare_apart) {
+    if (form == kMoeTwoLaunches) {
+        if ((e = launch_gemv_cb<2, true, true>(a, s)) != hipSuccess) return e;
+        return launch_gemv_cb<1, false, true>(a, s);
+    }
+    if (form == kMoeFiveLaunches) {
         hipLaunchKernelGGL(moe_prep, dim3(a.hidden / 128u, rkt), dim3(64), 0, s, a);
         if ((e = hipGetLastError()) != hipSuccess) return e;
-        if ((e = launch_gemv_cb<2, false>(a, s)) != hipSuccess) return e;
+        if ((e = launch_gemv_cb<2, false, false>(a, s)) != hipSuccess) return e;
     } else {
-        if ((e = launch_gemv_cb<2, true>(a, s)) != hipSuccess) return e;
+        if ((e = launch_gemv_cb<2, true, false>(a, s)) != hipSuccess) return e;
     }
     hipLaunchKernelGGL(moe_mid, dim3(a.inter / 128u, rkt), dim3(64), 0, s, a);
     if ((e = hipGetLastError()) != hipSuccess) return e;
-    if ((e = launch_gemv_cb<1, false>(a, s)) != hipSuccess) return e;
+    if ((e = launch_gemv_cb<1, false, false>(a, s)) != hipSuccess) return e;
     hipLaunchKernelGGL(moe_combine, dim3(a.hidden / 128u, a.rows), dim3(64), 0, s, a);
     return hipGetLastError();
 }

@@ -350,6 +350,31 @@ __global__ void __launch_bounds__(64) pf_dense_prep(const void* x, const uint16_
     if (lane == 0u) xs[static_cast<size_t>(row) * nb + b] = sum;
 }
 
+// grid (in / 128 * rows), 64 threads: plain f16 in natural order, for a plain GEMM
+__global__ void __launch_bounds__(64) pf_dense_prep_natural(const void* x, const uint16_t* suh, uint16_t* xp,
+                                                            uint32_t in, int dt) {
+    const uint32_t nb = in / 128u, row = blockIdx.x / nb, b = blockIdx.x % nb, lane = threadIdx.x;
+    uint32_t hv[2];
+    float sum;
+    prep_values(dt, x, suh, in, row, b, lane, hv, sum);
+#pragma unroll
+    for (uint32_t j = 0; j < 2u; ++j)
+        xp[static_cast<size_t>(row) * in + b * 128u + lane + 64u * j] = static_cast<uint16_t>(hv[j]);
+}
+
+// grid (out / 128 * rows), 64 threads: the finish of z already rounded to f16 (format.innerGemv's rounding point)
+__global__ void __launch_bounds__(64) pf_dense_finish_half(const uint16_t* z, const uint16_t* svh, void* y,
+                                                           uint32_t out, int dt) {
+    const uint32_t nb = out / 128u, row = blockIdx.x / nb, b = blockIdx.x % nb, lane = threadIdx.x;
+    float v[2];
+#pragma unroll
+    for (uint32_t j = 0; j < 2u; ++j) v[j] = half_value(z[static_cast<size_t>(row) * out + b * 128u + lane + 64u * j]);
+    finish_values(v, svh, b, lane);
+#pragma unroll
+    for (uint32_t j = 0; j < 2u; ++j)
+        store_act_rt(dt, y, static_cast<size_t>(row) * out + b * 128u + lane + 64u * j, v[j]);
+}
+
 template <int CB, bool WIDE>
 hipError_t launch_gemm_rb(const PfGemm& g, uint32_t max_items, uint32_t nproj, uint32_t item_rows, hipStream_t s) {
     const dim3 grid(8u * g.nblk * ((max_items + 7u) / 8u), nproj), block(256);
@@ -428,6 +453,18 @@ hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s) {
     if ((e = launch_gemm(g, a.codebook, a.max_items, 1u, a.item_rows, s)) != hipSuccess) return e;
 
     hipLaunchKernelGGL(pf_combine, dim3(a.rows * (a.hidden / 128u)), dim3(64), 0, s, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_dense_prep_natural(const DenseLaunch& d, uint16_t* xp, hipStream_t s) {
+    hipLaunchKernelGGL(pf_dense_prep_natural, dim3(d.rows * (d.in / 128u)), dim3(64), 0, s, d.x, d.suh, xp, d.in,
+                       d.dtype);
+    return hipGetLastError();
+}
+
+hipError_t launch_dense_finish_half(const DenseLaunch& d, const uint16_t* z, hipStream_t s) {
+    hipLaunchKernelGGL(pf_dense_finish_half, dim3(d.rows * (d.out / 128u)), dim3(64), 0, s, z, d.svh, d.y, d.out,
+                       d.dtype);
     return hipGetLastError();
 }
 

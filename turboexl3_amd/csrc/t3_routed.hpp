@@ -40,21 +40,23 @@ __device__ __forceinline__ float score_of(const MoeLaunch& a, uint32_t row, uint
 }
 
 // One block's sums over the K slices (slice order; the first plane starts the sum) and the deferred MUL1 map.
+// COH: the planes and block sums were stored by other workgroups of this launch.
+template <bool COH>
 __device__ __forceinline__ void plane_sums(const float* z, size_t planes_stride, uint32_t ks, const float* bsum,
                                            uint32_t nb, int defer, uint32_t lane, float (&s)[2]) {
+    auto get = [](const float* p) { return COH ? load_coherent(p) : *p; };
 #pragma unroll
-    for (uint32_t j = 0; j < 2u; ++j) s[j] = z[lane + 64u * j];
+    for (uint32_t j = 0; j < 2u; ++j) s[j] = get(z + lane + 64u * j);
     for (uint32_t k = 1; k < ks; ++k)
 #pragma unroll
-        for (uint32_t j = 0; j < 2u; ++j) s[j] += z[k * planes_stride + lane + 64u * j];
+        for (uint32_t j = 0; j < 2u; ++j) s[j] += get(z + k * planes_stride + lane + 64u * j);
     if (defer) {
         float xsum = 0.0f;
-        for (uint32_t q = 0; q < nb; ++q) xsum += bsum[q];
+        for (uint32_t q = 0; q < nb; ++q) xsum += get(bsum + q);
 #pragma unroll
         for (uint32_t j = 0; j < 2u; ++j) s[j] = __builtin_fmaf(s[j], mul1_a(), mul1_b() * xsum);
     }
 }
-
 
 // ---- the routed chain's per-block stages ----------------------------------------------------------------------
 // One wave a 128-block. rk: the row-slot; q: where its scratch lives (decode rows: q = rk; prefill: its position in
@@ -91,7 +93,7 @@ __device__ __forceinline__ void routed_prep_block(const MoeLaunch& a, uint32_t r
 
 // gate and up finishes, the (clamped) SwiGLU in f32 on their f16 values, and the down's prepare: hd [.][inter],
 // hs f32 [.][inter / 128]
-template <bool PF>
+template <bool PF, bool COH = false>
 __device__ __forceinline__ void routed_mid_block(const MoeLaunch& a, uint32_t rk, uint32_t q, uint32_t b,
                                                  uint32_t lane) {
     const SlotRef s = resolve_slot(a, rk);
@@ -101,8 +103,8 @@ __device__ __forceinline__ void routed_mid_block(const MoeLaunch& a, uint32_t rk
     const uint32_t ks = PF ? 1u : a.ks_gu;
     const size_t plane = static_cast<size_t>(rkt) * a.inter, at = static_cast<size_t>(q) * a.inter + b * 128u;
     float g[2], u[2];
-    plane_sums(a.zg + at, plane, ks, a.sg + static_cast<size_t>(q) * nb, nb, a.defer, lane, g);
-    plane_sums(a.zu + at, plane, ks, a.su + static_cast<size_t>(q) * nb, nb, a.defer, lane, u);
+    plane_sums<COH>(a.zg + at, plane, ks, a.sg + static_cast<size_t>(q) * nb, nb, a.defer, lane, g);
+    plane_sums<COH>(a.zu + at, plane, ks, a.su + static_cast<size_t>(q) * nb, nb, a.defer, lane, u);
     finish_values(g, bank.gate_svh + static_cast<size_t>(s.e) * a.inter, b, lane);
     finish_values(u, bank.up_svh + static_cast<size_t>(s.e) * a.inter, b, lane);
     float d[2];
@@ -129,32 +131,41 @@ __device__ __forceinline__ void routed_mid_block(const MoeLaunch& a, uint32_t rk
     if (lane == 0u) a.hs[static_cast<size_t>(q) * (a.inter / 128u) + b] = sum;
 }
 
-// every slot's down finish of block b of one row, then the score-weighted sum in slot order
-template <bool PF>
-__device__ __forceinline__ void routed_combine_block(const MoeLaunch& a, uint32_t row, uint32_t b, uint32_t lane) {
-    const uint32_t kt = a.topk + a.shared_slots, rkt = a.rows * kt, nbi = a.inter / 128u;
-    const uint32_t ks = PF ? 1u : a.ks_dn;
+// One slot's finished down outputs of block b (f16-valued), false for a skipped slot. COH: only the planes cross
+// workgroups inside the launch; the block sums hs came from the launch before.
+template <bool COH>
+__device__ __forceinline__ bool routed_down_finish(const MoeLaunch& a, uint32_t rk, uint32_t q, uint32_t b,
+                                                   uint32_t lane, float (&v)[2], uint32_t ks) {
+    const SlotRef s = resolve_slot(a, rk);
+    if (!s.live) return false;  // uniform over the wave
+    const uint32_t rkt = a.rows * (a.topk + a.shared_slots), nbi = a.inter / 128u;
+    const RoutedBank& bank = s.shared ? a.shared : a.bank;
+    const float* z = a.zd + static_cast<size_t>(q) * a.hidden + b * 128u;
     const size_t plane = static_cast<size_t>(rkt) * a.hidden;
-    float acc[2] = {0.0f, 0.0f};
-    for (uint32_t k = 0; k < kt; ++k) {
-        const uint32_t rk = row * kt + k;
-        const SlotRef s = resolve_slot(a, rk);
-        if (!s.live) continue;  // uniform over the wave
-        const uint32_t q = PF ? a.inv[rk] : rk;
-        const RoutedBank& bank = s.shared ? a.shared : a.bank;
-        float v[2];
-        plane_sums(a.zd + static_cast<size_t>(q) * a.hidden + b * 128u, plane, ks, a.hs + static_cast<size_t>(q) * nbi,
-                   nbi, a.defer, lane, v);
-        finish_values(v, bank.down_svh + static_cast<size_t>(s.e) * a.hidden, b, lane);
-        const float w = s.shared ? 1.0f : score_of(a, row, k);
+    auto get = [](const float* p) { return COH ? load_coherent(p) : *p; };
 #pragma unroll
-        for (uint32_t j = 0; j < 2u; ++j) acc[j] = __builtin_fmaf(w, v[j], acc[j]);
+    for (uint32_t j = 0; j < 2u; ++j) v[j] = get(z + lane + 64u * j);
+    for (uint32_t k = 1; k < ks; ++k)
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j) v[j] += get(z + k * plane + lane + 64u * j);
+    if (a.defer) {
+        float xsum = 0.0f;
+        for (uint32_t i = 0; i < nbi; ++i) xsum += a.hs[static_cast<size_t>(q) * nbi + i];
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j) v[j] = __builtin_fmaf(v[j], mul1_a(), mul1_b() * xsum);
     }
+    finish_values(v, bank.down_svh + static_cast<size_t>(s.e) * a.hidden, b, lane);
+    return true;
+}
+
+// a row's block b from its f32 sums: y's dtype, or `moeWithShared`'s two roundings
+__device__ __forceinline__ void routed_store_row(const MoeLaunch& a, uint32_t row, uint32_t b, uint32_t lane,
+                                                 const float (&acc)[2]) {
 #pragma unroll
     for (uint32_t j = 0; j < 2u; ++j) {
         const size_t o = static_cast<size_t>(row) * a.hidden + b * 128u + lane + 64u * j;
         if (a.shared_add) {
-            // `moeWithShared`: the routed output rounds to x's dtype, then the add rounds again (src/root.zig:976-984)
+            // the routed output rounds to x's dtype, then the add rounds again (src/root.zig:976-984)
             float r = acc[j];
             if (a.dtype == kF16) r = round_half(r);
             else if (a.dtype == kBf16) r = bf16_value(bf16_bits(r));
@@ -163,6 +174,24 @@ __device__ __forceinline__ void routed_combine_block(const MoeLaunch& a, uint32_
             store_act_rt(a.dtype, a.y, o, acc[j]);
         }
     }
+}
+
+// every slot's down finish of block b of one row, then the score-weighted sum in slot order
+template <bool PF>
+__device__ __forceinline__ void routed_combine_block(const MoeLaunch& a, uint32_t row, uint32_t b, uint32_t lane) {
+    const uint32_t kt = a.topk + a.shared_slots;
+    float acc[2] = {0.0f, 0.0f};
+    for (uint32_t k = 0; k < kt; ++k) {
+        const uint32_t rk = row * kt + k;
+        const SlotRef s = resolve_slot(a, rk);
+        if (!s.live) continue;  // uniform over the wave
+        float v[2];
+        routed_down_finish<false>(a, rk, PF ? a.inv[rk] : rk, b, lane, v, PF ? 1u : a.ks_dn);
+        const float w = s.shared ? 1.0f : score_of(a, row, k);
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j) acc[j] = __builtin_fmaf(w, v[j], acc[j]);
+    }
+    routed_store_row(a, row, b, lane, acc);
 }
 
 }  // namespace t3
