@@ -190,7 +190,7 @@ int32_t t3_linear(t3_stream stream, const t3_array* x, const t3_array* trellis, 
     if (const int32_t st = t3::check_dense(x, trellis, suh, svh, dec, y, 0, &call); st != T3_OK) return st;
     if (!workspace) return T3_BadArgs;
     if (call.launch.rows > t3::kGemvRowsMax) {
-        if (!t3::config().prefill || call.launch.rows > 65535u) return T3_Exl3EngineNotImplemented;
+        if (!t3::config().prefill) return T3_Exl3EngineNotImplemented;
         if (t3::takes_w_hat(call.launch)) {
             const t3::WhatScratch w = t3::carve_dense_w_hat(&call, workspace);
             if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;

@@ -21,10 +21,10 @@
 namespace t3 {
 namespace {
 
-constexpr uint32_t kPfTiles = 4;           // adjacent tiles a wave (a tile row's chunk: 4 * 2n <= 1 KB)
 constexpr uint32_t kPfSlot = 256;          // LDS bytes a staged tile
 constexpr uint32_t kPfRowStride = 80;      // LDS bytes an activation row a step: 64 + 16 so 16 rows hit 16 bank groups
-constexpr uint32_t kPfWStage = 2u * kPfTiles * kPfSlot + 1024u;  // two tile rows, then the dump of the idle lanes
+// a wave's stage: two tile rows of NT tiles, then the dump of the idle lanes
+constexpr uint32_t pf_stage_bytes(uint32_t nt) { return 2u * nt * kPfSlot + 1024u; }
 
 struct PfGemm {
     const uint32_t* w[2];    // the bank's trellis a projection (gate, up) or (down, -)
@@ -33,7 +33,7 @@ struct PfGemm {
     float* z[2];             // f32 [positions][out]
     const uint32_t* items;   // {expert, first position, rows, 0} an item; null: dense, item i = rows i RB 16 ...
     const uint32_t* n_items; // the route's item count (device)
-    uint32_t in, out, n, wbits, positions, experts, nblk;
+    uint32_t in, out, n, wbits, positions, experts, nblk;  // nblk: workgroup columns (64 NT output columns each)
 };
 
 // The weight a GEMM feeds the matrix core as one f16: exact, or MUL1's h = 1024 + t when its map is deferred.
@@ -43,11 +43,39 @@ __device__ __forceinline__ uint32_t weight_half(uint32_t cw) {
     else return static_cast<uint32_t>(decode_exact<CB>(cw));
 }
 
+// Two weights as the two halves of one register. MCG: each weight is one f16 add of its hashed pair's halves, and the
+// sub-dword forms of v_add_f16 write the low half, then the high half of the same register (the plain form costs a
+// third instruction to merge them).
+template <int CB>
+__device__ __forceinline__ uint32_t weight_halves(uint32_t cw_lo, uint32_t cw_hi) {
+    if constexpr (CB == kMcg) {
+        const uint32_t pa = mcg_pair(cw_lo), pb = mcg_pair(cw_hi);
+        uint32_t d;
+        asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1"
+            : "=v"(d)
+            : "v"(pa));
+        asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1"
+            : "+v"(d)
+            : "v"(pb));
+        return d;
+    } else {
+        return weight_half<CB>(cw_lo) | (weight_half<CB>(cw_hi) << 16);
+    }
+}
+
 // Grid (8 * nblk * ceil(max_items / 8), projections), 256 threads. Consecutive workgroup ids go round the eight dies,
 // so the workgroups that share an item's activations (its nblk column blocks) are given ids 8 apart: one die's L2
 // serves them all.
-template <int CB, bool WIDE, int RB>
+//
+// Shapes: RB 16-row blocks an item and NT adjacent tiles a wave, 64 NT columns a workgroup. (4, 4): 64 rows. (8, 4):
+// 128 rows: a decoded weight feeds twice the MFMAs, and an expert with 65-128 rows stays one item (a second, short
+// item would pay the whole decode again). (2, 4): 32 rows for sparse routings. Row blocks past the item's last row
+// skip their MFMAs. (Measured: (8, 2) gains nothing over (4, 4): halving NT doubles the LDS and L2 traffic of the
+// activations a flop.)
+template <int CB, bool WIDE, int RB, int NT>
 __global__ void __launch_bounds__(256) pf_gemm(const PfGemm a) {
+    constexpr uint32_t kPfTiles = NT;
+    constexpr uint32_t kPfWStage = pf_stage_bytes(NT);
     constexpr uint32_t BM = RB * 16u;
     constexpr uint32_t kABuf = BM * kPfRowStride;
     constexpr uint32_t kPieces = BM * 4u;                      // 16-byte pieces of an item's rows a step
@@ -72,7 +100,7 @@ __global__ void __launch_bounds__(256) pf_gemm(const PfGemm a) {
     const bool from_shared = e >= a.experts;
     const uint32_t* wmat = (from_shared ? a.ws[proj] : a.w[proj]) +
                            static_cast<size_t>(from_shared ? e - a.experts : e) * in_tiles * out_tiles * nw;
-    const uint32_t col0 = blk * 16u + wave * kPfTiles;  // the wave's first tile column
+    const uint32_t col0 = (blk * 4u + wave) * kPfTiles;  // the wave's first tile column
     const bool active = col0 < out_tiles;               // uniform over the wave (out is a multiple of 128, not of 256)
     const uint32_t wstep = out_tiles * nw * 4u;
     const uint32_t tile_bytes = 2u * a.n, chunk_bytes = kPfTiles * tile_bytes;
@@ -149,78 +177,107 @@ __global__ void __launch_bounds__(256) pf_gemm(const PfGemm a) {
             }
     };
 
-    float4v acc[RB][kPfTiles];
-#pragma unroll
-    for (int mb = 0; mb < RB; ++mb)
-#pragma unroll
-        for (uint32_t t = 0; t < kPfTiles; ++t) acc[mb][t] = float4v{0.f, 0.f, 0.f, 0.f};
+    const uint32_t steps = in_tiles >> 1;  // even: in is a multiple of 128
+    float* z = a.z[proj];
 
-    // one step: K = 32 = tile rows 2 step and 2 step + 1
-    auto compute = [&](const QuadWords<WIDE>(&wd)[2][kPfTiles], uint32_t parity) {
-        uint4v bf[RB];
+    // The K loop and the stores for an item of LB live 16-row blocks: no branch inside the loop.
+    auto run = [&]<int LB>() {
+        float4v acc[LB][kPfTiles];
 #pragma unroll
-        for (int mb = 0; mb < RB; ++mb)
-            bf[mb] = *reinterpret_cast<const uint4v*>(abuf + parity * kABuf +
-                                                      (static_cast<uint32_t>(mb) * 16u + (lane & 15u)) * kPfRowStride +
-                                                      (lane >> 4) * 16u);
+        for (int mb = 0; mb < LB; ++mb)
 #pragma unroll
-        for (uint32_t t = 0; t < kPfTiles; ++t) {
-            uint32_t c0[4], c1[4];
-            quad_codewords<WIDE>(wd[0][t], plan, a.wbits, c0);
-            quad_codewords<WIDE>(wd[1][t], plan, a.wbits, c1);
-            uint4v af;
-            af[0] = weight_half<CB>(c0[0]) | (weight_half<CB>(c0[1]) << 16);
-            af[1] = weight_half<CB>(c0[2]) | (weight_half<CB>(c0[3]) << 16);
-            af[2] = weight_half<CB>(c1[0]) | (weight_half<CB>(c1[1]) << 16);
-            af[3] = weight_half<CB>(c1[2]) | (weight_half<CB>(c1[3]) << 16);
+            for (uint32_t t = 0; t < kPfTiles; ++t) acc[mb][t] = float4v{0.f, 0.f, 0.f, 0.f};
+
+        // one step: K = 32 = tile rows 2 step and 2 step + 1
+        auto compute = [&](const QuadWords<WIDE>(&wd)[2][kPfTiles], uint32_t parity) {
+            uint4v bf[LB];
 #pragma unroll
-            for (int mb = 0; mb < RB; ++mb)
-                acc[mb][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, af),
-                                                                    __builtin_bit_cast(half8, bf[mb]), acc[mb][t], 0, 0, 0);
+            for (int mb = 0; mb < LB; ++mb)
+                bf[mb] = *reinterpret_cast<const uint4v*>(abuf + parity * kABuf +
+                                                          (static_cast<uint32_t>(mb) * 16u + (lane & 15u)) * kPfRowStride +
+                                                          (lane >> 4) * 16u);
+#pragma unroll
+            for (uint32_t t = 0; t < kPfTiles; ++t) {
+                uint32_t c0[4], c1[4];
+                quad_codewords<WIDE>(wd[0][t], plan, a.wbits, c0);
+                quad_codewords<WIDE>(wd[1][t], plan, a.wbits, c1);
+                uint4v af;
+                af[0] = weight_halves<CB>(c0[0], c0[1]);
+                af[1] = weight_halves<CB>(c0[2], c0[3]);
+                af[2] = weight_halves<CB>(c1[0], c1[1]);
+                af[3] = weight_halves<CB>(c1[2], c1[3]);
+#pragma unroll
+                for (int mb = 0; mb < LB; ++mb)
+                    acc[mb][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                        __builtin_bit_cast(half8, af), __builtin_bit_cast(half8, bf[mb]), acc[mb][t], 0, 0, 0);
+            }
+        };
+
+        uint4v wreg[2], areg[kALoads];
+        QuadWords<WIDE> wd0[2][kPfTiles], wd1[2][kPfTiles];
+        load_w(0u, wreg);
+        load_a(0u, areg);
+        put_a(areg, 0u);
+        stage_w(wreg);
+        fetch_w(wd0);
+        load_w(1u, wreg);
+        load_a(1u, areg);
+        __syncthreads();
+        for (uint32_t s = 0; s < steps; s += 2u) {
+            // even step: words in wd0, activations in buffer 0; wreg / areg hold step s + 1
+            stage_w(wreg);
+            load_w(s + 2u, wreg);
+            fetch_w(wd1);
+            compute(wd0, 0u);
+            put_a(areg, 1u);
+            load_a(s + 2u, areg);
+            __syncthreads();
+            // odd step
+            stage_w(wreg);
+            load_w(s + 3u, wreg);
+            fetch_w(wd0);
+            compute(wd1, 1u);
+            put_a(areg, 0u);
+            load_a(s + 3u, areg);
+            __syncthreads();
+        }
+
+        if (!active) return;
+        // D[i][j]: i = the weight's column inside its tile (this lane: 4 (lane / 16) .. + 3), j = activation row
+        // lane % 16
+#pragma unroll
+        for (int mb = 0; mb < LB; ++mb) {
+            const uint32_t row = static_cast<uint32_t>(mb) * 16u + (lane & 15u);
+            if (row >= count) continue;
+#pragma unroll
+            for (uint32_t t = 0; t < kPfTiles; ++t)
+                *reinterpret_cast<float4v*>(z + static_cast<size_t>(first + row) * a.out + (col0 + t) * 16u +
+                                            4u * (lane >> 4)) = acc[mb][t];
         }
     };
 
-    const uint32_t steps = in_tiles >> 1;  // even: in is a multiple of 128
-    uint4v wreg[2], areg[kALoads];
-    QuadWords<WIDE> wd0[2][kPfTiles], wd1[2][kPfTiles];
-    load_w(0u, wreg);
-    load_a(0u, areg);
-    put_a(areg, 0u);
-    stage_w(wreg);
-    fetch_w(wd0);
-    load_w(1u, wreg);
-    load_a(1u, areg);
-    __syncthreads();
-    for (uint32_t s = 0; s < steps; s += 2u) {
-        // even step: words in wd0, activations in buffer 0; wreg / areg hold step s + 1
-        stage_w(wreg);
-        load_w(s + 2u, wreg);
-        fetch_w(wd1);
-        compute(wd0, 0u);
-        put_a(areg, 1u);
-        load_a(s + 2u, areg);
-        __syncthreads();
-        // odd step
-        stage_w(wreg);
-        load_w(s + 3u, wreg);
-        fetch_w(wd0);
-        compute(wd1, 1u);
-        put_a(areg, 0u);
-        load_a(s + 3u, areg);
-        __syncthreads();
-    }
-
-    if (!active) return;
-    // D[i][j]: i = the weight's column inside its tile (this lane: 4 (lane / 16) .. + 3), j = activation row lane % 16
-    float* z = a.z[proj];
-#pragma unroll
-    for (int mb = 0; mb < RB; ++mb) {
-        const uint32_t row = static_cast<uint32_t>(mb) * 16u + (lane & 15u);
-        if (row >= count) continue;
-#pragma unroll
-        for (uint32_t t = 0; t < kPfTiles; ++t)
-            *reinterpret_cast<float4v*>(z + static_cast<size_t>(first + row) * a.out + (col0 + t) * 16u + 4u * (lane >> 4)) =
-                acc[mb][t];
+    const uint32_t live_blocks = (count + 15u) >> 4;  // uniform over the workgroup
+    if constexpr (RB == 2) {
+        if (live_blocks <= 1u) run.template operator()<1>();
+        else run.template operator()<2>();
+    } else if constexpr (RB == 4) {
+        switch (live_blocks) {
+            case 1: run.template operator()<1>(); break;
+            case 2: run.template operator()<2>(); break;
+            case 3: run.template operator()<3>(); break;
+            default: run.template operator()<4>(); break;
+        }
+    } else {
+        switch (live_blocks) {
+            case 1: run.template operator()<1>(); break;
+            case 2: run.template operator()<2>(); break;
+            case 3: run.template operator()<3>(); break;
+            case 4: run.template operator()<4>(); break;
+            case 5: run.template operator()<5>(); break;
+            case 6: run.template operator()<6>(); break;
+            case 7: run.template operator()<7>(); break;
+            default: run.template operator()<8>(); break;
+        }
     }
 }
 
@@ -315,71 +372,258 @@ __global__ void __launch_bounds__(256) pf_place(const MoeLaunch a) {
     a.inv[rk] = q;
 }
 
-// ---- the routed chain's stages by sorted position: grid (blocks * positions), 64 threads -------------------------
+// ---- the chains' stages around the GEMM -----------------------------------------------------------------------
+// One wave takes kPfUnit adjacent 128-blocks of one row (or sorted position) and issues every load of all of them
+// before the first transform: a block is 256 bytes a load instruction, so one block a wave leaves the memory system
+// almost idle (measured: 1.8 TB/s). Four waves a workgroup; grid ceil(units / 4). The arithmetic of a block is
+// that of t3_stages.hpp, statement for statement.
 
-__global__ void __launch_bounds__(64) pf_prep(const MoeLaunch a) {
-    const uint32_t nb = a.hidden / 128u, q = blockIdx.x / nb, b = blockIdx.x % nb;
+constexpr uint32_t kPfUnit = 4;
+
+__device__ __forceinline__ uint32_t wave_unit() { return blockIdx.x * 4u + (threadIdx.x >> 6); }
+
+template <int DT>
+__global__ void __launch_bounds__(256) pf_prep(const MoeLaunch a) {
+    const uint32_t nb = a.hidden / 128u, groups = (nb + kPfUnit - 1u) / kPfUnit;
+    const uint32_t u0 = wave_unit(), q = u0 / groups, b0 = (u0 % groups) * kPfUnit, lane = threadIdx.x & 63u;
     if (q >= a.counts[a.bank.experts + a.shared_slots + 1u]) return;
-    routed_prep_block<true>(a, a.order[q], q, b, threadIdx.x);
-}
-
-__global__ void __launch_bounds__(64) pf_mid(const MoeLaunch a) {
-    const uint32_t nb = a.inter / 128u, q = blockIdx.x / nb, b = blockIdx.x % nb;
-    if (q >= a.counts[a.bank.experts + a.shared_slots + 1u]) return;
-    routed_mid_block<true>(a, a.order[q], q, b, threadIdx.x);
-}
-
-__global__ void __launch_bounds__(64) pf_combine(const MoeLaunch a) {
-    const uint32_t nb = a.hidden / 128u;
-    routed_combine_block<true>(a, blockIdx.x / nb, blockIdx.x % nb, threadIdx.x);
-}
-
-// ---- dense prepare: grid (in / 128 * rows), 64 threads: plain f16 in quad order, block sums ----------------------
-
-__global__ void __launch_bounds__(64) pf_dense_prep(const void* x, const uint16_t* suh, uint16_t* xq, float* xs,
-                                                    uint32_t in, int dt) {
-    const uint32_t nb = in / 128u, row = blockIdx.x / nb, b = blockIdx.x % nb, lane = threadIdx.x;
-    uint32_t hv[2];
-    float sum;
-    prep_values(dt, x, suh, in, row, b, lane, hv, sum);
+    const SlotRef s = resolve_slot(a, a.order[q]);
+    const RoutedBank& bank = s.shared ? a.shared : a.bank;
+    const uint16_t* gs = bank.gate_suh + static_cast<size_t>(s.e) * a.hidden;
+    const uint16_t* us = bank.up_suh + static_cast<size_t>(s.e) * a.hidden;
+    float xv[kPfUnit][2], g[kPfUnit][2], up[kPfUnit][2];
 #pragma unroll
-    for (uint32_t j = 0; j < 2u; ++j) {
-        const uint32_t i = b * 128u + lane + 64u * j;
-        xq[static_cast<size_t>(row) * in + (i & ~15u) + quad_slot(i & 15u)] = static_cast<uint16_t>(hv[j]);
+    for (uint32_t u = 0; u < kPfUnit; ++u)
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j) {
+            const uint32_t b = b0 + u < nb ? b0 + u : nb - 1u, i = b * 128u + lane + 64u * j;
+            xv[u][j] = round_half(load_act<DT>(a.x, static_cast<size_t>(s.row) * a.hidden + i));
+            g[u][j] = half_value(gs[i]);
+            up[u][j] = half_value(us[i]);
+        }
+#pragma unroll
+    for (uint32_t u = 0; u < kPfUnit; ++u) {
+        if (b0 + u >= nb) break;
+#pragma unroll
+        for (uint32_t proj = 0; proj < 2u; ++proj) {
+            float v[2] = {xv[u][0] * (proj ? up[u][0] : g[u][0]), xv[u][1] * (proj ? up[u][1] : g[u][1])};
+            uint32_t hv[2];
+            float sum;
+            prep_core(v, lane, hv, sum);
+#pragma unroll
+            for (uint32_t j = 0; j < 2u; ++j)
+                store_prepared<true>(proj ? a.xu : a.xg, static_cast<size_t>(q) * a.hidden,
+                                     (b0 + u) * 128u + lane + 64u * j, hv[j]);
+            if (lane == 0u) (proj ? a.su : a.sg)[static_cast<size_t>(q) * nb + b0 + u] = sum;
+        }
     }
-    if (lane == 0u) xs[static_cast<size_t>(row) * nb + b] = sum;
 }
 
-// grid (in / 128 * rows), 64 threads: plain f16 in natural order, for a plain GEMM
-__global__ void __launch_bounds__(64) pf_dense_prep_natural(const void* x, const uint16_t* suh, uint16_t* xp,
-                                                            uint32_t in, int dt) {
-    const uint32_t nb = in / 128u, row = blockIdx.x / nb, b = blockIdx.x % nb, lane = threadIdx.x;
-    uint32_t hv[2];
-    float sum;
-    prep_values(dt, x, suh, in, row, b, lane, hv, sum);
+// gate and up finishes, the (clamped) SwiGLU, the down's prepare (routed_mid_block's statements)
+__global__ void __launch_bounds__(256) pf_mid(const MoeLaunch a) {
+    const uint32_t nb = a.inter / 128u, nbh = a.hidden / 128u, groups = (nb + kPfUnit - 1u) / kPfUnit;
+    const uint32_t u0 = wave_unit(), q = u0 / groups, b0 = (u0 % groups) * kPfUnit, lane = threadIdx.x & 63u;
+    if (q >= a.counts[a.bank.experts + a.shared_slots + 1u]) return;
+    const SlotRef s = resolve_slot(a, a.order[q]);
+    const RoutedBank& bank = s.shared ? a.shared : a.bank;
+    const size_t eo = static_cast<size_t>(s.e) * a.inter, qo = static_cast<size_t>(q) * a.inter;
+    float zg[kPfUnit][2], zu[kPfUnit][2], svg[kPfUnit][2], svu[kPfUnit][2], sdn[kPfUnit][2];
 #pragma unroll
-    for (uint32_t j = 0; j < 2u; ++j)
-        xp[static_cast<size_t>(row) * in + b * 128u + lane + 64u * j] = static_cast<uint16_t>(hv[j]);
+    for (uint32_t u = 0; u < kPfUnit; ++u)
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j) {
+            const uint32_t b = b0 + u < nb ? b0 + u : nb - 1u, i = b * 128u + lane + 64u * j;
+            zg[u][j] = a.zg[qo + i];
+            zu[u][j] = a.zu[qo + i];
+            svg[u][j] = half_value(bank.gate_svh[eo + i]);
+            svu[u][j] = half_value(bank.up_svh[eo + i]);
+            sdn[u][j] = half_value(bank.down_suh[eo + i]);
+        }
+    float xg = 0.0f, xu = 0.0f;
+    if (a.defer)
+        for (uint32_t t = 0; t < nbh; ++t) {
+            xg += a.sg[static_cast<size_t>(q) * nbh + t];
+            xu += a.su[static_cast<size_t>(q) * nbh + t];
+        }
+#pragma unroll
+    for (uint32_t u = 0; u < kPfUnit; ++u) {
+        if (b0 + u >= nb) break;
+        float g[2] = {zg[u][0], zg[u][1]}, up[2] = {zu[u][0], zu[u][1]};
+        if (a.defer)
+#pragma unroll
+            for (uint32_t j = 0; j < 2u; ++j) {
+                g[j] = __builtin_fmaf(g[j], mul1_a(), mul1_b() * xg);
+                up[j] = __builtin_fmaf(up[j], mul1_a(), mul1_b() * xu);
+            }
+        finish_core(g, svg[u], lane);
+        finish_core(up, svu[u], lane);
+        float d[2];
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j) {
+            float gv = g[j], uv = up[j];
+            if (a.limit > 0.0f) {  // comparisons: a NaN passes through (ref.zig:132-140)
+                gv = gv > a.limit ? a.limit : gv;
+                uv = uv > a.limit ? a.limit : (uv < -a.limit ? -a.limit : uv);
+            }
+            d[j] = round_half((gv / (1.0f + expf(-gv))) * uv) * sdn[u][j];
+        }
+        uint32_t hv[2];
+        float sum;
+        prep_core(d, lane, hv, sum);
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j) store_prepared<true>(a.hd, qo, (b0 + u) * 128u + lane + 64u * j, hv[j]);
+        if (lane == 0u) a.hs[static_cast<size_t>(q) * nb + b0 + u] = sum;
+    }
 }
 
-// grid (out / 128 * rows), 64 threads: the finish of z already rounded to f16 (format.innerGemv's rounding point)
-__global__ void __launch_bounds__(64) pf_dense_finish_half(const uint16_t* z, const uint16_t* svh, void* y,
-                                                           uint32_t out, int dt) {
-    const uint32_t nb = out / 128u, row = blockIdx.x / nb, b = blockIdx.x % nb, lane = threadIdx.x;
-    float v[2];
+// every slot's down finish, then the score-weighted sum in slot order (routed_combine_block's statements)
+__global__ void __launch_bounds__(256) pf_combine(const MoeLaunch a) {
+    const uint32_t nb = a.hidden / 128u, nbi = a.inter / 128u, groups = (nb + kPfUnit - 1u) / kPfUnit;
+    const uint32_t u0 = wave_unit(), row = u0 / groups, b0 = (u0 % groups) * kPfUnit, lane = threadIdx.x & 63u;
+    if (row >= a.rows) return;
+    const uint32_t kt = a.topk + a.shared_slots;
+    float acc[kPfUnit][2];
 #pragma unroll
-    for (uint32_t j = 0; j < 2u; ++j) v[j] = half_value(z[static_cast<size_t>(row) * out + b * 128u + lane + 64u * j]);
-    finish_values(v, svh, b, lane);
+    for (uint32_t u = 0; u < kPfUnit; ++u) acc[u][0] = acc[u][1] = 0.0f;
+    for (uint32_t k = 0; k < kt; ++k) {
+        const uint32_t rk = row * kt + k;
+        const SlotRef s = resolve_slot(a, rk);
+        if (!s.live) continue;  // uniform over the wave
+        const uint32_t q = a.inv[rk];
+        const RoutedBank& bank = s.shared ? a.shared : a.bank;
+        float z[kPfUnit][2], sv[kPfUnit][2];
 #pragma unroll
-    for (uint32_t j = 0; j < 2u; ++j)
-        store_act_rt(dt, y, static_cast<size_t>(row) * out + b * 128u + lane + 64u * j, v[j]);
+        for (uint32_t u = 0; u < kPfUnit; ++u)
+#pragma unroll
+            for (uint32_t j = 0; j < 2u; ++j) {
+                const uint32_t b = b0 + u < nb ? b0 + u : nb - 1u, i = b * 128u + lane + 64u * j;
+                z[u][j] = a.zd[static_cast<size_t>(q) * a.hidden + i];
+                sv[u][j] = half_value(bank.down_svh[static_cast<size_t>(s.e) * a.hidden + i]);
+            }
+        float xsum = 0.0f;
+        if (a.defer)
+            for (uint32_t t = 0; t < nbi; ++t) xsum += a.hs[static_cast<size_t>(q) * nbi + t];
+        const float w = s.shared ? 1.0f : score_of(a, row, k);
+#pragma unroll
+        for (uint32_t u = 0; u < kPfUnit; ++u) {
+            float v[2] = {z[u][0], z[u][1]};
+            if (a.defer)
+#pragma unroll
+                for (uint32_t j = 0; j < 2u; ++j) v[j] = __builtin_fmaf(v[j], mul1_a(), mul1_b() * xsum);
+            finish_core(v, sv[u], lane);
+#pragma unroll
+            for (uint32_t j = 0; j < 2u; ++j) acc[u][j] = __builtin_fmaf(w, v[j], acc[u][j]);
+        }
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < kPfUnit; ++u)
+        if (b0 + u < nb) routed_store_row(a, row, b0 + u, lane, acc[u]);
+}
+
+// the dense prepare: plain f16 [rows][in], in quad order for the trellis GEMM (NATURAL: as is, for a plain GEMM);
+// xs: block sums (null: not wanted)
+template <int DT, bool NATURAL>
+__global__ void __launch_bounds__(256) pf_dense_prep(const void* x, const uint16_t* suh, uint16_t* xq, float* xs,
+                                                     uint32_t in, uint32_t rows) {
+    const uint32_t nb = in / 128u, groups = (nb + kPfUnit - 1u) / kPfUnit;
+    const uint32_t u0 = wave_unit(), row = u0 / groups, b0 = (u0 % groups) * kPfUnit, lane = threadIdx.x & 63u;
+    if (row >= rows) return;
+    float v[kPfUnit][2];
+#pragma unroll
+    for (uint32_t u = 0; u < kPfUnit; ++u)
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j) {
+            const uint32_t b = b0 + u < nb ? b0 + u : nb - 1u, i = b * 128u + lane + 64u * j;
+            v[u][j] = round_half(load_act<DT>(x, static_cast<size_t>(row) * in + i)) * half_value(suh[i]);
+        }
+#pragma unroll
+    for (uint32_t u = 0; u < kPfUnit; ++u) {
+        if (b0 + u >= nb) break;
+        uint32_t hv[2];
+        float sum;
+        prep_core(v[u], lane, hv, sum);
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j) {
+            const uint32_t i = (b0 + u) * 128u + lane + 64u * j;
+            const uint32_t at = NATURAL ? i : (i & ~15u) + quad_slot(i & 15u);
+            xq[static_cast<size_t>(row) * in + at] = static_cast<uint16_t>(hv[j]);
+        }
+        if (xs && lane == 0u) xs[static_cast<size_t>(row) * nb + b0 + u] = sum;
+    }
+}
+
+// the dense finish of one plane: z f32 [rows][out] with xs [rows][in / 128] for MUL1's deferred map, or (HALF) z
+// already rounded to f16 (format.innerGemv's rounding point) by a plain GEMM
+template <int DT, bool HALF>
+__global__ void __launch_bounds__(256) pf_dense_finish(const void* z, const float* xs, const uint16_t* svh, void* y,
+                                                       uint32_t out, uint32_t rows, uint32_t inblk, int defer) {
+    const uint32_t nb = out / 128u, groups = (nb + kPfUnit - 1u) / kPfUnit;
+    const uint32_t u0 = wave_unit(), row = u0 / groups, b0 = (u0 % groups) * kPfUnit, lane = threadIdx.x & 63u;
+    if (row >= rows) return;
+    float v[kPfUnit][2], sv[kPfUnit][2];
+#pragma unroll
+    for (uint32_t u = 0; u < kPfUnit; ++u)
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j) {
+            const uint32_t b = b0 + u < nb ? b0 + u : nb - 1u, i = b * 128u + lane + 64u * j;
+            const size_t at = static_cast<size_t>(row) * out + i;
+            v[u][j] = HALF ? half_value(static_cast<const uint16_t*>(z)[at]) : static_cast<const float*>(z)[at];
+            sv[u][j] = half_value(svh[i]);
+        }
+    float xsum = 0.0f;
+    if (!HALF && defer)
+        for (uint32_t t = 0; t < inblk; ++t) xsum += xs[static_cast<size_t>(row) * inblk + t];
+#pragma unroll
+    for (uint32_t u = 0; u < kPfUnit; ++u) {
+        if (b0 + u >= nb) break;
+        if (!HALF && defer)
+#pragma unroll
+            for (uint32_t j = 0; j < 2u; ++j) v[u][j] = __builtin_fmaf(v[u][j], mul1_a(), mul1_b() * xsum);
+        finish_core(v[u], sv[u], lane);
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j)
+            store_act<DT>(y, static_cast<size_t>(row) * out + (b0 + u) * 128u + lane + 64u * j, v[u][j]);
+    }
+}
+
+inline dim3 unit_grid(uint32_t rows, uint32_t width) {
+    const uint32_t groups = (width / 128u + kPfUnit - 1u) / kPfUnit;
+    return dim3((rows * groups + 3u) / 4u);
+}
+
+template <bool NATURAL>
+hipError_t launch_pf_dense_prep(const DenseLaunch& d, uint16_t* xq, float* xs, hipStream_t s) {
+    const dim3 grid = unit_grid(d.rows, d.in), block(256);
+    if (d.dtype == kF32) hipLaunchKernelGGL((pf_dense_prep<kF32, NATURAL>), grid, block, 0, s, d.x, d.suh, xq, xs, d.in, d.rows);
+    else if (d.dtype == kF16) hipLaunchKernelGGL((pf_dense_prep<kF16, NATURAL>), grid, block, 0, s, d.x, d.suh, xq, xs, d.in, d.rows);
+    else hipLaunchKernelGGL((pf_dense_prep<kBf16, NATURAL>), grid, block, 0, s, d.x, d.suh, xq, xs, d.in, d.rows);
+    return hipGetLastError();
+}
+
+template <bool HALF>
+hipError_t launch_pf_dense_finish(const DenseLaunch& d, const void* z, hipStream_t s) {
+    const dim3 grid = unit_grid(d.rows, d.out), block(256);
+    const uint32_t inblk = d.in / 128u;
+    const int defer = d.codebook == kMul1Defer ? 1 : 0;
+    if (d.dtype == kF32) hipLaunchKernelGGL((pf_dense_finish<kF32, HALF>), grid, block, 0, s, z, d.xs, d.svh, d.y, d.out, d.rows, inblk, defer);
+    else if (d.dtype == kF16) hipLaunchKernelGGL((pf_dense_finish<kF16, HALF>), grid, block, 0, s, z, d.xs, d.svh, d.y, d.out, d.rows, inblk, defer);
+    else hipLaunchKernelGGL((pf_dense_finish<kBf16, HALF>), grid, block, 0, s, z, d.xs, d.svh, d.y, d.out, d.rows, inblk, defer);
+    return hipGetLastError();
+}
+
+// workgroup columns of a GEMM over `out` columns with `item_rows`-row items
+inline uint32_t gemm_nblk(uint32_t out, uint32_t item_rows) {
+    (void)item_rows;
+    return (out + 255u) / 256u;
 }
 
 template <int CB, bool WIDE>
-hipError_t launch_gemm_rb(const PfGemm& g, uint32_t max_items, uint32_t nproj, uint32_t item_rows, hipStream_t s) {
+hipError_t launch_gemm_rb(PfGemm g, uint32_t max_items, uint32_t nproj, uint32_t item_rows, hipStream_t s) {
+    g.nblk = gemm_nblk(g.out, item_rows);
     const dim3 grid(8u * g.nblk * ((max_items + 7u) / 8u), nproj), block(256);
-    if (item_rows == 32u) hipLaunchKernelGGL((pf_gemm<CB, WIDE, 2>), grid, block, 0, s, g);
-    else hipLaunchKernelGGL((pf_gemm<CB, WIDE, 4>), grid, block, 0, s, g);
+    if (item_rows == 32u) hipLaunchKernelGGL((pf_gemm<CB, WIDE, 2, 4>), grid, block, 0, s, g);
+    else if (item_rows == 128u) hipLaunchKernelGGL((pf_gemm<CB, WIDE, 8, 4>), grid, block, 0, s, g);
+    else hipLaunchKernelGGL((pf_gemm<CB, WIDE, 4, 4>), grid, block, 0, s, g);
     return hipGetLastError();
 }
 
@@ -413,7 +657,9 @@ hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s) {
     if ((e = hipGetLastError()) != hipSuccess) return e;
     hipLaunchKernelGGL(pf_place, dim3((p + 255u) / 256u), dim3(256), 0, s, a);
     if ((e = hipGetLastError()) != hipSuccess) return e;
-    hipLaunchKernelGGL(pf_prep, dim3(p * (a.hidden / 128u)), dim3(64), 0, s, a);
+    if (a.dtype == kF32) hipLaunchKernelGGL(pf_prep<kF32>, unit_grid(p, a.hidden), dim3(256), 0, s, a);
+    else if (a.dtype == kF16) hipLaunchKernelGGL(pf_prep<kF16>, unit_grid(p, a.hidden), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(pf_prep<kBf16>, unit_grid(p, a.hidden), dim3(256), 0, s, a);
     if ((e = hipGetLastError()) != hipSuccess) return e;
 
     PfGemm g{};
@@ -433,10 +679,9 @@ hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s) {
     g.wbits = a.wbits;
     g.positions = p;
     g.experts = a.bank.experts;
-    g.nblk = (a.inter + 255u) / 256u;
     if ((e = launch_gemm(g, a.codebook, a.max_items, 2u, a.item_rows, s)) != hipSuccess) return e;
 
-    hipLaunchKernelGGL(pf_mid, dim3(p * (a.inter / 128u)), dim3(64), 0, s, a);
+    hipLaunchKernelGGL(pf_mid, unit_grid(p, a.inter), dim3(256), 0, s, a);
     if ((e = hipGetLastError()) != hipSuccess) return e;
 
     g.w[0] = a.bank.down_t;
@@ -449,30 +694,23 @@ hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s) {
     g.in = a.inter;
     g.out = a.hidden;
     g.n = a.n_dn;
-    g.nblk = (a.hidden + 255u) / 256u;
     if ((e = launch_gemm(g, a.codebook, a.max_items, 1u, a.item_rows, s)) != hipSuccess) return e;
 
-    hipLaunchKernelGGL(pf_combine, dim3(a.rows * (a.hidden / 128u)), dim3(64), 0, s, a);
+    hipLaunchKernelGGL(pf_combine, unit_grid(a.rows, a.hidden), dim3(256), 0, s, a);
     return hipGetLastError();
 }
 
 hipError_t launch_dense_prep_natural(const DenseLaunch& d, uint16_t* xp, hipStream_t s) {
-    hipLaunchKernelGGL(pf_dense_prep_natural, dim3(d.rows * (d.in / 128u)), dim3(64), 0, s, d.x, d.suh, xp, d.in,
-                       d.dtype);
-    return hipGetLastError();
+    return launch_pf_dense_prep<true>(d, xp, nullptr, s);
 }
 
 hipError_t launch_dense_finish_half(const DenseLaunch& d, const uint16_t* z, hipStream_t s) {
-    hipLaunchKernelGGL(pf_dense_finish_half, dim3(d.rows * (d.out / 128u)), dim3(64), 0, s, z, d.svh, d.y, d.out,
-                       d.dtype);
-    return hipGetLastError();
+    return launch_pf_dense_finish<true>(d, z, s);
 }
 
 hipError_t launch_dense_prefill(const DenseLaunch& d, hipStream_t s) {
     hipError_t e;
-    hipLaunchKernelGGL(pf_dense_prep, dim3(d.rows * (d.in / 128u)), dim3(64), 0, s, d.x, d.suh,
-                       reinterpret_cast<uint16_t*>(d.xq), d.xs, d.in, d.dtype);
-    if ((e = hipGetLastError()) != hipSuccess) return e;
+    if ((e = launch_pf_dense_prep<false>(d, reinterpret_cast<uint16_t*>(d.xq), d.xs, s)) != hipSuccess) return e;
     PfGemm g{};
     g.w[0] = d.trellis;
     g.xq[0] = reinterpret_cast<const uint16_t*>(d.xq);
@@ -483,9 +721,9 @@ hipError_t launch_dense_prefill(const DenseLaunch& d, hipStream_t s) {
     g.wbits = d.wbits;
     g.positions = d.rows;
     g.experts = 1u;
-    g.nblk = (d.out + 255u) / 256u;
-    if ((e = launch_gemm(g, d.codebook, (d.rows + 63u) / 64u, 1u, 64u, s)) != hipSuccess) return e;
-    return launch_dense_finish(d, s);
+    const uint32_t item_rows = d.rows <= 64u ? 64u : 128u;
+    if ((e = launch_gemm(g, d.codebook, (d.rows + item_rows - 1u) / item_rows, 1u, item_rows, s)) != hipSuccess) return e;
+    return launch_pf_dense_finish<false>(d, d.z, s);
 }
 
 }  // namespace t3

@@ -18,16 +18,9 @@ __device__ __forceinline__ void store_act_rt(int dt, void* p, size_t i, float v)
     else store_act<kBf16>(p, i, v);
 }
 
-// One 128-block of one row, one wave: lane L owns elements L and L + 64. Returns the lane's two prepared f16 values
-// (bits) and the block's sum of them (the same in every lane).
-__device__ __forceinline__ void prep_values(int dt, const void* x, const uint16_t* suh, uint32_t in, uint32_t row,
-                                            uint32_t b, uint32_t lane, uint32_t (&hv)[2], float& sum) {
-    float v[2];
-#pragma unroll
-    for (uint32_t j = 0; j < 2u; ++j) {
-        const uint32_t i = b * 128u + lane + 64u * j;
-        v[j] = round_half(load_act_rt(dt, x, static_cast<size_t>(row) * in + i)) * half_value(suh[i]);
-    }
+// The prepare of one 128-block from its scaled inputs v = f16(x) * suh (lane L owns elements L and L + 64): the
+// lane's two prepared f16 values (bits) and the block's sum of them (the same in every lane).
+__device__ __forceinline__ void prep_core(float (&v)[2], uint32_t lane, uint32_t (&hv)[2], float& sum) {
     h128_wave(v, lane);
     sum = 0.0f;
 #pragma unroll
@@ -39,14 +32,30 @@ __device__ __forceinline__ void prep_values(int dt, const void* x, const uint16_
     for (int m = 32; m > 0; m >>= 1) sum += __shfl_xor(sum, m, 64);
 }
 
+// One 128-block of one row, one wave: loads, then prep_core.
+__device__ __forceinline__ void prep_values(int dt, const void* x, const uint16_t* suh, uint32_t in, uint32_t row,
+                                            uint32_t b, uint32_t lane, uint32_t (&hv)[2], float& sum) {
+    float v[2];
+#pragma unroll
+    for (uint32_t j = 0; j < 2u; ++j) {
+        const uint32_t i = b * 128u + lane + 64u * j;
+        v[j] = round_half(load_act_rt(dt, x, static_cast<size_t>(row) * in + i)) * half_value(suh[i]);
+    }
+    prep_core(v, lane, hv, sum);
+}
+
 // The block's outputs from its summed inner products: f16, H128, * svh / sqrt(128), f16. s[j]: the lane's two sums
-// (already through the deferred map when there is one); returns the two finished values (f16-valued).
-__device__ __forceinline__ void finish_values(float (&s)[2], const uint16_t* svh, uint32_t b, uint32_t lane) {
+// (already through the deferred map when there is one); sv: the lane's two svh values; returns the two finished values
+// (f16-valued).
+__device__ __forceinline__ void finish_core(float (&s)[2], const float (&sv)[2], uint32_t lane) {
     float v[2] = {round_half(s[0]), round_half(s[1])};
     h128_wave(v, lane);
 #pragma unroll
-    for (uint32_t j = 0; j < 2u; ++j)
-        s[j] = round_half(v[j] * kHadScale * half_value(svh[b * 128u + lane + 64u * j]));
+    for (uint32_t j = 0; j < 2u; ++j) s[j] = round_half(v[j] * kHadScale * sv[j]);
+}
+__device__ __forceinline__ void finish_values(float (&s)[2], const uint16_t* svh, uint32_t b, uint32_t lane) {
+    const float sv[2] = {half_value(svh[b * 128u + lane]), half_value(svh[b * 128u + lane + 64u])};
+    finish_core(s, sv, lane);
 }
 
 }  // namespace t3
