@@ -409,7 +409,7 @@ __global__ void __launch_bounds__(256) pf_prep(const MoeLaunch a) {
             float v[2] = {xv[u][0] * (proj ? up[u][0] : g[u][0]), xv[u][1] * (proj ? up[u][1] : g[u][1])};
             uint32_t hv[2];
             float sum;
-            prep_core(v, lane, hv, sum);
+            prep_core(v, lane, hv, sum, a.defer != 0);
 #pragma unroll
             for (uint32_t j = 0; j < 2u; ++j)
                 store_prepared<true>(proj ? a.xu : a.xg, static_cast<size_t>(q) * a.hidden,
@@ -469,7 +469,7 @@ __global__ void __launch_bounds__(256) pf_mid(const MoeLaunch a) {
         }
         uint32_t hv[2];
         float sum;
-        prep_core(d, lane, hv, sum);
+        prep_core(d, lane, hv, sum, a.defer != 0);
 #pragma unroll
         for (uint32_t j = 0; j < 2u; ++j) store_prepared<true>(a.hd, qo, (b0 + u) * 128u + lane + 64u * j, hv[j]);
         if (lane == 0u) a.hs[static_cast<size_t>(q) * nb + b0 + u] = sum;
@@ -541,7 +541,7 @@ __global__ void __launch_bounds__(256) pf_dense_prep(const void* x, const uint16
         if (b0 + u >= nb) break;
         uint32_t hv[2];
         float sum;
-        prep_core(v[u], lane, hv, sum);
+        prep_core(v[u], lane, hv, sum, xs != nullptr);
 #pragma unroll
         for (uint32_t j = 0; j < 2u; ++j) {
             const uint32_t i = (b0 + u) * 128u + lane + 64u * j;
@@ -710,7 +710,9 @@ hipError_t launch_dense_finish_half(const DenseLaunch& d, const uint16_t* z, hip
 
 hipError_t launch_dense_prefill(const DenseLaunch& d, hipStream_t s) {
     hipError_t e;
-    if ((e = launch_pf_dense_prep<false>(d, reinterpret_cast<uint16_t*>(d.xq), d.xs, s)) != hipSuccess) return e;
+    // the block sums feed MUL1's deferred map only
+    float* xs = d.codebook == kMul1Defer ? d.xs : nullptr;
+    if ((e = launch_pf_dense_prep<false>(d, reinterpret_cast<uint16_t*>(d.xq), xs, s)) != hipSuccess) return e;
     PfGemm g{};
     g.w[0] = d.trellis;
     g.xq[0] = reinterpret_cast<const uint16_t*>(d.xq);

@@ -20,13 +20,19 @@ __device__ __forceinline__ void store_act_rt(int dt, void* p, size_t i, float v)
 
 // The prepare of one 128-block from its scaled inputs v = f16(x) * suh (lane L owns elements L and L + 64): the
 // lane's two prepared f16 values (bits) and the block's sum of them (the same in every lane).
-__device__ __forceinline__ void prep_core(float (&v)[2], uint32_t lane, uint32_t (&hv)[2], float& sum) {
+// want_sum false (uniform): the sum is not needed (only MUL1's deferred map reads it) and comes back 0.
+__device__ __forceinline__ void prep_core(float (&v)[2], uint32_t lane, uint32_t (&hv)[2], float& sum,
+                                          bool want_sum = true) {
     h128_wave(v, lane);
     sum = 0.0f;
 #pragma unroll
     for (uint32_t j = 0; j < 2u; ++j) {
         hv[j] = half_bits(v[j] * kHadScale);
         sum += half_value(hv[j]);
+    }
+    if (!want_sum) {
+        sum = 0.0f;
+        return;
     }
 #pragma unroll
     for (int m = 32; m > 0; m >>= 1) sum += __shfl_xor(sum, m, 64);
