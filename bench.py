@@ -11,7 +11,11 @@ HBM, not from the 256 MB Infinity Cache. Inputs are resident in HBM before the t
 Prints ONE JSON line: the whole-call rate as GB/s of trellis code bytes (`value`), the dominant kernel's roofline
 (`roofline`: algorithmic code bytes of one launch / its average duration, timed alone with HIP events on the launch
 stream, against 8 TB/s), and the CPU oracle (`format.project` restated in C) timed on this box's host cores
-(`cpu_baseline`). `--sweep` adds K = 3, 4, 5 x rows = 1, 4, 16, 32.
+(`cpu_baseline`). The same line carries the other configurations of BASELINE.json as extra objects: `moe_decode`
+(config 3: routed decode at 1 and 8 tokens), `moe_prefill` (config 4: the routed prefill chain, TFLOP/s against the
+2.5 PFLOP/s dense f16 MFMA peak) and `dense_prefill` (config 5: 4096 rows); `--quick` leaves them out. `--sweep` adds
+K = 3, 4, 5 x rows = 1, 4, 16, 32; `--in-f/--out-f/--k/--rows` time another dense shape (lm_head: --in-f 4096
+--out-f 151936 --k 6).
 """
 from __future__ import annotations
 
@@ -275,9 +279,11 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--k", type=int, default=4)
     ap.add_argument("--rows", type=int, default=1)
-    ap.add_argument("--moe", action="store_true", help="also time the routed-expert decode chain (config 3)")
+    ap.add_argument("--moe", action="store_true", help="(default on) time the routed-expert decode chain (config 3)")
+    ap.add_argument("--quick", action="store_true", help="the headline workload only: no routed or prefill timings")
     ap.add_argument("--prefill", action="store_true",
-                    help="also time the routed prefill chain (config 4) and the dense 4096-row projection (config 5)")
+                    help="(default on) time the routed prefill chain (config 4) and the dense 4096-row projection "
+                         "(config 5)")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run one 256 MiB device copy, the known-size kernel that scales the profiler's "
                          "FETCH_SIZE / WRITE_SIZE readings")
@@ -286,6 +292,8 @@ def main() -> int:
     args = ap.parse_args()
     global IN_F, OUT_F
     IN_F, OUT_F = args.in_f, args.out_f
+    if not args.quick:
+        args.moe = args.prefill = True
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU (the path has no collective); --gpus {args.gpus} is not served",
               file=sys.stderr)
