@@ -1,0 +1,133 @@
+"""The BASELINE configurations at their full sizes: decoded weights bit-exact, sampled rows (and, where a whole row is
+too much for the CPU oracle, sampled 128-column output blocks, which are independent of the rest of the row) within
+the reference's bars, and the size-independent byte equalities."""
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_util import MCG, MUL1, bytes_of, dev_f16_bits, dev_u16, host_u16, make_x, to_f32
+from tests.test_gpu_moe import RefBank, dev_bank
+
+pytestmark = pytest.mark.gpu
+
+F32_BAR, BF16_DENSE_BAR, BF16_MOE_BAR = 5e-3, 2.5e-2, 1.5e-2
+
+
+@pytest.fixture(scope="module")
+def t3():
+    from turboexl3_amd import api
+    return api
+
+
+def block_ref(oracle, trellis, suh, svh, x_f32, in_f, n, codebook, blk):
+    """Output columns [128 blk, 128 blk + 128) of format.project: the block's own 8 tile columns and svh slice."""
+    sub = np.ascontiguousarray(trellis[:, 8 * blk:8 * blk + 8, :])
+    return oracle.project_rows(x_f32, sub, suh, np.ascontiguousarray(svh[128 * blk:128 * blk + 128]), in_f, 128, n,
+                               codebook, 0xFFFF, threads=8)
+
+
+@pytest.mark.parametrize("k", [3, 4, 5])
+def test_config2_qkv_shape_rows_1_4_16_32(oracle, t3, k):
+    in_f, out_f, n = 4096, 12288, 16 * k
+    rng = np.random.default_rng(0xC2 + k)
+    trellis, suh, svh = oracle.synth_linear(rng, in_f, out_f, n)
+    d_t, d_suh, d_svh = dev_u16(trellis), dev_f16_bits(suh), dev_f16_bits(svh)
+    w_hat = oracle.reconstruct_inner(trellis, in_f, out_f, n, MCG)
+    assert np.array_equal(host_u16(t3.dequant(d_t, t3.Decode.mcg)), w_hat), "W_hat is not bit-exact at full size"
+    x_dev, x_f32 = make_x(rng, 32, in_f, torch.float16, outliers=True)
+    ref = oracle.project_rows(x_f32, trellis, suh, svh, in_f, out_f, n, MCG, 0xFFFF, threads=8, w_hat=w_hat)
+    alone = t3.linear(x_dev[:1], d_t, d_suh, d_svh, t3.Decode.mcg)
+    for rows in (1, 4, 16, 32):
+        y = t3.linear(x_dev[:rows], d_t, d_suh, d_svh, t3.Decode.mcg)
+        got = to_f32(y)
+        for r in range(rows):
+            e = oracle.compare(got[r], ref[r], 2.0 ** -11)  # f16 outputs: half an ulp of the store on top of the bar
+            assert e <= F32_BAR, f"K{k} rows {rows} row {r}: {e:.3e}"
+        assert bytes_of(y[0]) == bytes_of(alone[0]), "row 0 differs from the row alone"
+
+
+def test_config5_lm_head_k6_rows_1_and_256(oracle, t3):
+    in_f, out_f, n = 4096, 151936, 96
+    rng = np.random.default_rng(0xC5)
+    trellis = rng.integers(0, 65536, (in_f // 16, out_f // 16, n), dtype=np.uint16)
+    _, suh, svh = oracle.synth_linear(rng, in_f, 128, n)
+    svh = np.tile(svh, out_f // 128)
+    d_t, d_suh, d_svh = dev_u16(trellis), dev_f16_bits(suh), dev_f16_bits(svh)
+    x_dev, x_f32 = make_x(rng, 256, in_f, torch.bfloat16)
+    y1 = to_f32(t3.linear(x_dev[:1], d_t, d_suh, d_svh, t3.Decode.mul1))
+    y256 = to_f32(t3.linear(x_dev, d_t, d_suh, d_svh, t3.Decode.mul1))
+    for blk in (0, 1, 593, out_f // 128 - 1):
+        ref = block_ref(oracle, trellis, suh, svh, x_f32[[0, 100, 255]], in_f, n, MUL1, blk)
+        cols = slice(128 * blk, 128 * blk + 128)
+        assert oracle.compare(y1[0, cols], ref[0]) <= BF16_DENSE_BAR
+        for i, r in enumerate((0, 100, 255)):
+            assert oracle.compare(y256[r, cols], ref[i]) <= BF16_DENSE_BAR, (blk, r)
+
+
+def test_config5_dense_4096_rows_w_hat_form(oracle, t3):
+    in_f, out_f, n, rows = 4096, 14336, 64, 4096
+    rng = np.random.default_rng(0xC55)
+    trellis, suh, svh = oracle.synth_linear(rng, in_f, out_f, n)
+    d_t, d_suh, d_svh = dev_u16(trellis), dev_f16_bits(suh), dev_f16_bits(svh)
+    x_dev, x_f32 = make_x(rng, rows, in_f, torch.bfloat16)
+    y = t3.linear(x_dev, d_t, d_suh, d_svh, t3.Decode.mcg)
+    sample = [0, 1, 2047, 4095]
+    got = to_f32(y[sample])
+    for blk in (0, 55, out_f // 128 - 1):
+        ref = block_ref(oracle, trellis, suh, svh, x_f32[sample], in_f, n, MCG, blk)
+        for i in range(len(sample)):
+            assert oracle.compare(got[i, 128 * blk:128 * blk + 128], ref[i]) <= BF16_DENSE_BAR, (blk, sample[i])
+
+
+def routing_softmax(rng, tokens, topk, experts):
+    logits = rng.standard_normal((tokens, experts)).astype(np.float32)
+    slots = np.argsort(-logits, axis=1)[:, :topk].astype(np.int32)
+    top = np.take_along_axis(logits, slots, axis=1)
+    w = np.exp(top - top.max(axis=1, keepdims=True))
+    return slots, (w / w.sum(axis=1, keepdims=True)).astype(np.float32)
+
+
+def test_config3_routed_decode_with_shared_expert(oracle, t3):
+    experts, hidden, inter, n, topk, limit = 512, 2048, 512, 48, 10, 7
+    rng = np.random.default_rng(0xC3)
+    bank = oracle.synth_bank(rng, experts, hidden, inter, n)
+    shared = oracle.synth_bank(rng, 1, hidden, inter, n)
+    dbank, dshared = dev_bank(t3, bank), dev_bank(t3, shared)
+    ref, sref = RefBank(oracle, bank, MCG, 0xFFFF), RefBank(oracle, shared, MCG, 0xFFFF)
+    x_dev, x_f32 = make_x(rng, 8, hidden, torch.bfloat16)
+    slots, scores = routing_softmax(rng, 8, topk, experts)
+    d_slots, d_scores = torch.from_numpy(slots).cuda(), torch.from_numpy(scores).cuda()
+    for tokens in (1, 8):
+        y = t3.moe_shared_expert(x_dev[:tokens].reshape(1, tokens, hidden), dbank, d_slots[:tokens].reshape(1, tokens, topk),
+                                 d_scores[:tokens].reshape(1, tokens, topk), t3.Decode.mcg, limit, dshared)
+        got = to_f32(y).reshape(tokens, hidden)
+        for r in range(tokens):
+            want = (ref.row(x_f32[r], slots[r], scores[r], float(limit)) + sref.slot(0, x_f32[r], float(limit))).astype(np.float32)
+            e = oracle.compare(got[r], want)
+            assert e <= BF16_MOE_BAR, f"{tokens} tokens row {r}: {e:.3e}"
+        if tokens == 1:
+            first = bytes_of(y[0, 0])
+        else:
+            assert bytes_of(y[0, 0]) == first, "row 0 of 8 tokens differs from the row alone"
+
+
+def test_config4_routed_prefill_widths_mixed_rates(oracle, t3):
+    # config 4's widths and rates (7168 / 2048, gate|up K2, down K3, top-8, clamp 7, bf16) with 64 rows an expert as
+    # there (2048 tokens x 8 / 256), on a quarter of its experts and tokens so the CPU side stays small
+    experts, hidden, inter, topk, tokens, limit = 64, 7168, 2048, 8, 512, 7
+    rng = np.random.default_rng(0xC4)
+    bank = oracle.synth_bank(rng, experts, hidden, inter, 32, 48)
+    dbank = dev_bank(t3, bank)
+    ref = RefBank(oracle, bank, MCG, 0xFFFF)
+    x_dev, x_f32 = make_x(rng, tokens, hidden, torch.bfloat16)
+    slots, scores = routing_softmax(rng, tokens, topk, experts)
+    d_slots, d_scores = torch.from_numpy(slots).cuda(), torch.from_numpy(scores).cuda()
+    y = t3.moe_clamped(x_dev.reshape(1, tokens, hidden), dbank, d_slots.reshape(1, tokens, topk),
+                       d_scores.reshape(1, tokens, topk), t3.Decode.mcg, limit)
+    got = to_f32(y).reshape(tokens, hidden)
+    for r in (0, 300, tokens - 1):
+        e = oracle.compare(got[r], ref.row(x_f32[r], slots[r], scores[r], float(limit)))
+        assert e <= BF16_MOE_BAR, f"row {r}: {e:.3e}"
+    y17 = t3.moe_clamped(x_dev[:17].reshape(1, 17, hidden), dbank, d_slots[:17].reshape(1, 17, topk),
+                         d_scores[:17].reshape(1, 17, topk), t3.Decode.mcg, limit)
+    assert bytes_of(y17[0]) == bytes_of(y[0, :17]), "rows 0-16 of 512 tokens differ from the 17-row call"
