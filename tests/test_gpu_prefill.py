@@ -190,3 +190,20 @@ def test_dense_w_hat_form_from_512_rows(oracle, t3, in_f, out_f, n, codebook, dt
             worst = max(worst, e)
             assert e <= bar, f"{name} form row {r}: {e:.3e} over the bar {bar}"
     print(f"dense W_hat form {in_f}x{out_f} n={n} {dtype}: worst {worst:.3e} (bar {bar})")
+
+
+def test_trellis_gemm_every_live_block_count(oracle, t3):
+    """The GEMM's K loop is specialised by the item's live 16-row blocks (1..4 in the 64-row shape, 1..8 in the 128-row
+    shape): row counts that end an item at every block count, both codebooks."""
+    for codebook, seed in ((MCG, 5), (MUL1, 6)):
+        case = DenseCase(oracle, t3, seed, 512, 256, 64, codebook)
+        x_dev, x_f32 = make_x(case.rng, 257, 512, torch.float32)
+        yref = case.ref(x_f32)
+        t3.configure(dense_gemm_rows=0)
+        try:
+            for rows in (33, 47, 48, 49, 63, 64, 65, 80, 81, 96, 97, 112, 113, 128, 129, 145, 161, 177, 193, 209, 225, 241, 257):
+                got = to_f32(t3.linear(x_dev[:rows], case.d_trellis, case.d_suh, case.d_svh, case.dec))
+                worst = max(oracle.compare(got[r], yref[r]) for r in range(rows))
+                assert worst <= F32_BAR, f"codebook {codebook} rows {rows}: {worst:.3e}"
+        finally:
+            t3.configure()

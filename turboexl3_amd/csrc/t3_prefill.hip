@@ -54,7 +54,10 @@ __device__ __forceinline__ uint32_t weight_halves(uint32_t cw_lo, uint32_t cw_hi
         asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1"
             : "=v"(d)
             : "v"(pa));
-        asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1"
+        // the two wait states a sub-dword write needs before a matrix instruction reads the register: the compiler
+        // adds them for its own SDWA instructions, not for this one
+        asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+            "s_nop 1"
             : "+v"(d)
             : "v"(pb));
         return d;
