@@ -48,7 +48,16 @@ typedef enum t3_status {
     T3_InvalidTurboexl3Config = 10,     /* src/core/config.zig:175-178 */
     T3_WorkspaceTooSmall = 11,          /* this ABI: the caller's scratch is smaller than *_workspace_bytes says */
     T3_HipFailed = 12,                  /* src/hip/runtime.zig:6 */
-    T3_BadArgs = 13                     /* src/hip/runtime.zig:6: a null pointer or a descriptor that is not one */
+    T3_BadArgs = 13,                    /* src/hip/runtime.zig:6: a null pointer or a descriptor that is not one */
+    /* the quant table's names (table/config.zig:26, table/table.zig:128-174) */
+    T3_NotExl3 = 14,
+    T3_Exl3CodebookUnsupported = 15,
+    T3_Exl3RateUnsupported = 16,
+    T3_MissingWeight = 17,
+    T3_Exl3TrellisGeometry = 18,
+    T3_Exl3WidthNotMultipleOf128 = 19,
+    T3_Exl3SideGeometry = 20,
+    T3_Exl3SideDtype = 21
 } t3_status;
 
 /* The reference's error name of a status ("BadExl3Shape", ...); "ok" for T3_OK; never NULL. */
@@ -185,6 +194,66 @@ int32_t t3_admit_topk(int64_t topk);
 /* A stacked trellis [E, in/16, out/16, n] at or under rate n_max (src/core/spec.zig:80-88): 1 admitted, 0 not. */
 int32_t t3_trellis_admitted(const int64_t* shape, int32_t ndim, int64_t experts, int64_t in_dim, int64_t out_dim,
                             int64_t n_max);
+
+/* ---- the quant table (table/config.zig, table/table.zig) -------------------------------------------------------
+ * turboexl3 as an mlx-serve quant table: which blocks of a pack's config it claims, what validation names, the bill,
+ * the checks a weight passes as it loads, and the table's compute members over loaded weights. JSON arrives as
+ * NUL-terminated text. A verdict (`Verdict`, table/table.zig:62,591-593) is its kind plus a reason written to `why`
+ * (NUL-terminated, truncated to why_bytes; the reference's error name or message; empty for ok). The plugin kit's ABI
+ * struct layouts are not part of the reference tree: these entry points carry the same semantics over this header's own
+ * descriptors. */
+
+enum { T3_CLAIM_NO = 0, T3_CLAIM_BY_TYPE = 1, T3_CLAIM_BY_MARKER = 2 };          /* docs/core/glossary.md:220-221 */
+enum { T3_VERDICT_OK = 0, T3_VERDICT_UNSUPPORTED = 1, T3_VERDICT_FAILED = 2, T3_VERDICT_TOO_LARGE = 3 };
+enum { T3_BLOCK_TRUNK = 0, T3_BLOCK_BANK = 1 };                                    /* table/config.zig:14 */
+
+/* A claimed block (table/config.zig:16-25): a dense trunk's (`trunk_quant`) or a routed bank set's (`expert_quant`). */
+typedef struct t3_block {
+    int32_t kind;        /* T3_BLOCK_* */
+    int32_t codebook;    /* 0 MUL1, 1 MCG */
+    int32_t window_bits; /* 8..16 */
+    int32_t n;           /* a bank block's rate: halfwords a tile (16 k); 0 for a trunk block */
+} t3_block;
+
+/* A loaded weight with its decode (table/table.zig:174-194): `layout` the codebook, `flags` the window's bits, `block`
+ * the rate (halfwords a tile). The arrays stay the caller's. */
+typedef struct t3_weight {
+    t3_array w, scales, biases;
+    int32_t layout, flags, block;
+} t3_weight;
+
+/* table/config.zig:36-52 `parseBlock`: T3_OK, or NotExl3 / Exl3CodebookUnsupported / Exl3WindowUnsupported /
+ * Exl3RateUnsupported. */
+int32_t t3_table_parse_block(const char* block_json, t3_block* out);
+/* table/config.zig:59-72 `claimFor`: a trunk block always by marker; a bank block by marker on a fully EXL3 Qwen3.8
+ * pack, unclamped, where the matrix-engine gate holds (`matrix_gate`: the reference passes MLX's NAX gate; on MI355X
+ * the MFMA paths are always there, so a host passes 1). Returns T3_CLAIM_*. */
+int32_t t3_table_claims(const char* block_json, const char* config_json, int32_t matrix_gate);
+/* table/config.zig:74-85 `validate`: returns T3_VERDICT_*; the reason names an unserved codebook, window, rate, top-k. */
+int32_t t3_table_validate(const char* block_json, const char* config_json, char* why, size_t why_bytes);
+/* table/config.zig:88-92 `bill`: the weights are the server's loaded arrays, as stored. */
+uint64_t t3_table_bill(const char* block_json, const char* model_dir, uint64_t stored);
+/* table/table.zig:119-145 `loadTensor`: `<base>.weight` (trellis U16/I16 [in/16, out/16, n]), `.scales` (suh F16 [in]),
+ * `.biases` (svh F16 [out]) under a trunk block; in_dim 0 = unchecked. A NULL array is a missing tensor. */
+int32_t t3_table_load_tensor(const t3_block* block, const t3_array* weight, const t3_array* scales,
+                             const t3_array* biases, uint32_t in_dim, t3_weight* out, char* why, size_t why_bytes);
+/* table/table.zig:147-174 `loadBank`: `<base>.{trellis,suh,svh}` under a bank block: trellis U16 [E, in/16, out/16, n]
+ * at or under the block's rate, suh F16 [E, in], svh F16 [E, out]. */
+int32_t t3_table_load_bank(const t3_block* block, const t3_array* trellis, const t3_array* suh, const t3_array* svh,
+                           uint32_t in_dim, t3_weight* out, char* why, size_t why_bytes);
+/* table/table.zig:196-201 `matmul`: `t3_linear` with the weight's own decode. */
+int32_t t3_table_matmul(t3_stream stream, const t3_weight* w, const t3_array* x, t3_array* y, void* workspace,
+                        size_t workspace_bytes, char* why, size_t why_bytes);
+int32_t t3_table_matmul_workspace_bytes(const t3_weight* w, const t3_array* x, size_t* bytes);
+/* table/table.zig:203-205 `moe`: always refuses: a layer's banks run as one routed SwiGLU. */
+int32_t t3_table_moe(char* why, size_t why_bytes);
+/* table/table.zig:210-222 `swiglu`: refuses banks that decode differently; limit > 0 runs `t3_moe_clamped`. */
+int32_t t3_table_swiglu(t3_stream stream, const t3_weight* gate, const t3_weight* up, const t3_weight* down,
+                        const t3_array* x, const t3_array* inds, const t3_array* scores, int32_t limit,
+                        int32_t verify_rows, t3_array* y, void* workspace, size_t workspace_bytes, char* why,
+                        size_t why_bytes);
+int32_t t3_table_swiglu_workspace_bytes(const t3_weight* gate, const t3_weight* up, const t3_weight* down,
+                                        const t3_array* x, const t3_array* inds, size_t* bytes);
 
 /* ---- device self-tests (the roles of src/kernels/hip/test/lane.hip) ------------------------------------------ */
 

@@ -41,8 +41,22 @@ class Config(C.Structure):
                 ("mcg_pair", C.c_int32), ("mul1_defer", C.c_int32), ("dense_gemm_rows", C.c_int32)]
 
 
+class Block(C.Structure):
+    _fields_ = [("kind", C.c_int32), ("codebook", C.c_int32), ("window_bits", C.c_int32), ("n", C.c_int32)]
+
+
+class Weight(C.Structure):
+    _fields_ = [("w", Array), ("scales", Array), ("biases", Array), ("layout", C.c_int32), ("flags", C.c_int32),
+                ("block", C.c_int32)]
+
+
+CLAIM_NO, CLAIM_BY_TYPE, CLAIM_BY_MARKER = 0, 1, 2
+VERDICT_OK, VERDICT_UNSUPPORTED, VERDICT_FAILED, VERDICT_TOO_LARGE = 0, 1, 2, 3
+BLOCK_TRUNK, BLOCK_BANK = 0, 1
+
 # every symbol include/turboexl3_hip.h declares: name -> (restype, argtypes)
 _AP, _BP = C.POINTER(Array), C.POINTER(Bank)
+_KP, _WP, _SZP = C.POINTER(Block), C.POINTER(Weight), C.POINTER(C.c_size_t)
 _u16p = C.POINTER(C.c_uint16)
 SYMBOLS = {
     "t3_error_name": (C.c_char_p, [C.c_int32]),
@@ -64,6 +78,18 @@ SYMBOLS = {
     "t3_rate_admitted": (C.c_int32, [C.c_int64]),
     "t3_admit_topk": (C.c_int32, [C.c_int64]),
     "t3_trellis_admitted": (C.c_int32, [C.POINTER(C.c_int64), C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_int64]),
+    "t3_table_parse_block": (C.c_int32, [C.c_char_p, _KP]),
+    "t3_table_claims": (C.c_int32, [C.c_char_p, C.c_char_p, C.c_int32]),
+    "t3_table_validate": (C.c_int32, [C.c_char_p, C.c_char_p, C.c_char_p, C.c_size_t]),
+    "t3_table_bill": (C.c_uint64, [C.c_char_p, C.c_char_p, C.c_uint64]),
+    "t3_table_load_tensor": (C.c_int32, [_KP, _AP, _AP, _AP, C.c_uint32, _WP, C.c_char_p, C.c_size_t]),
+    "t3_table_load_bank": (C.c_int32, [_KP, _AP, _AP, _AP, C.c_uint32, _WP, C.c_char_p, C.c_size_t]),
+    "t3_table_matmul": (C.c_int32, [C.c_void_p, _WP, _AP, _AP, C.c_void_p, C.c_size_t, C.c_char_p, C.c_size_t]),
+    "t3_table_matmul_workspace_bytes": (C.c_int32, [_WP, _AP, _SZP]),
+    "t3_table_moe": (C.c_int32, [C.c_char_p, C.c_size_t]),
+    "t3_table_swiglu": (C.c_int32, [C.c_void_p, _WP, _WP, _WP, _AP, _AP, _AP, C.c_int32, C.c_int32, _AP, C.c_void_p,
+                                    C.c_size_t, C.c_char_p, C.c_size_t]),
+    "t3_table_swiglu_workspace_bytes": (C.c_int32, [_WP, _WP, _WP, _AP, _AP, _SZP]),
     "t3_test_codebooks": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "t3_test_lane": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int64, C.c_void_p, C.c_void_p,
                                  C.c_void_p]),

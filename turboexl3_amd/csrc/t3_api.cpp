@@ -40,6 +40,14 @@ const char* t3_error_name(int32_t status) {
         case T3_WorkspaceTooSmall: return "WorkspaceTooSmall";
         case T3_HipFailed: return "HipFailed";
         case T3_BadArgs: return "BadArgs";
+        case T3_NotExl3: return "NotExl3";
+        case T3_Exl3CodebookUnsupported: return "Exl3CodebookUnsupported";
+        case T3_Exl3RateUnsupported: return "Exl3RateUnsupported";
+        case T3_MissingWeight: return "MissingWeight";
+        case T3_Exl3TrellisGeometry: return "Exl3TrellisGeometry";
+        case T3_Exl3WidthNotMultipleOf128: return "Exl3WidthNotMultipleOf128";
+        case T3_Exl3SideGeometry: return "Exl3SideGeometry";
+        case T3_Exl3SideDtype: return "Exl3SideDtype";
         default: return "UnknownStatus";
     }
 }
