@@ -146,6 +146,12 @@ int32_t t3_linear_stages(t3_stream stream, const t3_array* x, const t3_array* tr
                          const t3_array* svh, t3_decode dec, t3_array* y, void* workspace, size_t workspace_bytes,
                          uint32_t stages);
 
+/* `t3_linear` plus a bias [out] in x's dtype: one add in x's dtype after the projection's own output rounding, so a
+ * sum rounds twice (src/root.zig:358-376 `linearBias`). */
+int32_t t3_linear_bias(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
+                       const t3_array* svh, const t3_array* bias, t3_decode dec, t3_array* y, void* workspace,
+                       size_t workspace_bytes);
+
 /* W_hat f16 [in, out] from trellis [in/16, out/16, n], bit-exact to format.reconstructInner
  * (src/core/format.zig:276-291; the role of src/core/dense.zig:909-922 `dequantize`). */
 int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_array* w_hat);
@@ -165,6 +171,14 @@ int32_t t3_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const t
 int32_t t3_moe_clamped(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
                        const t3_array* scores, t3_decode dec, int32_t limit, t3_array* y, void* workspace,
                        size_t workspace_bytes);
+/* Where a clamped SwiGLU clamps (src/core/format.zig:80-83 `ClampAt`): gate_in, DeepSeek-V4's and GLM's:
+ * silu(min(g, L)) * clamp(u, -L, L); silu_out, Ling-3.1's: min(silu(g), L) * clamp(u, -L, L). */
+enum { T3_CLAMP_GATE_IN = 0, T3_CLAMP_SILU_OUT = 1 };
+/* `moe`'s chains with the clamp `limit` (0: none; 1..128) at `clamp_at` (src/root.zig:826-833 `moeSwiglu`):
+ * `t3_moe` is this at limit 0, `t3_moe_clamped` at gate_in. */
+int32_t t3_moe_swiglu(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
+                      const t3_array* scores, t3_decode dec, int32_t limit, int32_t clamp_at, t3_array* y,
+                      void* workspace, size_t workspace_bytes);
 /* `t3_moe` plus an already gated shared-expert output of x's shape and dtype, added at the routed output's
  * rounding point (src/root.zig:976-984). */
 int32_t t3_moe_with_shared(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,

@@ -157,3 +157,21 @@ def test_dense_refusals(t3):
     assert name(lambda: t3.linear_chain(x, tr, suh, svh, t3.Decode(MCG, 17))) == "Exl3WindowUnsupported"
     # in = 16 * 30 is not a multiple of 128
     assert name(lambda: t3.linear_chain(x[:, :480], tr[:30].contiguous(), suh[:480], svh, t3.Decode.mcg)) == "BadExl3Shape"
+
+
+def test_linear_bias_is_linear_plus_one_rounded_add(oracle, t3):
+    # src/root.zig:358-376: the add is in x's dtype after linear's own output rounding
+    case = DenseCase(oracle, t3, 0xB1A5, 512, 256, 64, MCG)
+    for dtype, rows in ((torch.bfloat16, 3), (torch.float16, 40), (torch.float32, 1)):
+        x_dev, _ = make_x(case.rng, rows, 512, dtype)
+        bias = torch.from_numpy(case.rng.standard_normal(256).astype(np.float32)).cuda().to(dtype)
+        y = t3.linear(x_dev, case.d_trellis, case.d_suh, case.d_svh, case.dec)
+        got = t3.linear_bias(x_dev, case.d_trellis, case.d_suh, case.d_svh, bias, case.dec)
+        want = (y.to(torch.float32) + bias.to(torch.float32)).to(dtype)
+        assert bytes_of(got) == bytes_of(want)
+    with pytest.raises(t3.T3Error) as e:
+        t3.linear_bias(x_dev, case.d_trellis, case.d_suh, case.d_svh, bias[:128].contiguous(), case.dec)
+    assert e.value.name == "BadExl3Shape"
+    with pytest.raises(t3.T3Error) as e:
+        t3.linear_bias(x_dev, case.d_trellis, case.d_suh, case.d_svh, bias.to(torch.float16), case.dec)
+    assert e.value.name == "BadExl3Dtype"

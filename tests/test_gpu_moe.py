@@ -239,3 +239,32 @@ def test_moe_refusals(oracle, t3):
     bad = oracle.synth_bank(rng, 4, 256, 128, 32)
     bad.down_svh = bad.down_svh[:, :128]
     assert name(lambda: t3.moe(x, dev_bank(t3, bad), inds, scores, t3.Decode.mcg)) == "BadExl3Shape"
+
+
+def test_silu_out_clamp_decode_and_prefill_rows(oracle, t3):
+    # Ling-3.1's clamp (format.ClampAt.silu_out; ref.moeRowClampedAt at silu_out): min(silu(g), L) * clamp(u, -L, L)
+    rng = np.random.default_rng(0x51C)
+    hidden, inter, experts, topk, n = 512, 256, 6, 3, 64
+    bank = oracle.synth_bank(rng, experts, hidden, inter, n)
+    dbank = dev_bank(t3, bank)
+    rows = 40
+    x_dev, x_f32 = make_x(rng, rows, hidden, torch.float32)
+    x_dev, x_f32 = x_dev * 3.0, x_f32 * np.float32(3.0)  # gates large enough that silu(g) passes the limit
+    slots, scores = routing(rng, rows, topk, experts)
+    d_slots, d_scores = torch.from_numpy(slots).cuda(), torch.from_numpy(scores).cuda()
+    limit = 1
+    for count in (3, rows):  # the decode chain, then the prefill chain
+        args = (x_dev[:count].reshape(1, count, hidden), dbank, d_slots[:count].reshape(1, count, topk),
+                d_scores[:count].reshape(1, count, topk), t3.Decode.mcg)
+        out = to_f32(t3.moe_swiglu(*args, limit, t3.SILU_OUT)).reshape(count, hidden)
+        gate_in = to_f32(t3.moe_swiglu(*args, limit, t3.GATE_IN)).reshape(count, hidden)
+        assert bytes_of(t3.moe_swiglu(*args, limit, t3.GATE_IN)) == bytes_of(t3.moe_clamped(*args, limit))
+        assert bytes_of(t3.moe_swiglu(*args, 0, t3.SILU_OUT)) == bytes_of(t3.moe(*args))
+        for r in (0, count - 1):
+            want, hits = oracle.moe_row(bank, x_f32[r], slots[r], scores[r], MCG, limit=float(limit), clamp_at=1)
+            assert hits[0] > 0 and hits[1] > 0
+            assert oracle.compare(out[r], want) <= F32_BAR
+            assert oracle.compare(out[r], gate_in[r]) > 1e-2, "the two clamps should differ on this case"
+    with pytest.raises(t3.T3Error) as e:
+        t3.moe_swiglu(*args, 5, 2)
+    assert e.value.name == "InvalidExl3Clamp"

@@ -67,9 +67,12 @@ SYMBOLS = {
     "t3_linear_workspace_bytes": (C.c_int32, [_AP, _AP, Decode, C.POINTER(C.c_size_t)]),
     "t3_linear_chain": (C.c_int32, [C.c_void_p, _AP, _AP, _AP, _AP, Decode, _AP, C.c_void_p, C.c_size_t]),
     "t3_linear_stages": (C.c_int32, [C.c_void_p, _AP, _AP, _AP, _AP, Decode, _AP, C.c_void_p, C.c_size_t, C.c_uint32]),
+    "t3_linear_bias": (C.c_int32, [C.c_void_p, _AP, _AP, _AP, _AP, _AP, Decode, _AP, C.c_void_p, C.c_size_t]),
     "t3_dequant": (C.c_int32, [C.c_void_p, _AP, Decode, _AP]),
     "t3_moe": (C.c_int32, [C.c_void_p, _AP, _BP, _AP, _AP, Decode, C.c_int32, _AP, C.c_void_p, C.c_size_t]),
     "t3_moe_clamped": (C.c_int32, [C.c_void_p, _AP, _BP, _AP, _AP, Decode, C.c_int32, _AP, C.c_void_p, C.c_size_t]),
+    "t3_moe_swiglu": (C.c_int32, [C.c_void_p, _AP, _BP, _AP, _AP, Decode, C.c_int32, C.c_int32, _AP, C.c_void_p,
+                                   C.c_size_t]),
     "t3_moe_with_shared": (C.c_int32, [C.c_void_p, _AP, _BP, _AP, _AP, Decode, C.c_int32, _AP, _AP, C.c_void_p,
                                         C.c_size_t]),
     "t3_moe_shared_expert": (C.c_int32, [C.c_void_p, _AP, _BP, _AP, _AP, Decode, C.c_int32, _BP, _AP, C.c_void_p,

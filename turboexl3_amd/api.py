@@ -201,6 +201,38 @@ def moe_clamped(x, bank: Bank, inds, scores, dec: Decode, limit: int, stream=Non
     return y
 
 
+GATE_IN, SILU_OUT = 0, 1
+
+
+def moe_swiglu(x, bank: Bank, inds, scores, dec: Decode, limit: int, clamp_at: int = GATE_IN, stream=None) -> torch.Tensor:
+    """root.moeSwiglu: `moe` with the SwiGLU's clamp `limit` (0: none) at `clamp_at` (format.ClampAt)."""
+    L = _lib.lib()
+    ax, ai, asc = _arr(x), _arr(inds), _arr(scores)
+    cb, _keep = _cbank(bank)
+    if not (0 <= int(limit) <= 128) or clamp_at not in (GATE_IN, SILU_OUT):
+        raise T3Error(6)
+    ws = _moe_workspace(L, ax, cb, ai, x.device)
+    y = torch.empty_like(x)
+    ay = _arr(y)
+    _check(L.t3_moe_swiglu(_stream_ptr(stream), C.byref(ax), C.byref(cb), C.byref(ai), C.byref(asc), dec.c(), int(limit),
+                           int(clamp_at), C.byref(ay), ws.data_ptr(), ws.numel()))
+    return y
+
+
+def linear_bias(x, trellis, suh, svh, bias, dec: Decode = Decode.mul1, stream=None) -> torch.Tensor:
+    """root.linearBias: `linear` plus a bias [out] in x's dtype (one add after the output rounding)."""
+    L = _lib.lib()
+    ax, at, asu, asv, ab = _arr(x), _arr(trellis), _arr(suh), _arr(svh), _arr(bias)
+    need = C.c_size_t(0)
+    _check(L.t3_linear_workspace_bytes(C.byref(ax), C.byref(at), dec.c(), C.byref(need)))
+    y = torch.empty(*x.shape[:-1], trellis.shape[1] * 16, dtype=x.dtype, device=x.device)
+    ay = _arr(y)
+    ws = _workspace(x.device, need.value)
+    _check(L.t3_linear_bias(_stream_ptr(stream), C.byref(ax), C.byref(at), C.byref(asu), C.byref(asv), C.byref(ab), dec.c(),
+                            C.byref(ay), ws.data_ptr(), ws.numel()))
+    return y
+
+
 def moe_with_shared(x, bank: Bank, inds, scores, dec: Decode, verify_rows: bool, shared, stream=None) -> torch.Tensor:
     """root.moeWithShared: `moe` plus an already gated shared-expert output of x's shape and dtype."""
     L = _lib.lib()

@@ -297,6 +297,26 @@ hipError_t launch_gemv_cb(const DenseLaunch& d, int fuse, hipStream_t s) {
 
 }  // namespace
 
+namespace {
+// y[row][c] = dtype(y[row][c] + bias[c]): grid (ceil(out / 256), rows), 256 threads
+__global__ void __launch_bounds__(256) bias_add(void* y, const void* bias, uint32_t out, int dt) {
+    const uint32_t c = blockIdx.x * 256u + threadIdx.x;
+    if (c >= out) return;
+    const size_t at = static_cast<size_t>(blockIdx.y) * out + c;
+    store_act_rt(dt, y, at, load_act_rt(dt, y, at) + load_act_rt(dt, bias, c));
+}
+}  // namespace
+
+hipError_t launch_bias_add(void* y, const void* bias, uint32_t rows, uint32_t out, int dtype, hipStream_t s) {
+    for (uint32_t r0 = 0; r0 < rows; r0 += 65535u) {  // grid.y holds 65535 rows a launch
+        const uint32_t part = rows - r0 < 65535u ? rows - r0 : 65535u;
+        void* yp = static_cast<unsigned char*>(y) + static_cast<size_t>(r0) * out * (dtype == kF32 ? 4u : 2u);
+        hipLaunchKernelGGL(bias_add, dim3((out + 255u) / 256u, part), dim3(256), 0, s, yp, bias, out, dtype);
+        if (const hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
 hipError_t launch_dense_prep(const DenseLaunch& d, hipStream_t s) {
     hipLaunchKernelGGL(dense_prep, dim3(d.in / 128u, d.rows), dim3(64), 0, s, d.x, d.suh, d.xq, d.xs, d.in, d.dtype);
     return hipGetLastError();

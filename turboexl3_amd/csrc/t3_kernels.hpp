@@ -72,6 +72,7 @@ struct MoeLaunch {
     uint32_t per_gu = 8, per_dn = 4, parts_gu = 0, parts_dn = 0, ks_gu = 1, ks_dn = 1, bt_gu = 8, bt_dn = 8;
     int codebook = 0, dtype = 0, score_dt = 0, defer = 0;
     float limit = 0.0f;
+    int clamp_at = 0;  // format.ClampAt: 0 gate_in (the gate clamped before its SiLU), 1 silu_out (the SiLU's output)
     // prefill only (the route's roles, src/hip/plan.zig:40-45): row-slots sorted by expert. order [P] position ->
     // row-slot, inv [P] row-slot -> position (~0: skipped), items [max_items] {expert, first position, rows, 0},
     // counts [E + S + 4]: per-expert counts, then the item count and the placed total; cursor [E + S].
@@ -98,6 +99,9 @@ hipError_t launch_dense_prefill(const DenseLaunch& d, hipStream_t s);
 // finish of an f16 z [rows][out].
 hipError_t launch_dense_prep_natural(const DenseLaunch& d, uint16_t* xp, hipStream_t s);
 hipError_t launch_dense_finish_half(const DenseLaunch& d, const uint16_t* z, hipStream_t s);
+
+// y += bias in y's dtype (root.linearBias: one add after the projection's own output rounding)
+hipError_t launch_bias_add(void* y, const void* bias, uint32_t rows, uint32_t out, int dtype, hipStream_t s);
 
 // trellis [in/16][out/16][n] -> W_hat f16 [in][out], bit-exact (format.reconstructInner)
 hipError_t launch_dequant(const uint32_t* trellis, uint16_t* w_hat, uint32_t in, uint32_t out, uint32_t n,

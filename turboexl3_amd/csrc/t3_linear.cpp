@@ -207,6 +207,22 @@ int32_t t3_linear(t3_stream stream, const t3_array* x, const t3_array* trellis, 
     return t3::run_fused(call, static_cast<hipStream_t>(stream));
 }
 
+int32_t t3_linear_bias(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
+                       const t3_array* svh, const t3_array* bias, t3_decode dec, t3_array* y, void* workspace,
+                       size_t workspace_bytes) {
+    // root.linearBias's own checks (src/root.zig:365-370), then `linear`, then one add in x's dtype
+    if (!t3::array_ok(bias) || !t3::array_ok(trellis) || !t3::array_ok(x)) return T3_BadArgs;
+    if (trellis->ndim != 3 || bias->ndim != 1 || bias->shape[0] != trellis->shape[1] * 16) return T3_BadExl3Shape;
+    if (bias->dtype != x->dtype) return T3_BadExl3Dtype;
+    if (const int32_t st = t3_linear(stream, x, trellis, suh, svh, dec, y, workspace, workspace_bytes); st != T3_OK)
+        return st;
+    int64_t rows = 1;
+    for (int i = 0; i + 1 < x->ndim; ++i) rows *= x->shape[i];
+    return t3::hip_status(t3::launch_bias_add(y->data, bias->data, static_cast<uint32_t>(rows),
+                                              static_cast<uint32_t>(bias->shape[0]), x->dtype,
+                                              static_cast<hipStream_t>(stream)));
+}
+
 int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_array* w_hat) {
     if (!t3::array_ok(trellis) || !t3::array_ok(w_hat)) return T3_BadArgs;
     if (trellis->ndim != 3 || w_hat->ndim != 2) return T3_BadExl3Shape;

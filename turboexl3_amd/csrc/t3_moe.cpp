@@ -58,7 +58,7 @@ int32_t check_bank(const t3_bank* bank, int64_t hidden, RoutedBank* out, int64_t
 // root.validateCall (src/root.zig:128-141) and the partition of the decode chain.
 int32_t check_moe(const t3_array* x, const t3_bank* bank, const t3_array* inds, const t3_array* scores,
                   const t3_bank* shared_bank, const t3_array* shared_add, t3_decode dec, int32_t limit,
-                  const t3_array* y, MoeCall* call) {
+                  const t3_array* y, MoeCall* call, int32_t clamp_at = 0) {
     if (!array_ok(x) || !array_ok(inds) || (scores && !array_ok(scores)) || (y && !array_ok(y)) ||
         (shared_add && !array_ok(shared_add)))
         return T3_BadArgs;
@@ -118,6 +118,7 @@ int32_t check_moe(const t3_array* x, const t3_bank* bank, const t3_array* inds, 
     l.defer = d.gemv_form == 2;
     l.dtype = x->dtype;
     l.limit = static_cast<float>(limit);
+    l.clamp_at = clamp_at;
     // Partitions: functions of the bank's shapes alone. gate|up: a part is one 128-block of the input (8 tiles), so a
     // wave can prepare its own block; down: 4 tiles a part, its input being prepared by the mid launch.
     l.bt_gu = gemv_bt(l.n_gu);
@@ -191,10 +192,11 @@ int32_t admit_prefill(const MoeCall& call) {
 
 int32_t run_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
                 const t3_array* scores, const t3_bank* shared_bank, const t3_array* shared_add, t3_decode dec,
-                int32_t limit, t3_array* y, void* workspace, size_t workspace_bytes) {
+                int32_t limit, t3_array* y, void* workspace, size_t workspace_bytes, int32_t clamp_at = 0) {
     if (!scores || !y) return T3_BadArgs;
     MoeCall call;
-    if (const int32_t st = check_moe(x, bank, inds, scores, shared_bank, shared_add, dec, limit, y, &call); st != T3_OK)
+    if (const int32_t st = check_moe(x, bank, inds, scores, shared_bank, shared_add, dec, limit, y, &call, clamp_at);
+        st != T3_OK)
         return st;
     if (!workspace) return T3_BadArgs;
     // rows above the decode chain's take the prefill GEMM chain (src/root.zig:850-853)
@@ -252,6 +254,13 @@ int32_t t3_moe_clamped(t3_stream stream, const t3_array* x, const t3_bank* bank,
                        size_t workspace_bytes) {
     if (limit <= 0 || limit > 128) return T3_InvalidExl3Clamp;
     return t3::run_moe(stream, x, bank, inds, scores, nullptr, nullptr, dec, limit, y, workspace, workspace_bytes);
+}
+
+int32_t t3_moe_swiglu(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
+                      const t3_array* scores, t3_decode dec, int32_t limit, int32_t clamp_at, t3_array* y,
+                      void* workspace, size_t workspace_bytes) {
+    if (limit < 0 || limit > 128 || (clamp_at != T3_CLAMP_GATE_IN && clamp_at != T3_CLAMP_SILU_OUT)) return T3_InvalidExl3Clamp;
+    return t3::run_moe(stream, x, bank, inds, scores, nullptr, nullptr, dec, limit, y, workspace, workspace_bytes, clamp_at);
 }
 
 int32_t t3_moe_with_shared(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,

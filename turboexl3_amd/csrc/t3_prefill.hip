@@ -463,12 +463,7 @@ __global__ void __launch_bounds__(256) pf_mid(const MoeLaunch a) {
         float d[2];
 #pragma unroll
         for (uint32_t j = 0; j < 2u; ++j) {
-            float gv = g[j], uv = up[j];
-            if (a.limit > 0.0f) {  // comparisons: a NaN passes through (ref.zig:132-140)
-                gv = gv > a.limit ? a.limit : gv;
-                uv = uv > a.limit ? a.limit : (uv < -a.limit ? -a.limit : uv);
-            }
-            d[j] = round_half((gv / (1.0f + expf(-gv))) * uv) * sdn[u][j];
+            d[j] = round_half(swiglu_clamped(g[j], up[j], a.limit, a.clamp_at)) * sdn[u][j];
         }
         uint32_t hv[2];
         float sum;

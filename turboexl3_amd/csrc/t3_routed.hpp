@@ -110,12 +110,7 @@ __device__ __forceinline__ void routed_mid_block(const MoeLaunch& a, uint32_t rk
     float d[2];
 #pragma unroll
     for (uint32_t j = 0; j < 2u; ++j) {
-        float gv = g[j], uv = u[j];
-        if (a.limit > 0.0f) {  // comparisons: a NaN passes through (ref.zig:132-140)
-            gv = gv > a.limit ? a.limit : gv;
-            uv = uv > a.limit ? a.limit : (uv < -a.limit ? -a.limit : uv);
-        }
-        const float hv = round_half((gv / (1.0f + expf(-gv))) * uv);
+        const float hv = round_half(swiglu_clamped(g[j], u[j], a.limit, a.clamp_at));
         d[j] = hv * half_value(bank.down_suh[static_cast<size_t>(s.e) * a.inter + b * 128u + lane + 64u * j]);
     }
     h128_wave(d, lane);

@@ -64,4 +64,17 @@ __device__ __forceinline__ void finish_values(float (&s)[2], const uint16_t* svh
     finish_core(s, sv, lane);
 }
 
+// One element's SwiGLU in f32 on the f16-valued gate and up, with the clamp (turboexl3 src/core/ref.zig:119-140): limit 0
+// none; clamp_at 0 (gate_in) silu(min(g, L)) * clamp(u, -L, L); clamp_at 1 (silu_out) min(silu(g), L) * clamp(u, -L, L).
+// Comparisons, so a NaN passes through.
+__device__ __forceinline__ float swiglu_clamped(float g, float u, float limit, int clamp_at) {
+    if (limit > 0.0f) {
+        u = u > limit ? limit : (u < -limit ? -limit : u);
+        if (clamp_at == 0) g = g > limit ? limit : g;
+    }
+    float sg = g / (1.0f + expf(-g));
+    if (limit > 0.0f && clamp_at != 0) sg = sg > limit ? limit : sg;
+    return sg * u;
+}
+
 }  // namespace t3
