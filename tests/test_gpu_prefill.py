@@ -207,3 +207,21 @@ def test_trellis_gemm_every_live_block_count(oracle, t3):
                 assert worst <= F32_BAR, f"codebook {codebook} rows {rows}: {worst:.3e}"
         finally:
             t3.configure()
+
+
+def test_routed_prefill_many_experts_and_wide_topk(oracle, t3):
+    """More experts than the route's scan handles in one pass (1024), most of them without a row, and the widest
+    top-k (32)."""
+    rng = np.random.default_rng(0xE11)
+    hidden, inter, experts, topk, rows = 128, 128, 1100, 32, 24
+    bank = oracle.synth_bank(rng, experts, hidden, inter, 32)
+    dbank = dev_bank(t3, bank)
+    ref = RefBank(oracle, bank, MUL1, 0xFFFF)
+    x_dev, x_f32 = make_x(rng, rows, hidden, torch.float32)
+    slots = np.stack([rng.permutation(experts)[:topk] for _ in range(rows)]).astype(np.int32)
+    slots[:, 0] = experts - 1 - np.arange(rows)  # the last experts are used too
+    scores = (0.01 + rng.random((rows, topk)) * 0.05).astype(np.float32)
+    y = to_f32(t3.moe(x_dev.reshape(1, rows, hidden), dbank, torch.from_numpy(slots).cuda().reshape(1, rows, topk),
+                      torch.from_numpy(scores).cuda().reshape(1, rows, topk), t3.Decode.mul1)).reshape(rows, hidden)
+    for r in (0, 11, rows - 1):
+        assert oracle.compare(y[r], ref.row(x_f32[r], slots[r], scores[r])) <= F32_BAR
