@@ -37,16 +37,16 @@ __global__ void __launch_bounds__(64) moe_prep(const MoeLaunch a) {
 // gate|up -> the slot's mid block (counter a (row-slot, block of inter)); down -> the row's combine block (counter a
 // (row, block of hidden); skipped slots count themselves in too). The statements are the chain's, so are the bytes.
 template <int CB, bool WIDE, int BT, int NPROJ, bool XLDS, bool ARRIVE>
-__global__ void __launch_bounds__(256) moe_gemv(const MoeLaunch a) {
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ? 2 : 4))) moe_gemv(const MoeLaunch a) {
     // Two tile rows in flight a wave (measured: all 8 in flight is no faster; a call's time is its chain of dependent
     // round trips, not the depth of one wave's ring)
     constexpr int ST = 2;
     constexpr uint32_t kStage = gemv_stage_bytes<BT>();
-    constexpr uint32_t kRed = 4u * BT * 64u * 16u;
+    constexpr uint32_t kRed = 4u * BT * 4u * 16u;  // the one live row: four lanes a tile a wave
     constexpr uint32_t kMain = kRed > 4u * kStage ? kRed : 4u * kStage;
     __shared__ __attribute__((aligned(16))) unsigned char smem[kMain];
     __shared__ uint32_t last_flag;
-    float4v(*red)[BT * 64] = reinterpret_cast<float4v(*)[BT * 64]>(smem);
+    float4v(*red)[BT * 4] = reinterpret_cast<float4v(*)[BT * 4]>(smem);
     const uint32_t blk = blockIdx.x, rk = blockIdx.y / NPROJ, proj = blockIdx.y % NPROJ, ksl = blockIdx.z;
     const uint32_t sg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
     const SlotRef s = resolve_slot(a, rk);
@@ -113,16 +113,16 @@ __global__ void __launch_bounds__(256) moe_gemv(const MoeLaunch a) {
         }
     }
     __syncthreads();
-#pragma unroll
-    for (int t = 0; t < BT; ++t) red[sg][t * 64 + lane] = acc[0][t];
-    __syncthreads();
     // activation row 0 of the fragment is the slot's row: lanes with lane % 16 == 0 hold its sums
+    if ((lane & 15u) == 0u)
+#pragma unroll
+        for (int t = 0; t < BT; ++t) red[sg][t * 4 + (lane >> 4)] = acc[0][t];
+    __syncthreads();
     float* z = NPROJ == 1 ? a.zd : (proj ? a.zu : a.zg);
-    for (uint32_t i = threadIdx.x; i < static_cast<uint32_t>(BT * 64); i += 256u) {
-        const uint32_t l = i & 63u, t = i >> 6;
-        if ((l & 15u) != 0u) continue;
+    if (threadIdx.x < static_cast<uint32_t>(BT * 4)) {
+        const uint32_t i = threadIdx.x, t = i >> 2;
         const float4v v = ((red[0][i] + red[1][i]) + red[2][i]) + red[3][i];
-        float* dst = z + (static_cast<size_t>(ksl) * rkt + rk) * out + (blk * BT + t) * 16u + 4u * (l >> 4);
+        float* dst = z + (static_cast<size_t>(ksl) * rkt + rk) * out + (blk * BT + t) * 16u + 4u * (i & 3u);
         if constexpr (ARRIVE) {
             if (s.live)
 #pragma unroll
