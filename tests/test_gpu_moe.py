@@ -117,8 +117,9 @@ def test_moe_decode_rows_1_to_16(oracle, t3, hidden, inter, experts, topk, n, co
 
 
 def test_launch_forms_give_the_same_bytes(oracle, t3):
-    # src/hip_tests.zig:885-928: form 9's bytes are form 3's. Here: two launches (default), four, five; twice in a row
-    # (the arrival counters go back to zero), with skipped slots, a clamp and a shared expert in the same launches
+    # src/hip_tests.zig:885-928: form 9's bytes are form 3's. Here: two launches (default), four, five; twice in a
+    # row (the arrival counters go back to zero), with skipped slots, a clamp and a shared expert in
+    # the same launches
     rng = np.random.default_rng(9)
     for codebook, n, rows, topk in ((MCG, 64, 5, 4), (MUL1, 48, 16, 4), (MUL1, 96, 3, 2)):
         bank = oracle.synth_bank(rng, 8, 512, 256, n)
@@ -144,6 +145,9 @@ def test_launch_forms_give_the_same_bytes(oracle, t3):
                 finally:
                     t3.configure()
                 assert bytes_of(nine) == bytes_of(other), f"form 9 differs from form {form}"
+    # every call left the workspace's counter area zero
+    for ws in t3._workspaces.values():
+        assert not ws[:65536].any()
 
 
 def test_clamp_skipped_slots_and_score_dtypes(oracle, t3):

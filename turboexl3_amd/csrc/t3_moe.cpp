@@ -208,8 +208,8 @@ int32_t run_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const 
     }
     carve_moe(&call, workspace);
     if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
-    // decode_form 3: the five-launch chain; 9: two launches while a counter a (row-slot, 128-block) fits the
-    // workspace's counter area, else four
+    // decode_form 3: the five-launch chain; 4: four launches; 9: two launches while a counter a (row-slot, 128-block)
+    // fits the workspace's counter area, else four
     const MoeLaunch& l = call.launch;
     const size_t widest = (l.hidden > l.inter ? l.hidden : l.inter) / 128u;
     const size_t counters = static_cast<size_t>(l.rows) * (l.topk + l.shared_slots) * widest;

@@ -36,22 +36,37 @@ __global__ void __launch_bounds__(64) moe_prep(const MoeLaunch a) {
 // itself in at its 128-column block, and the last to arrive runs that block's next stage on the complete planes:
 // gate|up -> the slot's mid block (counter a (row-slot, block of inter)); down -> the row's combine block (counter a
 // (row, block of hidden); skipped slots count themselves in too). The statements are the chain's, so are the bytes.
+// a workgroup's static LDS: the four waves' stages while they stream, their partial sums afterwards
+template <int BT>
+constexpr uint32_t role_lds_bytes() {
+    constexpr uint32_t stage = 4u * gemv_stage_bytes<BT>(), red = 4u * BT * 4u * 16u;
+    return stage > red ? stage : red;
+}
+
 template <int CB, bool WIDE, int BT, int NPROJ, bool XLDS, bool ARRIVE>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ? 2 : 4))) moe_gemv(const MoeLaunch a) {
+__device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint32_t yidx, uint32_t ksl,
+                                          unsigned char* smem, uint32_t& last_flag, uint32_t* cinfo, float* cscore) {
     // Two tile rows in flight a wave (measured: all 8 in flight is no faster; a call's time is its chain of dependent
     // round trips, not the depth of one wave's ring)
     constexpr int ST = 2;
     constexpr uint32_t kStage = gemv_stage_bytes<BT>();
-    constexpr uint32_t kRed = 4u * BT * 4u * 16u;  // the one live row: four lanes a tile a wave
-    constexpr uint32_t kMain = kRed > 4u * kStage ? kRed : 4u * kStage;
-    __shared__ __attribute__((aligned(16))) unsigned char smem[kMain];
-    __shared__ uint32_t last_flag;
-    float4v(*red)[BT * 4] = reinterpret_cast<float4v(*)[BT * 4]>(smem);
-    const uint32_t blk = blockIdx.x, rk = blockIdx.y / NPROJ, proj = blockIdx.y % NPROJ, ksl = blockIdx.z;
+    float4v(*red)[BT * 4] = reinterpret_cast<float4v(*)[BT * 4]>(smem);  // the one live row: four lanes a tile a wave
+    const uint32_t rk = yidx / NPROJ, proj = yidx % NPROJ;
     const uint32_t sg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
     const SlotRef s = resolve_slot(a, rk);
     // uniform over the workgroup; the down launch's arriving form still has to count a skipped slot in
     if (!s.live && !(ARRIVE && NPROJ == 1)) return;
+    if constexpr (ARRIVE && NPROJ == 1) {
+        // What the combine will need of the row's slots, fetched now: the workgroup that arrives last would otherwise
+        // wait for two dependent loads a slot at the very end of the call. cinfo: the expert, bit 31 for a shared
+        // slot, all ones for a skipped one.
+        const uint32_t kt = a.topk + a.shared_slots;
+        if (threadIdx.x < kt) {
+            const SlotRef sk = resolve_slot(a, s.row * kt + threadIdx.x);
+            cinfo[threadIdx.x] = !sk.live ? 0xFFFFFFFFu : (sk.shared ? 0x80000000u | sk.e : sk.e);
+            cscore[threadIdx.x] = sk.shared ? 1.0f : (sk.live ? score_of(a, s.row, threadIdx.x) : 0.0f);
+        }
+    }
     const RoutedBank& bank = s.shared ? a.shared : a.bank;
     const uint32_t in = NPROJ == 2 ? a.hidden : a.inter, out = NPROJ == 2 ? a.inter : a.hidden;
     const uint32_t n = NPROJ == 2 ? a.n_gu : a.n_dn;
@@ -150,26 +165,38 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ?
         if (threadIdx.x == 0u)  // zero again for the next call
             __hip_atomic_store(a.arrive + counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if constexpr (NPROJ == 2) {
-            if (sg == 0u) routed_mid_block<false, true>(a, rk, rk, b128, lane);
+            if (sg == 0u) routed_mid_block<false, true>(a, s, rk, b128, lane);
         } else {
-            // the slots' finishes four at a time, one a wave; wave 0 adds them in slot order
+            // The slots' finishes sixteen at a time, four a wave (slot k0 + 4 r + wave) with every load of the four in
+            // flight together; wave 0 adds them in slot order.
             float(*fin)[128] = reinterpret_cast<float(*)[128]>(smem);
             float acc2[2] = {0.0f, 0.0f};
-            for (uint32_t k0 = 0; k0 < kt; k0 += 4u) {
-                const uint32_t k = k0 + sg;
-                if (k < kt) {
-                    float v[2];
-                    if (routed_down_finish<true>(a, s.row * kt + k, s.row * kt + k, b128, lane, v, ks)) {
-                        fin[sg][lane] = v[0];
-                        fin[sg][lane + 64u] = v[1];
-                    }
+            for (uint32_t k0 = 0; k0 < kt; k0 += 16u) {
+                SlotRef sk[4];
+                uint32_t qk[4];
+                float v[4][2];
+#pragma unroll
+                for (uint32_t r = 0; r < 4u; ++r) {
+                    const uint32_t k = k0 + 4u * r + sg;
+                    const uint32_t info = k < kt ? cinfo[k] : 0xFFFFFFFFu;
+                    sk[r].row = s.row;
+                    sk[r].live = info != 0xFFFFFFFFu;
+                    sk[r].shared = sk[r].live && (info >> 31) != 0u;
+                    sk[r].e = info & 0x7FFFFFFFu;
+                    qk[r] = s.row * kt + (k < kt ? k : 0u);
                 }
+                routed_down_finish_many<true, false, 4>(a, sk, qk, b128, lane, v, ks);
+#pragma unroll
+                for (uint32_t r = 0; r < 4u; ++r)
+                    if (sk[r].live) {
+                        fin[4u * r + sg][lane] = v[r][0];
+                        fin[4u * r + sg][lane + 64u] = v[r][1];
+                    }
                 __syncthreads();
                 if (sg == 0u)
-                    for (uint32_t w = 0; w < 4u && k0 + w < kt; ++w) {
-                        const SlotRef sw = resolve_slot(a, s.row * kt + k0 + w);
-                        if (!sw.live) continue;
-                        const float wgt = sw.shared ? 1.0f : score_of(a, s.row, k0 + w);
+                    for (uint32_t w = 0; w < 16u && k0 + w < kt; ++w) {
+                        if (cinfo[k0 + w] == 0xFFFFFFFFu) continue;
+                        const float wgt = cscore[k0 + w];
                         acc2[0] = __builtin_fmaf(wgt, fin[w][lane], acc2[0]);
                         acc2[1] = __builtin_fmaf(wgt, fin[w][lane + 64u], acc2[1]);
                     }
@@ -180,9 +207,18 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ?
     }
 }
 
+template <int CB, bool WIDE, int BT, int NPROJ, bool XLDS, bool ARRIVE>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ? 2 : 4))) moe_gemv(const MoeLaunch a) {
+    __shared__ __attribute__((aligned(16))) unsigned char smem[role_lds_bytes<BT>()];
+    __shared__ uint32_t last_flag, cinfo[64];
+    __shared__ float cscore[64];
+    gemv_role<CB, WIDE, BT, NPROJ, XLDS, ARRIVE>(a, blockIdx.x, blockIdx.y, blockIdx.z, smem, last_flag, cinfo,
+                                                        cscore);
+}
+
 // Grid (inter / 128, RKT), 64 threads.
 __global__ void __launch_bounds__(64) moe_mid(const MoeLaunch a) {
-    routed_mid_block<false>(a, blockIdx.y, blockIdx.y, blockIdx.x, threadIdx.x);
+    routed_mid_block<false>(a, resolve_slot(a, blockIdx.y), blockIdx.y, blockIdx.x, threadIdx.x);
 }
 
 // Grid (hidden / 128, rows), 64 threads.

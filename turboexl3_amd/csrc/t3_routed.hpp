@@ -41,18 +41,66 @@ __device__ __forceinline__ float score_of(const MoeLaunch& a, uint32_t row, uint
 
 // One block's sums over the K slices (slice order; the first plane starts the sum) and the deferred MUL1 map.
 // COH: the planes and block sums were stored by other workgroups of this launch.
+// Loads go out eight at a time and are added in slice (or block) order: the sums do not depend on the batching, and a
+// block's finish waits for one round trip, not for one a plane.
+template <bool COH>
+__device__ __forceinline__ float ordered_sum(const float* p, size_t stride, uint32_t count, bool first_starts) {
+    auto get = [](const float* q) { return COH ? load_coherent(q) : *q; };
+    float acc = 0.0f;
+    for (uint32_t k0 = 0; k0 < count; k0 += 8u) {
+        float part[8];
+#pragma unroll
+        for (uint32_t k = 0; k < 8u; ++k) part[k] = k0 + k < count ? get(p + (k0 + k) * stride) : 0.0f;
+#pragma unroll
+        for (uint32_t k = 0; k < 8u; ++k)
+            if (k0 + k < count) acc = first_starts && k0 + k == 0u ? part[k] : acc + part[k];  // 0 + z would turn -0 into +0
+    }
+    return acc;
+}
+
+// N such sums at once: every load of all of them goes out before the first add (up to 8 planes; more fall back to one
+// sum after the other). The same order of additions a sum as ordered_sum's.
+template <bool COH, int N>
+__device__ __forceinline__ void ordered_sums(const float* const (&p)[N], size_t stride, uint32_t count, float (&out)[N]) {
+    auto get = [](const float* q) { return COH ? load_coherent(q) : *q; };
+    if (count <= 8u) {
+        float part[N][8];
+#pragma unroll
+        for (int i = 0; i < N; ++i)
+#pragma unroll
+            for (uint32_t k = 0; k < 8u; ++k) part[i][k] = k < count ? get(p[i] + k * stride) : 0.0f;
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            float acc = part[i][0];
+#pragma unroll
+            for (uint32_t k = 1; k < 8u; ++k)
+                if (k < count) acc += part[i][k];
+            out[i] = acc;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) out[i] = ordered_sum<COH>(p[i], stride, count, true);
+    }
+}
+
+// 0 + p[0] + p[1] + ... in that order, the values fetched by one load across the wave's lanes (up to 64 of them)
+template <bool COH>
+__device__ __forceinline__ float lane_ordered_sum(const float* p, uint32_t count, uint32_t lane) {
+    if (count > 64u) return ordered_sum<COH>(p, 1u, count, false);
+    const float mine = lane < count ? (COH ? load_coherent(p + lane) : p[lane]) : 0.0f;
+    float acc = 0.0f;
+    for (uint32_t q = 0; q < count; ++q)
+        acc += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), static_cast<int>(q)));
+    return acc;
+}
+
 template <bool COH>
 __device__ __forceinline__ void plane_sums(const float* z, size_t planes_stride, uint32_t ks, const float* bsum,
                                            uint32_t nb, int defer, uint32_t lane, float (&s)[2]) {
-    auto get = [](const float* p) { return COH ? load_coherent(p) : *p; };
 #pragma unroll
-    for (uint32_t j = 0; j < 2u; ++j) s[j] = get(z + lane + 64u * j);
-    for (uint32_t k = 1; k < ks; ++k)
-#pragma unroll
-        for (uint32_t j = 0; j < 2u; ++j) s[j] += get(z + k * planes_stride + lane + 64u * j);
+    for (uint32_t j = 0; j < 2u; ++j) s[j] = ordered_sum<COH>(z + lane + 64u * j, planes_stride, ks, true);
     if (defer) {
-        float xsum = 0.0f;
-        for (uint32_t q = 0; q < nb; ++q) xsum += get(bsum + q);
+        const float xsum = ordered_sum<COH>(bsum, 1u, nb, false);
 #pragma unroll
         for (uint32_t j = 0; j < 2u; ++j) s[j] = __builtin_fmaf(s[j], mul1_a(), mul1_b() * xsum);
     }
@@ -94,25 +142,40 @@ __device__ __forceinline__ void routed_prep_block(const MoeLaunch& a, uint32_t r
 // gate and up finishes, the (clamped) SwiGLU in f32 on their f16 values, and the down's prepare: hd [.][inter],
 // hs f32 [.][inter / 128]
 template <bool PF, bool COH = false>
-__device__ __forceinline__ void routed_mid_block(const MoeLaunch& a, uint32_t rk, uint32_t q, uint32_t b,
+__device__ __forceinline__ void routed_mid_block(const MoeLaunch& a, const SlotRef& s, uint32_t q, uint32_t b,
                                                  uint32_t lane) {
-    const SlotRef s = resolve_slot(a, rk);
     if (!s.live) return;
     const RoutedBank& bank = s.shared ? a.shared : a.bank;
     const uint32_t rkt = a.rows * (a.topk + a.shared_slots), nb = a.hidden / 128u;
     const uint32_t ks = PF ? 1u : a.ks_gu;
     const size_t plane = static_cast<size_t>(rkt) * a.inter, at = static_cast<size_t>(q) * a.inter + b * 128u;
-    float g[2], u[2];
-    plane_sums<COH>(a.zg + at, plane, ks, a.sg + static_cast<size_t>(q) * nb, nb, a.defer, lane, g);
-    plane_sums<COH>(a.zu + at, plane, ks, a.su + static_cast<size_t>(q) * nb, nb, a.defer, lane, u);
-    finish_values(g, bank.gate_svh + static_cast<size_t>(s.e) * a.inter, b, lane);
-    finish_values(u, bank.up_svh + static_cast<size_t>(s.e) * a.inter, b, lane);
-    float d[2];
+    // every load of the block goes out together: one round trip, not one a plane and a projection
+    const size_t eo = static_cast<size_t>(s.e) * a.inter + b * 128u;
+    float svg[2], svu[2], sdn[2];
 #pragma unroll
     for (uint32_t j = 0; j < 2u; ++j) {
-        const float hv = round_half(swiglu_clamped(g[j], u[j], a.limit, a.clamp_at));
-        d[j] = hv * half_value(bank.down_suh[static_cast<size_t>(s.e) * a.inter + b * 128u + lane + 64u * j]);
+        svg[j] = half_value(bank.gate_svh[eo + lane + 64u * j]);
+        svu[j] = half_value(bank.up_svh[eo + lane + 64u * j]);
+        sdn[j] = half_value(bank.down_suh[eo + lane + 64u * j]);
     }
+    const float* const planes[4] = {a.zg + at + lane, a.zg + at + lane + 64u, a.zu + at + lane, a.zu + at + lane + 64u};
+    float sums[4];
+    ordered_sums<COH, 4>(planes, plane, ks, sums);
+    float g[2] = {sums[0], sums[1]}, u[2] = {sums[2], sums[3]};
+    if (a.defer) {
+        const float xg = lane_ordered_sum<COH>(a.sg + static_cast<size_t>(q) * nb, nb, lane);
+        const float xu = lane_ordered_sum<COH>(a.su + static_cast<size_t>(q) * nb, nb, lane);
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j) {
+            g[j] = __builtin_fmaf(g[j], mul1_a(), mul1_b() * xg);
+            u[j] = __builtin_fmaf(u[j], mul1_a(), mul1_b() * xu);
+        }
+    }
+    finish_core(g, svg, lane);
+    finish_core(u, svu, lane);
+    float d[2];
+#pragma unroll
+    for (uint32_t j = 0; j < 2u; ++j) d[j] = round_half(swiglu_clamped(g[j], u[j], a.limit, a.clamp_at)) * sdn[j];
     h128_wave(d, lane);
     float sum = 0.0f;
 #pragma unroll
@@ -128,29 +191,62 @@ __device__ __forceinline__ void routed_mid_block(const MoeLaunch& a, uint32_t rk
 
 // One slot's finished down outputs of block b (f16-valued), false for a skipped slot. COH: only the planes cross
 // workgroups inside the launch; the block sums hs came from the launch before.
-template <bool COH>
-__device__ __forceinline__ bool routed_down_finish(const MoeLaunch& a, uint32_t rk, uint32_t q, uint32_t b,
+template <bool COH, bool HS_COH = false>
+__device__ __forceinline__ bool routed_down_finish(const MoeLaunch& a, const SlotRef& s, uint32_t q, uint32_t b,
                                                    uint32_t lane, float (&v)[2], uint32_t ks) {
-    const SlotRef s = resolve_slot(a, rk);
     if (!s.live) return false;  // uniform over the wave
     const uint32_t rkt = a.rows * (a.topk + a.shared_slots), nbi = a.inter / 128u;
     const RoutedBank& bank = s.shared ? a.shared : a.bank;
     const float* z = a.zd + static_cast<size_t>(q) * a.hidden + b * 128u;
     const size_t plane = static_cast<size_t>(rkt) * a.hidden;
-    auto get = [](const float* p) { return COH ? load_coherent(p) : *p; };
+    // the block's scales go out with the planes, not after them
+    const uint16_t* svh = bank.down_svh + static_cast<size_t>(s.e) * a.hidden + b * 128u;
+    const float sv[2] = {half_value(svh[lane]), half_value(svh[lane + 64u])};
 #pragma unroll
-    for (uint32_t j = 0; j < 2u; ++j) v[j] = get(z + lane + 64u * j);
-    for (uint32_t k = 1; k < ks; ++k)
-#pragma unroll
-        for (uint32_t j = 0; j < 2u; ++j) v[j] += get(z + k * plane + lane + 64u * j);
+    for (uint32_t j = 0; j < 2u; ++j) v[j] = ordered_sum<COH>(z + lane + 64u * j, plane, ks, true);
     if (a.defer) {
-        float xsum = 0.0f;
-        for (uint32_t i = 0; i < nbi; ++i) xsum += a.hs[static_cast<size_t>(q) * nbi + i];
+        const float xsum = ordered_sum<HS_COH>(a.hs + static_cast<size_t>(q) * nbi, 1u, nbi, false);
 #pragma unroll
         for (uint32_t j = 0; j < 2u; ++j) v[j] = __builtin_fmaf(v[j], mul1_a(), mul1_b() * xsum);
     }
-    finish_values(v, bank.down_svh + static_cast<size_t>(s.e) * a.hidden, b, lane);
+    finish_core(v, sv, lane);
     return true;
+}
+
+// R slots' finished down outputs of block b at once (a skipped slot's entry is left alone): all their planes, scales
+// and block sums are fetched together. q[r]: where slot r's scratch lives.
+template <bool COH, bool HS_COH, int R>
+__device__ __forceinline__ void routed_down_finish_many(const MoeLaunch& a, const SlotRef (&s)[R], const uint32_t (&q)[R],
+                                                        uint32_t b, uint32_t lane, float (&v)[R][2], uint32_t ks) {
+    const uint32_t rkt = a.rows * (a.topk + a.shared_slots), nbi = a.inter / 128u;
+    const size_t plane = static_cast<size_t>(rkt) * a.hidden;
+    const float* planes[2 * R];
+    float sv[R][2], sums[2 * R], xsum[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        // a skipped slot reads its own (unwritten) scratch and expert 0's scales: valid memory, values unused
+        const RoutedBank& bank = s[r].live && s[r].shared ? a.shared : a.bank;
+        const uint16_t* svh = bank.down_svh + static_cast<size_t>(s[r].live ? s[r].e : 0u) * a.hidden + b * 128u;
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j) {
+            sv[r][j] = half_value(svh[lane + 64u * j]);
+            planes[2 * r + j] = a.zd + static_cast<size_t>(q[r]) * a.hidden + b * 128u + lane + 64u * j;
+        }
+    }
+    ordered_sums<COH, 2 * R>(planes, plane, ks, sums);
+    if (a.defer)
+#pragma unroll
+        for (int r = 0; r < R; ++r) xsum[r] = lane_ordered_sum<HS_COH>(a.hs + static_cast<size_t>(q[r]) * nbi, nbi, lane);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (!s[r].live) continue;  // uniform over the wave
+        v[r][0] = sums[2 * r];
+        v[r][1] = sums[2 * r + 1];
+        if (a.defer)
+#pragma unroll
+            for (uint32_t j = 0; j < 2u; ++j) v[r][j] = __builtin_fmaf(v[r][j], mul1_a(), mul1_b() * xsum[r]);
+        finish_core(v[r], sv[r], lane);
+    }
 }
 
 // a row's block b from its f32 sums: y's dtype, or `moeWithShared`'s two roundings
@@ -181,7 +277,7 @@ __device__ __forceinline__ void routed_combine_block(const MoeLaunch& a, uint32_
         const SlotRef s = resolve_slot(a, rk);
         if (!s.live) continue;  // uniform over the wave
         float v[2];
-        routed_down_finish<false>(a, rk, PF ? a.inv[rk] : rk, b, lane, v, PF ? 1u : a.ks_dn);
+        routed_down_finish<false>(a, s, PF ? a.inv[rk] : rk, b, lane, v, PF ? 1u : a.ks_dn);
         const float w = s.shared ? 1.0f : score_of(a, row, k);
 #pragma unroll
         for (uint32_t j = 0; j < 2u; ++j) acc[j] = __builtin_fmaf(w, v[j], acc[j]);
