@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--sweep]
 
-A step is one `linear` call of the dense decode-row GEMV workload BASELINE.json quotes its metric on
+A step is one `linear` call of the dense decode-row GEMV workload the headline metric is quoted on
 (in=4096, out=12288, K=4 bits/weight, 1 row, MCG codebook, f16 activations with 1 % outliers x20; synthetic seeded
 codes). Calls rotate over enough distinct weight copies (> 512 MB in total) that every call reads its codes from
 HBM, not from the 256 MB Infinity Cache. Inputs are resident in HBM before the timed region starts.
@@ -11,7 +11,7 @@ HBM, not from the 256 MB Infinity Cache. Inputs are resident in HBM before the t
 Prints ONE JSON line: the whole-call rate as GB/s of trellis code bytes (`value`), the dominant kernel's roofline
 (`roofline`: algorithmic code bytes of one launch / its average duration, timed alone with HIP events on the launch
 stream, against 8 TB/s), and the CPU oracle (`format.project` restated in C) timed on this box's host cores
-(`cpu_baseline`). The same line carries the other configurations of BASELINE.json as extra objects: `moe_decode`
+(`cpu_baseline`). The same line carries the other benchmark configurations as extra objects: `moe_decode`
 (config 3: routed decode at 1 and 8 tokens), `moe_prefill` (config 4: the routed prefill chain, TFLOP/s against the
 2.5 PFLOP/s dense f16 MFMA peak) and `dense_prefill` (config 5: 4096 rows); `--quick` leaves them out. `--sweep` adds
 K = 3, 4, 5 x rows = 1, 4, 16, 32; `--in-f/--out-f/--k/--rows` time another dense shape (lm_head: --in-f 4096
@@ -123,7 +123,7 @@ class DenseRunner:
 
 
 class MoeRunner:
-    """BASELINE config 3: 512 experts, hidden 2048, inter 512, K3, top-10, clamp 7, one shared expert (inter 512) in the
+    """Benchmark configuration 3: 512 experts, hidden 2048, inter 512, K3, top-10, clamp 7, one shared expert (inter 512) in the
     same launches. Every call routes to a fresh set of experts (a rotation of disjoint routings) so the codes come from
     HBM: the bank alone is 604 MB."""
 
@@ -189,7 +189,7 @@ class MoeRunner:
 
 
 class PrefillRunner:
-    """BASELINE config 4: 2048 tokens, 256 experts, top-8, hidden 7168, inter 2048, gate|up K2, down K3, bf16, clamp 7.
+    """Benchmark configuration 4: 2048 tokens, 256 experts, top-8, hidden 7168, inter 2048, gate|up K2, down K3, bf16, clamp 7.
     flops = tokens * topk * 3 * 2 * hidden * inter. `scale` shrinks experts and tokens together (same rows an expert)."""
 
     def __init__(self, torch, api, tokens=2048, experts=256, topk=8, hidden=7168, inter=2048, k_gu=2, k_dn=3, seed=9):

@@ -1,4 +1,4 @@
-"""The BASELINE configurations at their full sizes: decoded weights bit-exact, sampled rows (and, where a whole row is
+"""The benchmark configurations at their full sizes: decoded weights bit-exact, sampled rows (and, where a whole row is
 too much for the CPU oracle, sampled 128-column output blocks, which are independent of the rest of the row) within
 the reference's bars, and the size-independent byte equalities."""
 import numpy as np
