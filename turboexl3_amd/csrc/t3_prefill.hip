@@ -22,9 +22,11 @@ namespace t3 {
 namespace {
 
 constexpr uint32_t kPfSlot = 256;          // LDS bytes a staged tile
-constexpr uint32_t kPfRowStride = 80;      // LDS bytes an activation row a step: 64 + 16 so 16 rows hit 16 bank groups
-// a wave's stage: two tile rows of NT tiles, then the dump of the idle lanes
-constexpr uint32_t pf_stage_bytes(uint32_t nt) { return 2u * nt * kPfSlot + 1024u; }
+// LDS bytes an activation row a step: 64 + 32. Measured on gfx950: a wave's 16-byte reads at row stride 96 (or 64 with
+// an xor swizzle) take 4.2 cycles, at stride 64 or 80 they take 8.
+constexpr uint32_t kPfRowStride = 96;
+// a wave's stage: two tile rows of NT tiles
+constexpr uint32_t pf_stage_bytes(uint32_t nt) { return 2u * nt * kPfSlot; }
 
 struct PfGemm {
     const uint32_t* w[2];    // the bank's trellis a projection (gate, up) or (down, -)
@@ -143,13 +145,16 @@ __global__ void __launch_bounds__(256) pf_gemm(const PfGemm a) {
 
     const QuadPlan<WIDE> plan = quad_plan<WIDE>(a.n, lane);
     const uint32_t inv_tile = (1u << 16) / tile_bytes + 1u;
+    // A lane's 16 bytes of a tile row's chunk go to the tiles' slots: in one piece where a tile is whole 16-byte
+    // pieces (every integer rate), else word by word. Lanes past the chunk write nothing.
     const bool writer = lane * 16u < chunk_bytes;
+    const bool whole = (tile_bytes & 15u) == 0u;  // uniform
     uint32_t put[4];
 #pragma unroll
     for (uint32_t jj = 0; jj < 4u; ++jj) {
         const uint32_t b = lane * 16u + 4u * jj;
         const uint32_t t = (b * inv_tile) >> 16;
-        put[jj] = writer ? t * kPfSlot + (b - t * tile_bytes) : 2u * kPfTiles * kPfSlot + lane * 16u + 4u * jj;
+        put[jj] = t * kPfSlot + (b - t * tile_bytes);
     }
     const uint32_t get_bp = plan.ib_prev * 4u, get_bl = plan.ib_last * 4u;
     const uint32_t get_ap = plan.ia_prev * 4u, get_al = plan.ia_last * 4u;
@@ -159,11 +164,18 @@ __global__ void __launch_bounds__(256) pf_gemm(const PfGemm a) {
         dst[1] = buf_load_u128(wres, wvoff, (2u * step + 1u) * wstep);
     };
     auto stage_w = [&](const uint4v(&src)[2]) {
+        if (!writer) return;
+        if (whole) {
 #pragma unroll
-        for (uint32_t r = 0; r < 2u; ++r)
+            for (uint32_t r = 0; r < 2u; ++r)
+                *reinterpret_cast<uint4v*>(stage + r * (kPfTiles * kPfSlot) + put[0]) = src[r];
+        } else {
 #pragma unroll
-            for (uint32_t jj = 0; jj < 4u; ++jj)
-                *reinterpret_cast<uint32_t*>(stage + (writer ? r * (kPfTiles * kPfSlot) : 0u) + put[jj]) = src[r][jj];
+            for (uint32_t r = 0; r < 2u; ++r)
+#pragma unroll
+                for (uint32_t jj = 0; jj < 4u; ++jj)
+                    *reinterpret_cast<uint32_t*>(stage + r * (kPfTiles * kPfSlot) + put[jj]) = src[r][jj];
+        }
     };
     auto fetch_w = [&](QuadWords<WIDE>(&wd)[2][kPfTiles]) {
 #pragma unroll
