@@ -103,6 +103,15 @@ __device__ __forceinline__ uint32_t quad_slot(uint32_t r) {
     return 4u * q + m;
 }
 
+// Where input i of a row sits in the prepared activations the GEMM reads ("pair-quad order"): inside every 32 inputs
+// (two tile rows A, B), quad q of A then quad q of B, q = 0..3: the 16 bytes at q are the eight K slots of the MFMA's B
+// fragment that meet a lane's eight weights (tile rows 2q + {0, 1, 8, 9} of A, then of B).
+__device__ __forceinline__ uint32_t pair_quad_slot(uint32_t i) {
+    const uint32_t r = i & 15u;
+    const uint32_t q = (r & 7u) >> 1u, m = (r & 1u) | ((r >> 3u) << 1u);
+    return (i & ~31u) + 8u * q + 4u * ((i >> 4u) & 1u) + m;
+}
+
 // MUL1's affine map w = A h + B with h = 1024 + t (format.zig:158-167): A = f16 0x1EEE, B = f16 0xC931
 __device__ __forceinline__ float mul1_a() { return half_value(0x1EEEu); }
 __device__ __forceinline__ float mul1_b() { return half_value(0xC931u); }

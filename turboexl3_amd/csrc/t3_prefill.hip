@@ -21,21 +21,18 @@
 namespace t3 {
 namespace {
 
-constexpr uint32_t kPfSlot = 256;          // LDS bytes a staged tile
-// LDS bytes an activation row a step: 64 + 32. Measured on gfx950: a wave's 16-byte reads at row stride 96 (or 64 with
-// an xor swizzle) take 4.2 cycles, at stride 64 or 80 they take 8.
-constexpr uint32_t kPfRowStride = 96;
-// a wave's stage: two tile rows of NT tiles
-constexpr uint32_t pf_stage_bytes(uint32_t nt) { return 2u * nt * kPfSlot; }
+constexpr uint32_t kPfSlot = 256;   // LDS bytes a tile's words take (a tile is at most 256 bytes)
+constexpr uint32_t kPfTiles = 4;    // adjacent tiles a wave
+constexpr uint32_t kPfWaveStep = 2u * kPfTiles * kPfSlot;  // LDS bytes of a wave's weight words a step (two tile rows)
 
 struct PfGemm {
     const uint32_t* w[2];    // the bank's trellis a projection (gate, up) or (down, -)
     const uint32_t* ws[2];   // the shared bank's: experts numbered from `experts` up
-    const uint16_t* xq[2];   // prepared activations f16 [positions][in], quad order
+    const uint16_t* xq[2];   // prepared activations f16 [positions][in], pair-quad order
     float* z[2];             // f32 [positions][out]
     const uint32_t* items;   // {expert, first position, rows, 0} an item; null: dense, item i = rows i RB 16 ...
     const uint32_t* n_items; // the route's item count (device)
-    uint32_t in, out, n, wbits, positions, experts, nblk;  // nblk: workgroup columns (64 NT output columns each)
+    uint32_t in, out, n, wbits, positions, experts, nblk;  // nblk: workgroup columns (256 output columns each)
 };
 
 // The weight a GEMM feeds the matrix core as one f16: exact, or MUL1's h = 1024 + t when its map is deferred.
@@ -68,28 +65,57 @@ __device__ __forceinline__ uint32_t weight_halves(uint32_t cw_lo, uint32_t cw_hi
     }
 }
 
+// ---- loads that bypass the registers --------------------------------------------------------------------------
+// A raw buffer descriptor as four scalars, and a wave's load of 16 bytes a lane from it straight into LDS: lane L's
+// bytes land at lds + 16 L, from byte voff (the lane's) + soff (uniform) of the buffer; past the buffer's end they are
+// zeros. The compiler does not know these loads: the kernel counts them itself (wait_loads) and issues no other
+// vector memory load while they fly.
+__device__ __forceinline__ uint4v rsrc_words(const void* p, uint64_t bytes) {
+    const uint64_t addr = reinterpret_cast<uint64_t>(p);
+    const uint32_t n = bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : static_cast<uint32_t>(bytes);
+    return uint4v{static_cast<uint32_t>(addr), static_cast<uint32_t>(addr >> 32) & 0xFFFFu, n, 0x00020000u};
+}
+__device__ __forceinline__ void load_to_lds(uint4v desc, uint32_t lds, uint32_t voff, uint32_t soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds), "v"(voff), "s"(desc), "s"(soff)
+                 : "memory");
+}
+// at most N of the wave's loads are still in flight (they complete in order)
+template <int N>
+__device__ __forceinline__ void wait_loads() {
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
 // Grid (8 * nblk * ceil(max_items / 8), projections), 256 threads. Consecutive workgroup ids go round the eight dies,
 // so the workgroups that share an item's activations (its nblk column blocks) are given ids 8 apart: one die's L2
 // serves them all.
 //
-// Shapes: RB 16-row blocks an item and NT adjacent tiles a wave, 64 NT columns a workgroup. (4, 4): 64 rows. (8, 4):
-// 128 rows: a decoded weight feeds twice the MFMAs, and an expert with 65-128 rows stays one item (a second, short
-// item would pay the whole decode again). (2, 4): 32 rows for sparse routings. Row blocks past the item's last row
-// skip their MFMAs. (Measured: (8, 2) gains nothing over (4, 4): halving NT doubles the LDS and L2 traffic of the
-// activations a flop.)
-template <int CB, bool WIDE, int RB, int NT>
+// Shapes: RB 16-row blocks an item, four adjacent tiles a wave, 256 columns a workgroup. RB 4: 64 rows. RB 8: 128 rows:
+// a decoded weight feeds twice the MFMAs, and an expert with 65-128 rows stays one item (a second, short item would
+// pay the whole decode again). RB 2: 32 rows for sparse routings. Row blocks past the item's last row skip their MFMAs.
+//
+// The operands reach LDS without passing through registers, D steps deep (a step = K 32 = two tile rows):
+//   weights      a wave's four tiles of a tile row, one load: lane L brings bytes 16 (L % 16).. of tile L / 16 to the
+//                tile's 256-byte slot; each lane then reads back the two (four) words its quad's windows span;
+//   activations  the item's rows, 64 bytes a row a step, 16 rows a load. Row r's 16-byte piece p is kept at position
+//                p ^ ((r >> 1) & 3) of the row, which spreads a B fragment's reads (16 rows, one piece each) over the
+//                banks at row stride 64 (measured: 4.2 cycles a wave's read, 8 unswizzled).
+// Measured before this form, with loads held in registers one step ahead: the kernel waited on the weight loads 12 %
+// of its time (strided 256-byte pieces come back slower than one step takes).
+template <int CB, bool WIDE, int RB>
 __global__ void __launch_bounds__(256) pf_gemm(const PfGemm a) {
-    constexpr uint32_t kPfTiles = NT;
-    constexpr uint32_t kPfWStage = pf_stage_bytes(NT);
+    constexpr uint32_t D = RB == 2 ? 3u : 4u;                // steps in flight + 1
     constexpr uint32_t BM = RB * 16u;
-    constexpr uint32_t kABuf = BM * kPfRowStride;
-    constexpr uint32_t kPieces = BM * 4u;                      // 16-byte pieces of an item's rows a step
-    constexpr uint32_t kALoads = (kPieces + 255u) / 256u;
-    __shared__ __attribute__((aligned(16))) unsigned char smem[2u * kABuf + 4u * kPfWStage];
+    constexpr uint32_t kAStep = BM * 64u;                     // LDS bytes of the item's rows a step
+    constexpr uint32_t kALoads = RB >= 4 ? RB / 4u : 1u;      // activation loads a wave a step (16 rows each)
+    constexpr int kPerStep = static_cast<int>(kALoads) + 2;   // loads a wave a step
+    __shared__ __attribute__((aligned(16))) unsigned char smem[D * kAStep + 4u * D * kPfWaveStep];
+    static_assert(sizeof(smem) <= 65536u, "the LDS addresses of the loads are 16 bits");
 
     const uint32_t id = blockIdx.x, proj = blockIdx.y;
     const uint32_t j = id >> 3, blk = j % a.nblk, item_i = (j / a.nblk) * 8u + (id & 7u);
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u, tid = threadIdx.x;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
     uint32_t e = 0, first, count;
     if (a.items) {
         if (item_i >= a.n_items[0]) return;
@@ -110,89 +136,56 @@ __global__ void __launch_bounds__(256) pf_gemm(const PfGemm a) {
     const uint32_t wstep = out_tiles * nw * 4u;
     const uint32_t tile_bytes = 2u * a.n, chunk_bytes = kPfTiles * tile_bytes;
     // the wave's window of the matrix: a tile row past the last one falls outside it and reads as zeros
-    const __amdgpu_buffer_rsrc_t wres =
-        make_rsrc(wmat + static_cast<size_t>(col0) * nw, active ? (in_tiles - 1u) * wstep + chunk_bytes : 0u);
-    const uint32_t wvoff = lane * 16u < chunk_bytes ? lane * 16u : 0x40000000u;
-    const __amdgpu_buffer_rsrc_t xres = make_rsrc(a.xq[proj], static_cast<uint64_t>(a.positions) * a.in * 2u);
+    const uint4v wdesc = rsrc_words(wmat + static_cast<size_t>(col0) * nw,
+                                    active ? (in_tiles - 1u) * wstep + chunk_bytes : 0u);
+    const uint4v xdesc = rsrc_words(a.xq[proj], static_cast<uint64_t>(a.positions) * a.in * 2u);
+    const uint32_t w_voff = (lane & 15u) * 16u < tile_bytes ? (lane >> 4) * tile_bytes + (lane & 15u) * 16u : 0x80000000u;
 
-    unsigned char* abuf = smem;
-    unsigned char* stage = smem + 2u * kABuf + wave * kPfWStage;
+    const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem));
+    const uint32_t a_lds = lds0, w_lds = lds0 + D * kAStep + wave * (D * kPfWaveStep);
+    const unsigned char* a_ring = smem;
+    const unsigned char* w_ring = smem + D * kAStep + wave * (D * kPfWaveStep);
 
-    // where this thread's pieces of the item's rows come from and go
-    uint32_t a_voff[kALoads], a_put[kALoads];
-    bool a_live[kALoads];
+    // the pieces of the item's rows this lane brings: load i of the wave covers rows 16 (4 i + wave) .. + 15 (RB 2 has
+    // two loads' worth of rows: waves 2 and 3 repeat the loads of waves 0 and 1)
+    const uint32_t wq = RB == 2 ? (wave & 1u) : wave;
+    uint32_t a_voff[kALoads];
 #pragma unroll
     for (uint32_t i = 0; i < kALoads; ++i) {
-        const uint32_t idx = tid + 256u * i, row = idx >> 2, piece = idx & 3u;
-        a_live[i] = idx < kPieces;
-        a_voff[i] = a_live[i] && row < count ? ((first + row) * a.in + piece * 8u) * 2u : 0x80000000u;
-        // 8 halves = tile piece / 2, quads 2 (piece % 2) and + 1: row, then quad, then tile, 8 bytes each
-        a_put[i] = row * kPfRowStride + (piece & 1u) * 32u + (piece >> 1) * 8u;
+        const uint32_t row = (4u * i + wq) * 16u + (lane >> 2), piece = (lane & 3u) ^ ((row >> 1) & 3u);
+        a_voff[i] = row < count ? ((first + row) * a.in + piece * 8u) * 2u : 0x80000000u;
     }
-    auto load_a = [&](uint32_t step, uint4v(&dst)[kALoads]) {
-#pragma unroll
-        for (uint32_t i = 0; i < kALoads; ++i) dst[i] = buf_load_u128(xres, a_voff[i], step * 64u);
-    };
-    auto put_a = [&](const uint4v(&src)[kALoads], uint32_t parity) {
+    auto issue = [&](uint32_t step, uint32_t slot) {
 #pragma unroll
         for (uint32_t i = 0; i < kALoads; ++i)
-            if (a_live[i]) {
-                unsigned char* p = abuf + parity * kABuf + a_put[i];
-                *reinterpret_cast<uint2*>(p) = make_uint2(src[i][0], src[i][1]);
-                *reinterpret_cast<uint2*>(p + 16u) = make_uint2(src[i][2], src[i][3]);
-            }
+            load_to_lds(xdesc, a_lds + slot * kAStep + (4u * i + wq) * 1024u, a_voff[i], step * 64u);
+#pragma unroll
+        for (uint32_t r = 0; r < 2u; ++r)
+            load_to_lds(wdesc, w_lds + slot * kPfWaveStep + r * (kPfTiles * kPfSlot), w_voff, (2u * step + r) * wstep);
     };
 
     const QuadPlan<WIDE> plan = quad_plan<WIDE>(a.n, lane);
-    const uint32_t inv_tile = (1u << 16) / tile_bytes + 1u;
-    // A lane's 16 bytes of a tile row's chunk go to the tiles' slots: in one piece where a tile is whole 16-byte
-    // pieces (every integer rate), else word by word. Lanes past the chunk write nothing.
-    const bool writer = lane * 16u < chunk_bytes;
-    const bool whole = (tile_bytes & 15u) == 0u;  // uniform
-    uint32_t put[4];
-#pragma unroll
-    for (uint32_t jj = 0; jj < 4u; ++jj) {
-        const uint32_t b = lane * 16u + 4u * jj;
-        const uint32_t t = (b * inv_tile) >> 16;
-        put[jj] = t * kPfSlot + (b - t * tile_bytes);
-    }
     const uint32_t get_bp = plan.ib_prev * 4u, get_bl = plan.ib_last * 4u;
     const uint32_t get_ap = plan.ia_prev * 4u, get_al = plan.ia_last * 4u;
-
-    auto load_w = [&](uint32_t step, uint4v(&dst)[2]) {
-        dst[0] = buf_load_u128(wres, wvoff, (2u * step) * wstep);
-        dst[1] = buf_load_u128(wres, wvoff, (2u * step + 1u) * wstep);
-    };
-    auto stage_w = [&](const uint4v(&src)[2]) {
-        if (!writer) return;
-        if (whole) {
-#pragma unroll
-            for (uint32_t r = 0; r < 2u; ++r)
-                *reinterpret_cast<uint4v*>(stage + r * (kPfTiles * kPfSlot) + put[0]) = src[r];
-        } else {
-#pragma unroll
-            for (uint32_t r = 0; r < 2u; ++r)
-#pragma unroll
-                for (uint32_t jj = 0; jj < 4u; ++jj)
-                    *reinterpret_cast<uint32_t*>(stage + r * (kPfTiles * kPfSlot) + put[jj]) = src[r][jj];
-        }
-    };
-    auto fetch_w = [&](QuadWords<WIDE>(&wd)[2][kPfTiles]) {
+    auto fetch_w = [&](QuadWords<WIDE>(&wd)[2][kPfTiles], uint32_t slot) {
+        const unsigned char* st = w_ring + slot * kPfWaveStep;
 #pragma unroll
         for (uint32_t r = 0; r < 2u; ++r)
 #pragma unroll
             for (uint32_t t = 0; t < kPfTiles; ++t) {
-                const unsigned char* slot = stage + (r * kPfTiles + t) * kPfSlot;
-                wd[r][t].b_prev = *reinterpret_cast<const uint32_t*>(slot + get_bp);
-                wd[r][t].b_last = *reinterpret_cast<const uint32_t*>(slot + get_bl);
+                const unsigned char* tile = st + (r * kPfTiles + t) * kPfSlot;
+                wd[r][t].b_prev = *reinterpret_cast<const uint32_t*>(tile + get_bp);
+                wd[r][t].b_last = *reinterpret_cast<const uint32_t*>(tile + get_bl);
                 if constexpr (WIDE) {
-                    wd[r][t].a_prev = *reinterpret_cast<const uint32_t*>(slot + get_ap);
-                    wd[r][t].a_last = *reinterpret_cast<const uint32_t*>(slot + get_al);
+                    wd[r][t].a_prev = *reinterpret_cast<const uint32_t*>(tile + get_ap);
+                    wd[r][t].a_last = *reinterpret_cast<const uint32_t*>(tile + get_al);
                 }
             }
     };
+    // the B fragment of block mb: row 16 mb + lane % 16, K slots 8 (lane / 16) ..: its swizzled piece
+    const uint32_t b_at = (lane & 15u) * 64u + (((lane >> 4) ^ ((lane >> 1) & 3u)) * 16u);
 
-    const uint32_t steps = in_tiles >> 1;  // even: in is a multiple of 128
+    const uint32_t steps = in_tiles >> 1;  // a multiple of 4: in is a multiple of 128
     float* z = a.z[proj];
 
     // The K loop and the stores for an item of LB live 16-row blocks: no branch inside the loop.
@@ -204,13 +197,11 @@ __global__ void __launch_bounds__(256) pf_gemm(const PfGemm a) {
             for (uint32_t t = 0; t < kPfTiles; ++t) acc[mb][t] = float4v{0.f, 0.f, 0.f, 0.f};
 
         // one step: K = 32 = tile rows 2 step and 2 step + 1
-        auto compute = [&](const QuadWords<WIDE>(&wd)[2][kPfTiles], uint32_t parity) {
+        auto compute = [&](const QuadWords<WIDE>(&wd)[2][kPfTiles], uint32_t slot) {
             uint4v bf[LB];
 #pragma unroll
             for (int mb = 0; mb < LB; ++mb)
-                bf[mb] = *reinterpret_cast<const uint4v*>(abuf + parity * kABuf +
-                                                          (static_cast<uint32_t>(mb) * 16u + (lane & 15u)) * kPfRowStride +
-                                                          (lane >> 4) * 16u);
+                bf[mb] = *reinterpret_cast<const uint4v*>(a_ring + slot * kAStep + static_cast<uint32_t>(mb) * 1024u + b_at);
 #pragma unroll
             for (uint32_t t = 0; t < kPfTiles; ++t) {
                 uint32_t c0[4], c1[4];
@@ -227,35 +218,33 @@ __global__ void __launch_bounds__(256) pf_gemm(const PfGemm a) {
                         __builtin_bit_cast(half8, af), __builtin_bit_cast(half8, bf[mb]), acc[mb][t], 0, 0, 0);
             }
         };
+        // Step s: its operands are in ring slot s % D. The loads of step s + D - 1 go out (into the slot step s - 1
+        // left: every wave is past the barrier that ended it), step s + 1's have landed once at most D - 2 steps' loads
+        // are in flight, its words are read while step s computes, and the barrier publishes every wave's part of its
+        // activations. Loads past the last step fall outside the buffers: they keep the count and bring zeros.
+        auto step = [&](uint32_t s, uint32_t slot, const QuadWords<WIDE>(&cur)[2][kPfTiles],
+                        QuadWords<WIDE>(&next)[2][kPfTiles]) {
+            issue(s + D - 1u, slot == 0u ? D - 1u : slot - 1u);
+            wait_loads<static_cast<int>(D - 2u) * kPerStep>();
+            fetch_w(next, slot + 1u == D ? 0u : slot + 1u);
+            compute(cur, slot);
+            __syncthreads();
+        };
 
-        uint4v wreg[2], areg[kALoads];
         QuadWords<WIDE> wd0[2][kPfTiles], wd1[2][kPfTiles];
-        load_w(0u, wreg);
-        load_a(0u, areg);
-        put_a(areg, 0u);
-        stage_w(wreg);
-        fetch_w(wd0);
-        load_w(1u, wreg);
-        load_a(1u, areg);
+#pragma unroll
+        for (uint32_t t = 0; t + 1u < D; ++t) issue(t, t);
+        wait_loads<static_cast<int>(D - 2u) * kPerStep>();
+        fetch_w(wd0, 0u);
         __syncthreads();
+        uint32_t slot = 0;
         for (uint32_t s = 0; s < steps; s += 2u) {
-            // even step: words in wd0, activations in buffer 0; wreg / areg hold step s + 1
-            stage_w(wreg);
-            load_w(s + 2u, wreg);
-            fetch_w(wd1);
-            compute(wd0, 0u);
-            put_a(areg, 1u);
-            load_a(s + 2u, areg);
-            __syncthreads();
-            // odd step
-            stage_w(wreg);
-            load_w(s + 3u, wreg);
-            fetch_w(wd0);
-            compute(wd1, 1u);
-            put_a(areg, 0u);
-            load_a(s + 3u, areg);
-            __syncthreads();
+            step(s, slot, wd0, wd1);
+            slot = slot + 1u == D ? 0u : slot + 1u;
+            step(s + 1u, slot, wd1, wd0);
+            slot = slot + 1u == D ? 0u : slot + 1u;
         }
+        wait_loads<0>();
 
         if (!active) return;
         // D[i][j]: i = the weight's column inside its tile (this lane: 4 (lane / 16) .. + 3), j = activation row
@@ -530,7 +519,7 @@ __global__ void __launch_bounds__(256) pf_combine(const MoeLaunch a) {
         if (b0 + u < nb) routed_store_row(a, row, b0 + u, lane, acc[u]);
 }
 
-// the dense prepare: plain f16 [rows][in], in quad order for the trellis GEMM (NATURAL: as is, for a plain GEMM);
+// the dense prepare: plain f16 [rows][in], in pair-quad order for the trellis GEMM (NATURAL: as is, for a plain GEMM);
 // xs: block sums (null: not wanted)
 template <int DT, bool NATURAL>
 __global__ void __launch_bounds__(256) pf_dense_prep(const void* x, const uint16_t* suh, uint16_t* xq, float* xs,
@@ -555,7 +544,7 @@ __global__ void __launch_bounds__(256) pf_dense_prep(const void* x, const uint16
 #pragma unroll
         for (uint32_t j = 0; j < 2u; ++j) {
             const uint32_t i = (b0 + u) * 128u + lane + 64u * j;
-            const uint32_t at = NATURAL ? i : (i & ~15u) + quad_slot(i & 15u);
+            const uint32_t at = NATURAL ? i : pair_quad_slot(i);
             xq[static_cast<size_t>(row) * in + at] = static_cast<uint16_t>(hv[j]);
         }
         if (xs && lane == 0u) xs[static_cast<size_t>(row) * nb + b0 + u] = sum;
@@ -631,9 +620,9 @@ template <int CB, bool WIDE>
 hipError_t launch_gemm_rb(PfGemm g, uint32_t max_items, uint32_t nproj, uint32_t item_rows, hipStream_t s) {
     g.nblk = gemm_nblk(g.out, item_rows);
     const dim3 grid(8u * g.nblk * ((max_items + 7u) / 8u), nproj), block(256);
-    if (item_rows == 32u) hipLaunchKernelGGL((pf_gemm<CB, WIDE, 2, 4>), grid, block, 0, s, g);
-    else if (item_rows == 128u) hipLaunchKernelGGL((pf_gemm<CB, WIDE, 8, 4>), grid, block, 0, s, g);
-    else hipLaunchKernelGGL((pf_gemm<CB, WIDE, 4, 4>), grid, block, 0, s, g);
+    if (item_rows == 32u) hipLaunchKernelGGL((pf_gemm<CB, WIDE, 2>), grid, block, 0, s, g);
+    else if (item_rows == 128u) hipLaunchKernelGGL((pf_gemm<CB, WIDE, 8>), grid, block, 0, s, g);
+    else hipLaunchKernelGGL((pf_gemm<CB, WIDE, 4>), grid, block, 0, s, g);
     return hipGetLastError();
 }
 

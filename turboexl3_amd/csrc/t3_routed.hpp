@@ -113,9 +113,8 @@ __device__ __forceinline__ void plane_sums(const float* z, size_t planes_stride,
 
 template <bool PF>
 __device__ __forceinline__ void store_prepared(uint32_t* base, size_t row_at, uint32_t i, uint32_t hbits) {
-    const size_t at = row_at + (i & ~15u) + quad_slot(i & 15u);
-    if constexpr (PF) reinterpret_cast<uint16_t*>(base)[at] = static_cast<uint16_t>(hbits);
-    else base[at] = hbits | (hbits << 16);
+    if constexpr (PF) reinterpret_cast<uint16_t*>(base)[row_at + pair_quad_slot(i)] = static_cast<uint16_t>(hbits);
+    else base[row_at + (i & ~15u) + quad_slot(i & 15u)] = hbits | (hbits << 16);
 }
 
 // the gate's and the up's prepare of block b of row-slot rk: xg, xu [.][hidden], sg, su [.][hidden / 128]
