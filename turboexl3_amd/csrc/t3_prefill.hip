@@ -377,10 +377,11 @@ __global__ void __launch_bounds__(256) pf_place(const MoeLaunch a) {
 }
 
 // ---- the chains' stages around the GEMM -----------------------------------------------------------------------
-// One wave takes kPfUnit adjacent 128-blocks of one row (or sorted position) and issues every load of all of them
-// before the first transform: a block is 256 bytes a load instruction, so one block a wave leaves the memory system
-// almost idle (measured: 1.8 TB/s). Four waves a workgroup; grid ceil(units / 4). The arithmetic of a block is
-// that of t3_stages.hpp, statement for statement.
+// One wave takes kPfUnit adjacent 128-blocks of one row (or sorted position), 16 lanes a block and 8 adjacent elements
+// a lane (t3_stages.hpp, "four 128-blocks a wave"): every load and store is 16 bytes a lane, and a block's transform
+// is ~20 vector-ALU operations a lane (the one-block-a-wave form of the decode kernels spends ~100: these kernels were
+// bound by it). Four waves a workgroup; grid ceil(units / 4). Blocks past the row's last one load the last block and
+// store nothing. Every array these kernels touch starts 16-byte aligned (the host checks the caller's).
 
 constexpr uint32_t kPfUnit = 4;
 
@@ -389,134 +390,123 @@ __device__ __forceinline__ uint32_t wave_unit() { return blockIdx.x * 4u + (thre
 template <int DT>
 __global__ void __launch_bounds__(256) pf_prep(const MoeLaunch a) {
     const uint32_t nb = a.hidden / 128u, groups = (nb + kPfUnit - 1u) / kPfUnit;
-    const uint32_t u0 = wave_unit(), q = u0 / groups, b0 = (u0 % groups) * kPfUnit, lane = threadIdx.x & 63u;
-    if (q >= a.counts[a.bank.experts + a.shared_slots + 1u]) return;
-    const SlotRef s = resolve_slot(a, a.order[q]);
+    const uint32_t u0 = wave_unit(), pos = u0 / groups, lane = threadIdx.x & 63u, q = lane & 15u;
+    if (pos >= a.counts[a.bank.experts + a.shared_slots + 1u]) return;
+    const uint32_t b1 = (u0 % groups) * kPfUnit + (lane >> 4);
+    const bool live = b1 < nb;
+    const uint32_t b = live ? b1 : nb - 1u, i = b * 128u + 8u * q;
+    const SlotRef s = resolve_slot(a, a.order[pos]);
     const RoutedBank& bank = s.shared ? a.shared : a.bank;
-    const uint16_t* gs = bank.gate_suh + static_cast<size_t>(s.e) * a.hidden;
-    const uint16_t* us = bank.up_suh + static_cast<size_t>(s.e) * a.hidden;
-    float xv[kPfUnit][2], g[kPfUnit][2], up[kPfUnit][2];
+    const Row16 g16 = row16(lane);
+    float xv[8], sc[2][8];
+    load8_act<DT>(a.x, static_cast<size_t>(s.row) * a.hidden + i, xv);
+    load8_half(bank.gate_suh, static_cast<size_t>(s.e) * a.hidden + i, sc[0]);
+    load8_half(bank.up_suh, static_cast<size_t>(s.e) * a.hidden + i, sc[1]);
 #pragma unroll
-    for (uint32_t u = 0; u < kPfUnit; ++u)
+    for (uint32_t proj = 0; proj < 2u; ++proj) {
+        float v[8];
 #pragma unroll
-        for (uint32_t j = 0; j < 2u; ++j) {
-            const uint32_t b = b0 + u < nb ? b0 + u : nb - 1u, i = b * 128u + lane + 64u * j;
-            xv[u][j] = round_half(load_act<DT>(a.x, static_cast<size_t>(s.row) * a.hidden + i));
-            g[u][j] = half_value(gs[i]);
-            up[u][j] = half_value(us[i]);
-        }
-#pragma unroll
-    for (uint32_t u = 0; u < kPfUnit; ++u) {
-        if (b0 + u >= nb) break;
-#pragma unroll
-        for (uint32_t proj = 0; proj < 2u; ++proj) {
-            float v[2] = {xv[u][0] * (proj ? up[u][0] : g[u][0]), xv[u][1] * (proj ? up[u][1] : g[u][1])};
-            uint32_t hv[2];
-            float sum;
-            prep_core(v, lane, hv, sum, a.defer != 0);
-#pragma unroll
-            for (uint32_t j = 0; j < 2u; ++j)
-                store_prepared<true>(proj ? a.xu : a.xg, static_cast<size_t>(q) * a.hidden,
-                                     (b0 + u) * 128u + lane + 64u * j, hv[j]);
-            if (lane == 0u) (proj ? a.su : a.sg)[static_cast<size_t>(q) * nb + b0 + u] = sum;
-        }
+        for (uint32_t r = 0; r < 8u; ++r) v[r] = round_half(xv[r]) * sc[proj][r];
+        uint32_t hv[4];
+        float sum;
+        prep_row16(v, g16, hv, sum, a.defer != 0);
+        if (!live) continue;
+        store_pair_quad(reinterpret_cast<uint16_t*>(proj ? a.xu : a.xg), static_cast<size_t>(pos) * a.hidden, b, q, hv);
+        if (q == 0u) (proj ? a.su : a.sg)[static_cast<size_t>(pos) * nb + b] = sum;
     }
 }
 
 // gate and up finishes, the (clamped) SwiGLU, the down's prepare (routed_mid_block's statements)
 __global__ void __launch_bounds__(256) pf_mid(const MoeLaunch a) {
     const uint32_t nb = a.inter / 128u, nbh = a.hidden / 128u, groups = (nb + kPfUnit - 1u) / kPfUnit;
-    const uint32_t u0 = wave_unit(), q = u0 / groups, b0 = (u0 % groups) * kPfUnit, lane = threadIdx.x & 63u;
-    if (q >= a.counts[a.bank.experts + a.shared_slots + 1u]) return;
-    const SlotRef s = resolve_slot(a, a.order[q]);
+    const uint32_t u0 = wave_unit(), pos = u0 / groups, lane = threadIdx.x & 63u, q = lane & 15u;
+    if (pos >= a.counts[a.bank.experts + a.shared_slots + 1u]) return;
+    const uint32_t b1 = (u0 % groups) * kPfUnit + (lane >> 4);
+    const bool live = b1 < nb;
+    const uint32_t b = live ? b1 : nb - 1u, i = b * 128u + 8u * q;
+    const SlotRef s = resolve_slot(a, a.order[pos]);
     const RoutedBank& bank = s.shared ? a.shared : a.bank;
-    const size_t eo = static_cast<size_t>(s.e) * a.inter, qo = static_cast<size_t>(q) * a.inter;
-    float zg[kPfUnit][2], zu[kPfUnit][2], svg[kPfUnit][2], svu[kPfUnit][2], sdn[kPfUnit][2];
-#pragma unroll
-    for (uint32_t u = 0; u < kPfUnit; ++u)
-#pragma unroll
-        for (uint32_t j = 0; j < 2u; ++j) {
-            const uint32_t b = b0 + u < nb ? b0 + u : nb - 1u, i = b * 128u + lane + 64u * j;
-            zg[u][j] = a.zg[qo + i];
-            zu[u][j] = a.zu[qo + i];
-            svg[u][j] = half_value(bank.gate_svh[eo + i]);
-            svu[u][j] = half_value(bank.up_svh[eo + i]);
-            sdn[u][j] = half_value(bank.down_suh[eo + i]);
-        }
-    float xg = 0.0f, xu = 0.0f;
-    if (a.defer)
+    const size_t eo = static_cast<size_t>(s.e) * a.inter, qo = static_cast<size_t>(pos) * a.inter;
+    const Row16 g16 = row16(lane);
+    float gt[8], up[8], svg[8], svu[8], sdn[8];
+    load8_f32(a.zg, qo + i, gt);
+    load8_f32(a.zu, qo + i, up);
+    load8_half(bank.gate_svh, eo + i, svg);
+    load8_half(bank.up_svh, eo + i, svu);
+    load8_half(bank.down_suh, eo + i, sdn);
+    if (a.defer) {
+        float xg = 0.0f, xu = 0.0f;
         for (uint32_t t = 0; t < nbh; ++t) {
-            xg += a.sg[static_cast<size_t>(q) * nbh + t];
-            xu += a.su[static_cast<size_t>(q) * nbh + t];
+            xg += a.sg[static_cast<size_t>(pos) * nbh + t];
+            xu += a.su[static_cast<size_t>(pos) * nbh + t];
         }
 #pragma unroll
-    for (uint32_t u = 0; u < kPfUnit; ++u) {
-        if (b0 + u >= nb) break;
-        float g[2] = {zg[u][0], zg[u][1]}, up[2] = {zu[u][0], zu[u][1]};
-        if (a.defer)
-#pragma unroll
-            for (uint32_t j = 0; j < 2u; ++j) {
-                g[j] = __builtin_fmaf(g[j], mul1_a(), mul1_b() * xg);
-                up[j] = __builtin_fmaf(up[j], mul1_a(), mul1_b() * xu);
-            }
-        finish_core(g, svg[u], lane);
-        finish_core(up, svu[u], lane);
-        float d[2];
-#pragma unroll
-        for (uint32_t j = 0; j < 2u; ++j) {
-            d[j] = round_half(swiglu_clamped(g[j], up[j], a.limit, a.clamp_at)) * sdn[u][j];
+        for (uint32_t r = 0; r < 8u; ++r) {
+            gt[r] = __builtin_fmaf(gt[r], mul1_a(), mul1_b() * xg);
+            up[r] = __builtin_fmaf(up[r], mul1_a(), mul1_b() * xu);
         }
-        uint32_t hv[2];
-        float sum;
-        prep_core(d, lane, hv, sum, a.defer != 0);
-#pragma unroll
-        for (uint32_t j = 0; j < 2u; ++j) store_prepared<true>(a.hd, qo, (b0 + u) * 128u + lane + 64u * j, hv[j]);
-        if (lane == 0u) a.hs[static_cast<size_t>(q) * nb + b0 + u] = sum;
     }
+    finish_row16(gt, svg, g16);
+    finish_row16(up, svu, g16);
+    float d[8];
+#pragma unroll
+    for (uint32_t r = 0; r < 8u; ++r) d[r] = round_half(swiglu_clamped(gt[r], up[r], a.limit, a.clamp_at)) * sdn[r];
+    uint32_t hv[4];
+    float sum;
+    prep_row16(d, g16, hv, sum, a.defer != 0);
+    if (!live) return;
+    store_pair_quad(reinterpret_cast<uint16_t*>(a.hd), qo, b, q, hv);
+    if (q == 0u) a.hs[static_cast<size_t>(pos) * nb + b] = sum;
 }
 
 // every slot's down finish, then the score-weighted sum in slot order (routed_combine_block's statements)
 __global__ void __launch_bounds__(256) pf_combine(const MoeLaunch a) {
     const uint32_t nb = a.hidden / 128u, nbi = a.inter / 128u, groups = (nb + kPfUnit - 1u) / kPfUnit;
-    const uint32_t u0 = wave_unit(), row = u0 / groups, b0 = (u0 % groups) * kPfUnit, lane = threadIdx.x & 63u;
+    const uint32_t u0 = wave_unit(), row = u0 / groups, lane = threadIdx.x & 63u, q = lane & 15u;
     if (row >= a.rows) return;
+    const uint32_t b1 = (u0 % groups) * kPfUnit + (lane >> 4);
+    const bool live = b1 < nb;
+    const uint32_t b = live ? b1 : nb - 1u, i = b * 128u + 8u * q;
+    const Row16 g16 = row16(lane);
     const uint32_t kt = a.topk + a.shared_slots;
-    float acc[kPfUnit][2];
+    float acc[8];
 #pragma unroll
-    for (uint32_t u = 0; u < kPfUnit; ++u) acc[u][0] = acc[u][1] = 0.0f;
+    for (uint32_t r = 0; r < 8u; ++r) acc[r] = 0.0f;
     for (uint32_t k = 0; k < kt; ++k) {
         const uint32_t rk = row * kt + k;
         const SlotRef s = resolve_slot(a, rk);
         if (!s.live) continue;  // uniform over the wave
-        const uint32_t q = a.inv[rk];
+        const uint32_t pos = a.inv[rk];
         const RoutedBank& bank = s.shared ? a.shared : a.bank;
-        float z[kPfUnit][2], sv[kPfUnit][2];
+        float v[8], sv[8];
+        load8_f32(a.zd, static_cast<size_t>(pos) * a.hidden + i, v);
+        load8_half(bank.down_svh, static_cast<size_t>(s.e) * a.hidden + i, sv);
+        if (a.defer) {
+            float xsum = 0.0f;
+            for (uint32_t t = 0; t < nbi; ++t) xsum += a.hs[static_cast<size_t>(pos) * nbi + t];
 #pragma unroll
-        for (uint32_t u = 0; u < kPfUnit; ++u)
-#pragma unroll
-            for (uint32_t j = 0; j < 2u; ++j) {
-                const uint32_t b = b0 + u < nb ? b0 + u : nb - 1u, i = b * 128u + lane + 64u * j;
-                z[u][j] = a.zd[static_cast<size_t>(q) * a.hidden + i];
-                sv[u][j] = half_value(bank.down_svh[static_cast<size_t>(s.e) * a.hidden + i]);
-            }
-        float xsum = 0.0f;
-        if (a.defer)
-            for (uint32_t t = 0; t < nbi; ++t) xsum += a.hs[static_cast<size_t>(q) * nbi + t];
+            for (uint32_t r = 0; r < 8u; ++r) v[r] = __builtin_fmaf(v[r], mul1_a(), mul1_b() * xsum);
+        }
         const float w = s.shared ? 1.0f : score_of(a, row, k);
+        finish_row16(v, sv, g16);
 #pragma unroll
-        for (uint32_t u = 0; u < kPfUnit; ++u) {
-            float v[2] = {z[u][0], z[u][1]};
-            if (a.defer)
+        for (uint32_t r = 0; r < 8u; ++r) acc[r] = __builtin_fmaf(w, v[r], acc[r]);
+    }
+    if (!live) return;
+    const size_t o = static_cast<size_t>(row) * a.hidden + i;
+    if (a.shared_add) {
+        // the routed output rounds to x's dtype, then the add rounds again (src/root.zig:976-984)
+        float add[8];
+        load8_act_rt(a.dtype, a.shared_add, o, add);
 #pragma unroll
-                for (uint32_t j = 0; j < 2u; ++j) v[j] = __builtin_fmaf(v[j], mul1_a(), mul1_b() * xsum);
-            finish_core(v, sv[u], lane);
-#pragma unroll
-            for (uint32_t j = 0; j < 2u; ++j) acc[u][j] = __builtin_fmaf(w, v[j], acc[u][j]);
+        for (uint32_t r = 0; r < 8u; ++r) {
+            float t = acc[r];
+            if (a.dtype == kF16) t = round_half(t);
+            else if (a.dtype == kBf16) t = bf16_value(bf16_bits(t));
+            acc[r] = t + add[r];
         }
     }
-#pragma unroll
-    for (uint32_t u = 0; u < kPfUnit; ++u)
-        if (b0 + u < nb) routed_store_row(a, row, b0 + u, lane, acc[u]);
+    store8_act_rt(a.dtype, a.y, o, acc);
 }
 
 // the dense prepare: plain f16 [rows][in], in pair-quad order for the trellis GEMM (NATURAL: as is, for a plain GEMM);
@@ -525,30 +515,26 @@ template <int DT, bool NATURAL>
 __global__ void __launch_bounds__(256) pf_dense_prep(const void* x, const uint16_t* suh, uint16_t* xq, float* xs,
                                                      uint32_t in, uint32_t rows) {
     const uint32_t nb = in / 128u, groups = (nb + kPfUnit - 1u) / kPfUnit;
-    const uint32_t u0 = wave_unit(), row = u0 / groups, b0 = (u0 % groups) * kPfUnit, lane = threadIdx.x & 63u;
+    const uint32_t u0 = wave_unit(), row = u0 / groups, lane = threadIdx.x & 63u, q = lane & 15u;
     if (row >= rows) return;
-    float v[kPfUnit][2];
+    const uint32_t b1 = (u0 % groups) * kPfUnit + (lane >> 4);
+    const bool live = b1 < nb;
+    const uint32_t b = live ? b1 : nb - 1u, i = b * 128u + 8u * q;
+    const Row16 g16 = row16(lane);
+    float v[8], sc[8];
+    load8_act<DT>(x, static_cast<size_t>(row) * in + i, v);
+    load8_half(suh, i, sc);
 #pragma unroll
-    for (uint32_t u = 0; u < kPfUnit; ++u)
-#pragma unroll
-        for (uint32_t j = 0; j < 2u; ++j) {
-            const uint32_t b = b0 + u < nb ? b0 + u : nb - 1u, i = b * 128u + lane + 64u * j;
-            v[u][j] = round_half(load_act<DT>(x, static_cast<size_t>(row) * in + i)) * half_value(suh[i]);
-        }
-#pragma unroll
-    for (uint32_t u = 0; u < kPfUnit; ++u) {
-        if (b0 + u >= nb) break;
-        uint32_t hv[2];
-        float sum;
-        prep_core(v[u], lane, hv, sum, xs != nullptr);
-#pragma unroll
-        for (uint32_t j = 0; j < 2u; ++j) {
-            const uint32_t i = (b0 + u) * 128u + lane + 64u * j;
-            const uint32_t at = NATURAL ? i : pair_quad_slot(i);
-            xq[static_cast<size_t>(row) * in + at] = static_cast<uint16_t>(hv[j]);
-        }
-        if (xs && lane == 0u) xs[static_cast<size_t>(row) * nb + b0 + u] = sum;
-    }
+    for (uint32_t r = 0; r < 8u; ++r) v[r] = round_half(v[r]) * sc[r];
+    uint32_t hv[4];
+    float sum;
+    prep_row16(v, g16, hv, sum, xs != nullptr);
+    if (!live) return;
+    if constexpr (NATURAL)
+        *reinterpret_cast<uint4v*>(xq + static_cast<size_t>(row) * in + i) = uint4v{hv[0], hv[1], hv[2], hv[3]};
+    else
+        store_pair_quad(xq, static_cast<size_t>(row) * in, b, q, hv);
+    if (xs && q == 0u) xs[static_cast<size_t>(row) * nb + b] = sum;
 }
 
 // the dense finish of one plane: z f32 [rows][out] with xs [rows][in / 128] for MUL1's deferred map, or (HALF) z
@@ -557,32 +543,25 @@ template <int DT, bool HALF>
 __global__ void __launch_bounds__(256) pf_dense_finish(const void* z, const float* xs, const uint16_t* svh, void* y,
                                                        uint32_t out, uint32_t rows, uint32_t inblk, int defer) {
     const uint32_t nb = out / 128u, groups = (nb + kPfUnit - 1u) / kPfUnit;
-    const uint32_t u0 = wave_unit(), row = u0 / groups, b0 = (u0 % groups) * kPfUnit, lane = threadIdx.x & 63u;
+    const uint32_t u0 = wave_unit(), row = u0 / groups, lane = threadIdx.x & 63u, q = lane & 15u;
     if (row >= rows) return;
-    float v[kPfUnit][2], sv[kPfUnit][2];
-#pragma unroll
-    for (uint32_t u = 0; u < kPfUnit; ++u)
-#pragma unroll
-        for (uint32_t j = 0; j < 2u; ++j) {
-            const uint32_t b = b0 + u < nb ? b0 + u : nb - 1u, i = b * 128u + lane + 64u * j;
-            const size_t at = static_cast<size_t>(row) * out + i;
-            v[u][j] = HALF ? half_value(static_cast<const uint16_t*>(z)[at]) : static_cast<const float*>(z)[at];
-            sv[u][j] = half_value(svh[i]);
-        }
-    float xsum = 0.0f;
-    if (!HALF && defer)
+    const uint32_t b1 = (u0 % groups) * kPfUnit + (lane >> 4);
+    const bool live = b1 < nb;
+    const uint32_t b = live ? b1 : nb - 1u, i = b * 128u + 8u * q;
+    const Row16 g16 = row16(lane);
+    const size_t at = static_cast<size_t>(row) * out + i;
+    float v[8], sv[8];
+    if constexpr (HALF) load8_half(static_cast<const uint16_t*>(z), at, v);
+    else load8_f32(static_cast<const float*>(z), at, v);
+    load8_half(svh, i, sv);
+    if (!HALF && defer) {
+        float xsum = 0.0f;
         for (uint32_t t = 0; t < inblk; ++t) xsum += xs[static_cast<size_t>(row) * inblk + t];
 #pragma unroll
-    for (uint32_t u = 0; u < kPfUnit; ++u) {
-        if (b0 + u >= nb) break;
-        if (!HALF && defer)
-#pragma unroll
-            for (uint32_t j = 0; j < 2u; ++j) v[u][j] = __builtin_fmaf(v[u][j], mul1_a(), mul1_b() * xsum);
-        finish_core(v[u], sv[u], lane);
-#pragma unroll
-        for (uint32_t j = 0; j < 2u; ++j)
-            store_act<DT>(y, static_cast<size_t>(row) * out + (b0 + u) * 128u + lane + 64u * j, v[u][j]);
+        for (uint32_t r = 0; r < 8u; ++r) v[r] = __builtin_fmaf(v[r], mul1_a(), mul1_b() * xsum);
     }
+    finish_row16(v, sv, g16);
+    if (live) store8_act<DT>(y, at, v);
 }
 
 inline dim3 unit_grid(uint32_t rows, uint32_t width) {
