@@ -376,6 +376,24 @@ def main() -> int:
         out["dense_prefill"] = {"workload": "4096 rows x (4096 -> 14336) K4 bf16", "ms_per_call": t * 1e3,
                                 "tflops": 2 * rows * in_f * out_f / t / 1e12,
                                 "frac_of_f16_mfma_peak": 2 * rows * in_f * out_f / t / 2.5e15}
+        # the same projection with its un-rotated weight resident (made once a weight): one plain GEMM a call
+        e0.record()
+        w_std, bad = api.unrot_weight(tr, suh, svh, dec, torch.bfloat16)
+        e1.record()
+        torch.cuda.synchronize()
+        once = e0.elapsed_time(e1)
+        api.linear_unrot(x, w_std)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(5):
+            api.linear_unrot(x, w_std)
+        e1.record()
+        torch.cuda.synchronize()
+        t = e0.elapsed_time(e1) * 1e-3 / 5
+        out["dense_prefill_unrot"] = {"workload": "the same, W_std bf16 resident (117 MB)", "ms_per_call": t * 1e3,
+                                      "tflops": 2 * rows * in_f * out_f / t / 1e12,
+                                      "frac_of_f16_mfma_peak": 2 * rows * in_f * out_f / t / 2.5e15,
+                                      "ms_to_make_w_std_once": once, "nonfinite": bad}
     if args.sweep:
         out["sweep"] = [measure(k, r, max(50, args.steps // 4), 10) for k in (3, 4, 5) for r in (1, 4, 16, 32)]
     if not args.no_cpu:

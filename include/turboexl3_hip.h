@@ -156,6 +156,24 @@ int32_t t3_linear_bias(t3_stream stream, const t3_array* x, const t3_array* trel
  * (src/core/format.zig:276-291; the role of src/core/dense.zig:909-922 `dequantize`). */
 int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_array* w_hat);
 
+/* The un-rotated weight of a dense linear, made once a weight (src/core/dense.zig:1600-1676 `unrotCols`, `unrotRows`,
+ * `unrotWeight`; src/root.zig:392-505 `trunkUnrot` installs it): W_std = act(((H' W_hat H)[i, o] / 128) suh[i] svh[o]),
+ * one rounding, written to columns [col0, col0 + out) of w_std [in, N] (F16 or BF16: the activation dtype). A join of up
+ * to four linears reading one x is one w_std with the members side by side (dense.zig:1613). Workspace: six bytes a
+ * weight (the W_hat and pass 1's f32 copy), as in the reference. `nonfinite` (device, may be null): a u32 the kernels
+ * add the number of weights that left the dtype's range to; the reference keeps such a group on its trellis path
+ * (root.zig:456-468). The caller zeroes it before and reads it after the stream has run. */
+int32_t t3_unrot_workspace_bytes(const t3_array* trellis, size_t* bytes);
+int32_t t3_unrot_weight(t3_stream stream, const t3_array* trellis, const t3_array* suh, const t3_array* svh,
+                        t3_decode dec, t3_array* w_std, int64_t col0, uint32_t* nonfinite, void* workspace,
+                        size_t workspace_bytes);
+/* y [rows, cols] = x [rows, in] W_std[:, col0 : col0 + cols], x, w_std and y in one dtype (F16 or BF16), f32
+ * accumulation: one plain GEMM (rocBLAS, opened at run time; without it T3_Exl3EngineNotImplemented). Up to 32 rows
+ * (src/core/dense.zig:1611 `unrot_min_rows`) it refuses with T3_Exl3EngineNotImplemented: decode and verify rows keep
+ * the trellis paths byte for byte. */
+int32_t t3_linear_unrot(t3_stream stream, const t3_array* x, const t3_array* w_std, int64_t col0, int64_t cols,
+                        t3_array* y);
+
 /* ---- routed experts (src/root.zig:822-904,976-1004) ------------------------------------------------------- */
 
 /* x [B, S, D]; inds (U32/I32) and scores (F32/BF16/F16) [B, S, K], K <= 32; y [B, S, D] in x's dtype.

@@ -155,6 +155,35 @@ def dequant(trellis, dec: Decode = Decode.mul1, stream=None) -> torch.Tensor:
     return w
 
 
+def unrot_weight(trellis, suh, svh, dec: Decode = Decode.mul1, dtype=torch.bfloat16, into=None, col0: int = 0,
+                 stream=None):
+    """The un-rotated weight W_std [in, out] in `dtype` (dense.unrotWeight), or written into columns col0.. of `into`
+    (a join: one [in, N] array, its members side by side). Returns (w_std, nonfinite count)."""
+    L = _lib.lib()
+    at = _arr(trellis)
+    if trellis.dim() != 3:
+        raise T3Error(1)
+    in_f, out_f = trellis.shape[0] * 16, trellis.shape[1] * 16
+    w = into if into is not None else torch.empty(in_f, out_f, dtype=dtype, device=trellis.device)
+    need = C.c_size_t(0)
+    _check(L.t3_unrot_workspace_bytes(C.byref(at), C.byref(need)))
+    ws = torch.empty(max(need.value, 256), dtype=torch.uint8, device=trellis.device)
+    bad = torch.zeros(1, dtype=torch.int32, device=trellis.device)
+    asu, asv, aw = _arr(suh), _arr(svh), _arr(w)
+    _check(L.t3_unrot_weight(_stream_ptr(stream), C.byref(at), C.byref(asu), C.byref(asv), dec.c(), C.byref(aw), col0,
+                             bad.data_ptr(), ws.data_ptr(), ws.numel()))
+    return w, int(bad.item())
+
+
+def linear_unrot(x, w_std, col0: int = 0, cols=None, stream=None) -> torch.Tensor:
+    """y = x W_std[:, col0 : col0 + cols]: one plain GEMM in the activation dtype (above 32 rows)."""
+    cols = w_std.shape[1] - col0 if cols is None else cols
+    y = torch.empty(*x.shape[:-1], cols, dtype=x.dtype, device=x.device)
+    ax, aw, ay = _arr(x), _arr(w_std), _arr(y)
+    _check(_lib.lib().t3_linear_unrot(_stream_ptr(stream), C.byref(ax), C.byref(aw), col0, cols, C.byref(ay)))
+    return y
+
+
 def _cbank(bank: Bank):
     keep = []
 

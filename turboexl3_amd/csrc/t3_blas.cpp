@@ -52,22 +52,28 @@ Blas& blas() {
 
 bool blas_available() { return blas().ok; }
 
-// z f16 [rows][out] = xp f16 [rows][in] * w_hat f16 [in][out], f32 accumulation, on `s`. Row-major operands are the
-// column-major (out x in) and (in x rows) of a plain N, N product.
-int32_t blas_gemm_f16(hipStream_t s, const uint16_t* xp, const uint16_t* w_hat, uint16_t* z, uint32_t rows, uint32_t in,
-                      uint32_t out) {
+// y [rows][cols] = x [rows][in] * w [in][cols of ldw], all f16 or all bf16, f32 accumulation, on `s`. Row-major
+// operands are the column-major (cols x in, leading dimension ldw) and (in x rows) of a plain N, N product.
+int32_t blas_gemm_half(hipStream_t s, bool bf16, const void* x, const void* w, uint32_t ldw, void* y, uint32_t rows,
+                       uint32_t in, uint32_t cols) {
     Blas& b = blas();
     if (!b.ok) return T3_Exl3EngineNotImplemented;
     const float one = 1.0f, zero = 0.0f;
+    const rocblas_datatype dt = bf16 ? rocblas_datatype_bf16_r : rocblas_datatype_f16_r;
     std::lock_guard<std::mutex> lock(b.mutex);
     if (b.set_stream(b.handle, s) != rocblas_status_success) return T3_HipFailed;
     const rocblas_status st = b.gemm_ex(
-        b.handle, rocblas_operation_none, rocblas_operation_none, static_cast<rocblas_int>(out),
-        static_cast<rocblas_int>(rows), static_cast<rocblas_int>(in), &one, w_hat, rocblas_datatype_f16_r,
-        static_cast<rocblas_int>(out), xp, rocblas_datatype_f16_r, static_cast<rocblas_int>(in), &zero, z,
-        rocblas_datatype_f16_r, static_cast<rocblas_int>(out), z, rocblas_datatype_f16_r, static_cast<rocblas_int>(out),
-        rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+        b.handle, rocblas_operation_none, rocblas_operation_none, static_cast<rocblas_int>(cols),
+        static_cast<rocblas_int>(rows), static_cast<rocblas_int>(in), &one, w, dt, static_cast<rocblas_int>(ldw), x, dt,
+        static_cast<rocblas_int>(in), &zero, y, dt, static_cast<rocblas_int>(cols), y, dt,
+        static_cast<rocblas_int>(cols), rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
     return st == rocblas_status_success ? T3_OK : T3_HipFailed;
+}
+
+// z f16 [rows][out] = xp f16 [rows][in] * w_hat f16 [in][out]
+int32_t blas_gemm_f16(hipStream_t s, const uint16_t* xp, const uint16_t* w_hat, uint16_t* z, uint32_t rows, uint32_t in,
+                      uint32_t out) {
+    return blas_gemm_half(s, false, xp, w_hat, out, z, rows, in, out);
 }
 
 }  // namespace t3

@@ -107,6 +107,11 @@ hipError_t launch_bias_add(void* y, const void* bias, uint32_t rows, uint32_t ou
 hipError_t launch_dequant(const uint32_t* trellis, uint16_t* w_hat, uint32_t in, uint32_t out, uint32_t n,
                           uint32_t wbits, int codebook, hipStream_t s);
 
+// W_hat f16 [in][out] -> the un-rotated weight in `dtype` (f16 or bf16) at columns col0.. of w_std [in][ld]; r: f32
+// [in][out] scratch; nonfinite: a counter of the weights that left the dtype's range (may be null)
+hipError_t launch_unrot(const uint16_t* w_hat, float* r, const uint16_t* suh, const uint16_t* svh, void* w_std, uint32_t in,
+                        uint32_t out, uint32_t ld, uint32_t col0, int dtype, uint32_t* nonfinite, hipStream_t s);
+
 // test kernels: every codeword's MCG and MUL1 value and MUL1 byte sum; every tile's 256 codewords by code position
 hipError_t launch_test_codebooks(uint16_t* mcg, uint16_t* mul1, uint16_t* t, hipStream_t s);
 hipError_t launch_test_lane(const uint32_t* trellis, uint32_t n, uint32_t wbits, uint32_t tiles, uint16_t* cw,

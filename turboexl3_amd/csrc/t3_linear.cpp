@@ -239,4 +239,75 @@ int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_
                                              static_cast<hipStream_t>(stream)));
 }
 
+int32_t t3_unrot_workspace_bytes(const t3_array* trellis, size_t* bytes) {
+    if (!bytes || !t3::array_ok(trellis)) return T3_BadArgs;
+    if (trellis->ndim != 3) return T3_BadExl3Shape;
+    const int64_t in = trellis->shape[0] * 16, out = trellis->shape[1] * 16;
+    if (in <= 0 || out <= 0) return T3_BadExl3Shape;
+    t3::Carver c(nullptr);
+    c.take<uint16_t>(static_cast<size_t>(in) * out * 2u);
+    c.take<float>(static_cast<size_t>(in) * out * 4u);
+    *bytes = c.used;
+    return T3_OK;
+}
+
+int32_t t3_unrot_weight(t3_stream stream, const t3_array* trellis, const t3_array* suh, const t3_array* svh,
+                        t3_decode dec, t3_array* w_std, int64_t col0, uint32_t* nonfinite, void* workspace,
+                        size_t workspace_bytes) {
+    if (!t3::array_ok(trellis) || !t3::array_ok(suh) || !t3::array_ok(svh) || !t3::array_ok(w_std) || !workspace)
+        return T3_BadArgs;
+    if (trellis->ndim != 3 || w_std->ndim != 2 || suh->ndim != 1 || svh->ndim != 1) return T3_BadExl3Shape;
+    const int64_t in = trellis->shape[0] * 16, out = trellis->shape[1] * 16, n = trellis->shape[2];
+    if (!t3::rate_ok(n) || in <= 0 || out <= 0 || in % 128 != 0 || out % 128 != 0 || in > (1ll << 30) ||
+        out > (1ll << 30))
+        return T3_BadExl3Shape;
+    if (suh->shape[0] != in || svh->shape[0] != out || w_std->shape[0] != in || col0 < 0 || col0 % 8 != 0 ||
+        col0 + out > w_std->shape[1] || w_std->shape[1] > (1ll << 30))
+        return T3_BadExl3Shape;
+    if ((trellis->dtype != T3_U16 && trellis->dtype != T3_I16) || suh->dtype != T3_F16 || svh->dtype != T3_F16 ||
+        (w_std->dtype != T3_F16 && w_std->dtype != T3_BF16))
+        return T3_BadExl3Dtype;
+    t3::Dec d;
+    if (const int32_t st = t3::resolve_decode(dec, &d); st != T3_OK) return st;
+    t3::Carver c(workspace);
+    uint16_t* w_hat = c.take<uint16_t>(static_cast<size_t>(in) * out * 2u);
+    float* r = c.take<float>(static_cast<size_t>(in) * out * 4u);
+    if (workspace_bytes < c.used) return T3_WorkspaceTooSmall;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (const int32_t st = t3::hip_status(t3::launch_dequant(static_cast<const uint32_t*>(trellis->data), w_hat,
+                                                             static_cast<uint32_t>(in), static_cast<uint32_t>(out),
+                                                             static_cast<uint32_t>(n), d.wbits, d.codebook, s));
+        st != T3_OK)
+        return st;
+    return t3::hip_status(t3::launch_unrot(w_hat, r, static_cast<const uint16_t*>(suh->data),
+                                           static_cast<const uint16_t*>(svh->data), w_std->data,
+                                           static_cast<uint32_t>(in), static_cast<uint32_t>(out),
+                                           static_cast<uint32_t>(w_std->shape[1]), static_cast<uint32_t>(col0),
+                                           w_std->dtype, nonfinite, s));  // T3_F16, T3_BF16 = the kernels' numbering
+}
+
+int32_t t3_linear_unrot(t3_stream stream, const t3_array* x, const t3_array* w_std, int64_t col0, int64_t cols,
+                        t3_array* y) {
+    if (!t3::array_ok(x) || !t3::array_ok(w_std) || !t3::array_ok(y)) return T3_BadArgs;
+    if (x->ndim < 1 || w_std->ndim != 2 || y->ndim != x->ndim) return T3_BadExl3Shape;
+    const int64_t in = w_std->shape[0];
+    int64_t rows = 1;
+    for (int i = 0; i + 1 < x->ndim; ++i) {
+        if (x->shape[i] != y->shape[i]) return T3_BadExl3Shape;
+        rows *= x->shape[i];
+    }
+    if (x->shape[x->ndim - 1] != in || y->shape[y->ndim - 1] != cols || col0 < 0 || cols <= 0 ||
+        col0 + cols > w_std->shape[1] || rows <= 0 || rows > (1ll << 30) || in > (1ll << 30) ||
+        w_std->shape[1] > (1ll << 30))
+        return T3_BadExl3Shape;
+    if ((w_std->dtype != T3_F16 && w_std->dtype != T3_BF16) || x->dtype != w_std->dtype || y->dtype != w_std->dtype)
+        return T3_BadExl3Dtype;
+    if (rows <= 32 || !t3::blas_available()) return T3_Exl3EngineNotImplemented;
+    const size_t esz = 2u;
+    return t3::blas_gemm_half(static_cast<hipStream_t>(stream), w_std->dtype == T3_BF16, x->data,
+                              static_cast<const unsigned char*>(w_std->data) + static_cast<size_t>(col0) * esz,
+                              static_cast<uint32_t>(w_std->shape[1]), y->data, static_cast<uint32_t>(rows),
+                              static_cast<uint32_t>(in), static_cast<uint32_t>(cols));
+}
+
 }  // extern "C"
