@@ -210,6 +210,19 @@ int32_t t3_moe_with_shared(t3_stream stream, const t3_array* x, const t3_bank* b
 int32_t t3_moe_shared_expert(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
                              const t3_array* scores, t3_decode dec, int32_t limit, const t3_bank* shared_bank,
                              t3_array* y, void* workspace, size_t workspace_bytes);
+/* Decode / verify rows (up to T3_SHARED_ROWS_MAX) of a MoE with a GATED shared expert inside the routed launches
+ * (src/models/qwen38/api.zig:305-312 `moeFusedShared`): y = routed + sigmoid(logit) * shared(x), with the roundings of
+ * the host's chain it stands for: the routed sum rounds to x's dtype; the shared expert's SwiGLU is the table form in
+ * x's dtype (g * sigtab[g]) * u, one rounding an operation (src/models/qwen38/kernels/shared/shared_fin_head_4.metal:1-9);
+ * its output rounds to the dtype, is multiplied by sigtab[logit[row]], rounds, and the add rounds (dfin7s.metal:44-50).
+ * x F16 or BF16; shared_bank: one expert, the routed bank's widths and rates; sigtab [65536] in x's dtype: the sigmoid
+ * of every 16-bit pattern (the host's table); logit [rows] in x's dtype. No clamp. Anything else:
+ * T3_Exl3EngineNotImplemented before any launch (the caller keeps its chain). Workspace: t3_moe_workspace_bytes with
+ * shared_bank. */
+#define T3_SHARED_ROWS_MAX 4 /* src/models/qwen38/shared.zig:346 */
+int32_t t3_moe_fused_shared(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
+                            const t3_array* scores, t3_decode dec, const t3_bank* shared_bank, const t3_array* sigtab,
+                            const t3_array* logit, t3_array* y, void* workspace, size_t workspace_bytes);
 /* shared_bank: NULL, or the bank `t3_moe_shared_expert` will take (its slots need scratch too). */
 int32_t t3_moe_workspace_bytes(const t3_array* x, const t3_bank* bank, const t3_array* inds,
                                const t3_bank* shared_bank, size_t* bytes);

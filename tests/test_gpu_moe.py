@@ -272,3 +272,82 @@ def test_silu_out_clamp_decode_and_prefill_rows(oracle, t3):
     with pytest.raises(t3.T3Error) as e:
         t3.moe_swiglu(*args, 5, 2)
     assert e.value.name == "InvalidExl3Clamp"
+
+
+def sigmoid_table(dtype):
+    """The host's table: the sigmoid of every 16-bit pattern of `dtype`, in `dtype` (what MLX's Sigmoid gives the
+    reference; torch's here)."""
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16)
+    return torch.sigmoid(bits.view(dtype).to(torch.float32)).to(dtype)
+
+
+def _to(dtype, a):
+    """float32 values rounded to `dtype` and back."""
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(dtype).to(torch.float32).numpy()
+
+
+def _tab(table_f32, dtype, a):
+    """table[bits of a] for values already of `dtype`."""
+    bits = torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(dtype).view(torch.int16).to(torch.int32) & 0xFFFF
+    return table_f32[bits.numpy()]
+
+
+@pytest.mark.parametrize("codebook,n,dtype", [(MCG, 64, torch.bfloat16), (MUL1, 48, torch.float16)])
+def test_fused_gated_shared_expert(oracle, t3, codebook, n, dtype):
+    # src/models/qwen38/api.zig:305-312: y = routed + sigmoid(logit) * shared(x) at up to 4 rows, with the roundings of
+    # the host's chain (the routed sum, the table SwiGLU, the gate, the product and the add each round to the dtype)
+    rng = np.random.default_rng(0x5A3 + n)
+    hidden, inter, experts, topk = 512, 256, 8, 4
+    bank, shared = oracle.synth_bank(rng, experts, hidden, inter, n), oracle.synth_bank(rng, 1, hidden, inter, n)
+    dbank, dshared = dev_bank(t3, bank), dev_bank(t3, shared)
+    ref, sref = RefBank(oracle, bank, codebook, 0xFFFF), RefBank(oracle, shared, codebook, 0xFFFF)
+    dec = t3.Decode(codebook, 16)
+    rows = 4
+    x_dev, x_f32 = make_x(rng, rows, hidden, dtype)
+    slots, scores = routing(rng, rows, topk, experts)
+    slots[1, 2] = -1
+    logit = torch.from_numpy(rng.standard_normal(rows).astype(np.float32)).to(dtype)
+    table = sigmoid_table(dtype)
+    table_f32 = table.to(torch.float32).numpy()
+    want = []
+    for r in range(rows):
+        routed = _to(dtype, ref.row(x_f32[r], slots[r], scores[r]))
+        gt, ut = _to(dtype, sref.project("gate", 0, x_f32[r])), _to(dtype, sref.project("up", 0, x_f32[r]))
+        act = _to(dtype, gt * _tab(table_f32, dtype, gt))
+        h = _to(dtype, act * ut)
+        sterm = _to(dtype, sref.project("down", 0, h))
+        gated = _to(dtype, _tab(table_f32, dtype, logit[r:r + 1].to(torch.float32).numpy()) * sterm)
+        want.append(_to(dtype, routed + gated))
+    d_slots = torch.from_numpy(slots).cuda()
+    d_scores = torch.from_numpy(scores).cuda()
+    first = None
+    # bf16: the output passes three roundings of the dtype at the end (the routed sum, the gated product, the add) where
+    # `moe` has one, and a step of bf16 at 4 rms is 3e-2 of rms: the dense bar (src/hip_tests.zig:326), not the routed
+    # one. f16: two steps of f16 at 4 rms (8e-3 of rms) on top of the f32 bar's share
+    bar = 2.5e-2 if dtype == torch.bfloat16 else 1e-2
+    for form in (9, 4, 3):
+        t3.configure(decode_form=form)
+        try:
+            for count in (1, 3, 4):
+                y = t3.moe_fused_shared(x_dev[:count].reshape(1, count, hidden), dbank,
+                                        d_slots[:count].reshape(1, count, topk), d_scores[:count].reshape(1, count, topk),
+                                        dec, dshared, table.cuda(), logit[:count].cuda())
+                got = to_f32(y).reshape(count, hidden)
+                for r in range(count):
+                    e = oracle.compare(got[r], want[r])
+                    assert e <= bar, f"form {form} rows {count} row {r}: {e:.3e} over the bar {bar}"
+                if count == 4:
+                    if first is None:
+                        first = bytes_of(y)
+                    else:
+                        assert bytes_of(y) == first, f"form {form}: other bytes than the two-launch form"
+        finally:
+            t3.configure()
+    # beyond the shared rows the fused launches refuse, and so does an f32 call: the caller keeps its chain
+    x5, _ = make_x(rng, 5, hidden, dtype)
+    s5, w5 = routing(rng, 5, topk, experts)
+    with pytest.raises(t3.T3Error) as err:
+        t3.moe_fused_shared(x5.reshape(1, 5, hidden), dbank, torch.from_numpy(s5).cuda().reshape(1, 5, topk),
+                            torch.from_numpy(w5).cuda().reshape(1, 5, topk), dec, dshared, table.cuda(),
+                            torch.zeros(5, dtype=dtype, device="cuda"))
+    assert err.value.name == "Exl3EngineNotImplemented"

@@ -289,6 +289,21 @@ def moe_shared_expert(x, bank: Bank, inds, scores, dec: Decode, limit: int, shar
     return y
 
 
+def moe_fused_shared(x, bank: Bank, inds, scores, dec: Decode, shared_bank: Bank, sigtab, logit, stream=None) -> torch.Tensor:
+    """qwen38's moeFusedShared at decode rows: routed + sigmoid(logit) * shared(x) inside the routed launches; sigtab
+    [65536] in x's dtype (the sigmoid of every 16-bit pattern), logit [rows] in x's dtype."""
+    L = _lib.lib()
+    ax, ai, asc = _arr(x), _arr(inds), _arr(scores)
+    cb, _keep = _cbank(bank)
+    sb, _keep2 = _cbank(shared_bank)
+    ws = _moe_workspace(L, ax, cb, ai, x.device, sb)
+    y = torch.empty_like(x)
+    ay, at, al = _arr(y), _arr(sigtab), _arr(logit)
+    _check(L.t3_moe_fused_shared(_stream_ptr(stream), C.byref(ax), C.byref(cb), C.byref(ai), C.byref(asc), dec.c(),
+                                 C.byref(sb), C.byref(at), C.byref(al), C.byref(ay), ws.data_ptr(), ws.numel()))
+    return y
+
+
 # ---- device self-tests -------------------------------------------------------------------------------------
 
 def test_codebooks(device="cuda"):

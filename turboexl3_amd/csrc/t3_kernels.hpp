@@ -56,6 +56,10 @@ struct MoeLaunch {
     const int32_t* slots = nullptr;  // [rows][topk] expert ids
     const void* scores = nullptr;    // [rows][topk] in score_dt
     const void* shared_add = nullptr;  // moeWithShared: [rows][hidden] in dtype, or null
+    // the gated shared expert (src/models/qwen38/api.zig:305-312): sigtab [65536] in dtype = the sigmoid of every 16-bit
+    // pattern, slogit [rows] in dtype = the shared gate's logit; null: the shared slots are summed at weight 1
+    const void* sigtab = nullptr;
+    const void* slogit = nullptr;
     void* y = nullptr;
     uint32_t* arrive = nullptr;  // the two-launch form's arrival counters
     uint32_t* xg = nullptr;      // u32 [RKT][hidden]
@@ -90,9 +94,9 @@ enum MoeForm : int { kMoeFiveLaunches = 0, kMoeFourLaunches = 1, kMoeTwoLaunches
 hipError_t launch_moe_decode(const MoeLaunch& a, int form, hipStream_t s);
 
 // The same call above the decode rows: route, prepare, gate|up GEMM, mid, down GEMM, combine. xg, xu, hd hold plain f16
-// here (quad order), zg, zu, zd one plane each, all by sorted position.
+// here (pair-quad order), zg, zu, zd one plane each, all by sorted position.
 hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s);
-// One dense projection above 32 rows: prepare (f16, quad order), the trellis GEMM, finish. xq holds plain f16; ks = 1.
+// One dense projection above 32 rows: prepare (f16, pair-quad order), the trellis GEMM, finish. xq holds plain f16; ks = 1.
 hipError_t launch_dense_prefill(const DenseLaunch& d, hipStream_t s);
 
 // The W_hat form's own stages: the prepare in natural order (plain f16 [rows][in], what a plain GEMM multiplies), and the

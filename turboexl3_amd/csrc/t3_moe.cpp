@@ -278,4 +278,32 @@ int32_t t3_moe_shared_expert(t3_stream stream, const t3_array* x, const t3_bank*
     return t3::run_moe(stream, x, bank, inds, scores, shared_bank, nullptr, dec, limit, y, workspace, workspace_bytes);
 }
 
+int32_t t3_moe_fused_shared(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
+                            const t3_array* scores, t3_decode dec, const t3_bank* shared_bank, const t3_array* sigtab,
+                            const t3_array* logit, t3_array* y, void* workspace, size_t workspace_bytes) {
+    if (!shared_bank || !scores || !y || !t3::array_ok(sigtab) || !t3::array_ok(logit)) return T3_BadArgs;
+    t3::MoeCall call;
+    if (const int32_t st = t3::check_moe(x, bank, inds, scores, shared_bank, nullptr, dec, 0, y, &call, 0); st != T3_OK)
+        return st;
+    // what the fused launches do not carry stays with the caller's chain (src/models/qwen38/api.zig:312-322)
+    t3::MoeLaunch& l = call.launch;
+    int64_t tab = 1, lg = 1;
+    for (int i = 0; i < sigtab->ndim; ++i) tab *= sigtab->shape[i];
+    for (int i = 0; i < logit->ndim; ++i) lg *= logit->shape[i];
+    if (call.rows > T3_SHARED_ROWS_MAX || l.shared_slots != 1u || (x->dtype != T3_F16 && x->dtype != T3_BF16) ||
+        sigtab->dtype != x->dtype || tab != 65536 || logit->dtype != x->dtype || lg != static_cast<int64_t>(call.rows))
+        return T3_Exl3EngineNotImplemented;
+    if (!workspace) return T3_BadArgs;
+    t3::carve_moe(&call, workspace);
+    if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
+    l.sigtab = sigtab->data;
+    l.slogit = logit->data;
+    const size_t widest = (l.hidden > l.inter ? l.hidden : l.inter) / 128u;
+    const size_t counters = static_cast<size_t>(l.rows) * (l.topk + l.shared_slots) * widest;
+    const int form = t3::config().decode_form == 3 ? t3::kMoeFiveLaunches
+                     : t3::config().decode_form == 4 || counters * 4u > t3::kCounterBytes ? t3::kMoeFourLaunches
+                                                                                          : t3::kMoeTwoLaunches;
+    return t3::hip_status(t3::launch_moe_decode(l, form, static_cast<hipStream_t>(stream)));
+}
+
 }  // extern "C"

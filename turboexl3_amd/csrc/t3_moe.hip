@@ -170,7 +170,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
             // The slots' finishes sixteen at a time, four a wave (slot k0 + 4 r + wave) with every load of the four in
             // flight together; wave 0 adds them in slot order.
             float(*fin)[128] = reinterpret_cast<float(*)[128]>(smem);
-            float acc2[2] = {0.0f, 0.0f};
+            float acc2[2] = {0.0f, 0.0f}, gated[2] = {0.0f, 0.0f};
             for (uint32_t k0 = 0; k0 < kt; k0 += 16u) {
                 SlotRef sk[4];
                 uint32_t qk[4];
@@ -196,13 +196,18 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
                 if (sg == 0u)
                     for (uint32_t w = 0; w < 16u && k0 + w < kt; ++w) {
                         if (cinfo[k0 + w] == 0xFFFFFFFFu) continue;
+                        if (a.sigtab && (cinfo[k0 + w] >> 31) != 0u) {  // the gated shared expert's slot
+                            gated[0] = gated_term(a, s.row, fin[w][lane]);
+                            gated[1] = gated_term(a, s.row, fin[w][lane + 64u]);
+                            continue;
+                        }
                         const float wgt = cscore[k0 + w];
                         acc2[0] = __builtin_fmaf(wgt, fin[w][lane], acc2[0]);
                         acc2[1] = __builtin_fmaf(wgt, fin[w][lane + 64u], acc2[1]);
                     }
                 __syncthreads();
             }
-            if (sg == 0u) routed_store_row(a, s.row, b128, lane, acc2);
+            if (sg == 0u) routed_store_row(a, s.row, b128, lane, acc2, a.sigtab ? gated : nullptr);
         }
     }
 }

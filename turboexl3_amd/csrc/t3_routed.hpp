@@ -39,6 +39,30 @@ __device__ __forceinline__ float score_of(const MoeLaunch& a, uint32_t row, uint
     return bf16_value(static_cast<const uint16_t*>(a.scores)[i]);
 }
 
+// The gated shared expert's arithmetic lives in the activation dtype (f16 or bf16), one rounding an operation, as the
+// host's chain of MLX operations it stands for (src/models/qwen38/kernels/shared/shared_fin_head_4.metal:1-9,
+// dfin7s.metal:44-50).
+__device__ __forceinline__ float round_act(int dt, float v) {
+    return dt == kF16 ? round_half(v) : (dt == kBf16 ? bf16_value(bf16_bits(v)) : v);
+}
+// sigtab's entry for the 16-bit pattern of v (already a value of the dtype)
+__device__ __forceinline__ float sigmoid_of(const MoeLaunch& a, float v) {
+    const uint32_t bits = a.dtype == kF16 ? half_bits(v) : bf16_bits(v);
+    const uint16_t t = static_cast<const uint16_t*>(a.sigtab)[bits];
+    return a.dtype == kF16 ? half_value(t) : bf16_value(t);
+}
+// h = ((g * sigmoid(g)) * u), every step in the dtype
+__device__ __forceinline__ float swiglu_table(const MoeLaunch& a, float g, float u) {
+    const float gt = round_act(a.dtype, g), ut = round_act(a.dtype, u);
+    const float act = round_act(a.dtype, gt * sigmoid_of(a, gt));
+    return round_act(a.dtype, act * ut);
+}
+// the shared slot's term of a row's output: sigmoid(logit[row]) * dtype(v), in the dtype
+__device__ __forceinline__ float gated_term(const MoeLaunch& a, uint32_t row, float v) {
+    const float logit = load_act_rt(a.dtype, a.slogit, row);
+    return round_act(a.dtype, sigmoid_of(a, logit) * round_act(a.dtype, v));
+}
+
 // One block's sums over the K slices (slice order; the first plane starts the sum) and the deferred MUL1 map.
 // COH: the planes and block sums were stored by other workgroups of this launch.
 // Loads go out eight at a time and are added in slice (or block) order: the sums do not depend on the batching, and a
@@ -174,7 +198,10 @@ __device__ __forceinline__ void routed_mid_block(const MoeLaunch& a, const SlotR
     finish_core(u, svu, lane);
     float d[2];
 #pragma unroll
-    for (uint32_t j = 0; j < 2u; ++j) d[j] = round_half(swiglu_clamped(g[j], u[j], a.limit, a.clamp_at)) * sdn[j];
+    for (uint32_t j = 0; j < 2u; ++j) {
+        const float h = s.shared && a.sigtab ? swiglu_table(a, g[j], u[j]) : swiglu_clamped(g[j], u[j], a.limit, a.clamp_at);
+        d[j] = round_half(h) * sdn[j];
+    }
     h128_wave(d, lane);
     float sum = 0.0f;
 #pragma unroll
@@ -248,18 +275,17 @@ __device__ __forceinline__ void routed_down_finish_many(const MoeLaunch& a, cons
     }
 }
 
-// a row's block b from its f32 sums: y's dtype, or `moeWithShared`'s two roundings
+// a row's block b from its f32 sums: y's dtype; or two roundings: the routed output rounds to x's dtype, then the add
+// of `moeWithShared`'s tensor (src/root.zig:976-984) or of the gated shared expert's term (`gated`, null: none) rounds
+// again
 __device__ __forceinline__ void routed_store_row(const MoeLaunch& a, uint32_t row, uint32_t b, uint32_t lane,
-                                                 const float (&acc)[2]) {
+                                                 const float (&acc)[2], const float* gated = nullptr) {
 #pragma unroll
     for (uint32_t j = 0; j < 2u; ++j) {
         const size_t o = static_cast<size_t>(row) * a.hidden + b * 128u + lane + 64u * j;
-        if (a.shared_add) {
-            // the routed output rounds to x's dtype, then the add rounds again (src/root.zig:976-984)
-            float r = acc[j];
-            if (a.dtype == kF16) r = round_half(r);
-            else if (a.dtype == kBf16) r = bf16_value(bf16_bits(r));
-            store_act_rt(a.dtype, a.y, o, r + load_act_rt(a.dtype, a.shared_add, o));
+        if (a.shared_add || gated) {
+            const float r = round_act(a.dtype, acc[j]);
+            store_act_rt(a.dtype, a.y, o, r + (gated ? gated[j] : load_act_rt(a.dtype, a.shared_add, o)));
         } else {
             store_act_rt(a.dtype, a.y, o, acc[j]);
         }
@@ -270,18 +296,23 @@ __device__ __forceinline__ void routed_store_row(const MoeLaunch& a, uint32_t ro
 template <bool PF>
 __device__ __forceinline__ void routed_combine_block(const MoeLaunch& a, uint32_t row, uint32_t b, uint32_t lane) {
     const uint32_t kt = a.topk + a.shared_slots;
-    float acc[2] = {0.0f, 0.0f};
+    float acc[2] = {0.0f, 0.0f}, gated[2] = {0.0f, 0.0f};
     for (uint32_t k = 0; k < kt; ++k) {
         const uint32_t rk = row * kt + k;
         const SlotRef s = resolve_slot(a, rk);
         if (!s.live) continue;  // uniform over the wave
         float v[2];
         routed_down_finish<false>(a, s, PF ? a.inv[rk] : rk, b, lane, v, PF ? 1u : a.ks_dn);
+        if (s.shared && a.sigtab) {
+            gated[0] = gated_term(a, row, v[0]);
+            gated[1] = gated_term(a, row, v[1]);
+            continue;
+        }
         const float w = s.shared ? 1.0f : score_of(a, row, k);
 #pragma unroll
         for (uint32_t j = 0; j < 2u; ++j) acc[j] = __builtin_fmaf(w, v[j], acc[j]);
     }
-    routed_store_row(a, row, b, lane, acc);
+    routed_store_row(a, row, b, lane, acc, a.sigtab ? gated : nullptr);
 }
 
 }  // namespace t3
