@@ -73,7 +73,9 @@ typedef enum t3_dtype {
 
 #define T3_MAX_DIMS 8
 
-/* A row-contiguous device array: what an mlx_array handle carries for this path. */
+/* A row-contiguous device array: what an mlx_array handle carries for this path. Activations (x, y, an added shared
+ * output), scale vectors and trellises start on a 16-byte boundary and a workspace on a 256-byte one (any allocation
+ * or whole-row view does): the kernels read them 16 bytes a lane. T3_BadArgs otherwise. */
 typedef struct t3_array {
     void* data;
     int32_t ndim;

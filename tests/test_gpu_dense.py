@@ -175,3 +175,16 @@ def test_linear_bias_is_linear_plus_one_rounded_add(oracle, t3):
     with pytest.raises(t3.T3Error) as e:
         t3.linear_bias(x_dev, case.d_trellis, case.d_suh, case.d_svh, bias.to(torch.float16), case.dec)
     assert e.value.name == "BadExl3Dtype"
+
+
+def test_misaligned_arrays_are_refused(oracle, t3):
+    # the kernels read 16 bytes a lane: an activation or scale array that starts off a 16-byte boundary is refused
+    # before any launch
+    case = DenseCase(oracle, t3, 5, 256, 256, 64, MCG, 16)
+    x = torch.zeros(2 * 256 + 4, dtype=torch.float16, device="cuda")
+    ok = x[:512].reshape(2, 256)
+    off = x[4:516].reshape(2, 256)  # 8 bytes in
+    t3.linear(ok, case.d_trellis, case.d_suh, case.d_svh, case.dec)
+    with pytest.raises(t3.T3Error) as e:
+        t3.linear(off, case.d_trellis, case.d_suh, case.d_svh, case.dec)
+    assert e.value.name == "BadArgs"

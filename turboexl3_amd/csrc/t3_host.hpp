@@ -23,6 +23,12 @@ inline bool array_ok(const t3_array* a) {
     return true;
 }
 
+// The kernels read activations, scale vectors and trellises 16 bytes a lane and carve the workspace in 256-byte steps:
+// an array they touch that way starts on a 16-byte boundary, the workspace on a 256-byte one (what hipMalloc and any
+// tensor library's allocations and whole-row views give).
+inline bool aligned16(const t3_array* a) { return (reinterpret_cast<uintptr_t>(a->data) & 15u) == 0u; }
+inline bool workspace_ok(const void* w) { return w && (reinterpret_cast<uintptr_t>(w) & 255u) == 0u; }
+
 inline bool is_act_dtype(int32_t d) { return d == T3_F32 || d == T3_F16 || d == T3_BF16; }
 inline size_t dtype_size(int32_t d) { return d == T3_F32 || d == T3_U32 || d == T3_I32 ? 4 : 2; }
 

@@ -16,6 +16,8 @@ int32_t check_dense(const t3_array* x, const t3_array* trellis, const t3_array* 
                     t3_decode dec, const t3_array* y, uint32_t max_rows, DenseCall* call) {
     if (!array_ok(x) || !array_ok(trellis) || (suh && !array_ok(suh)) || (svh && !array_ok(svh)) || (y && !array_ok(y)))
         return T3_BadArgs;
+    if (!aligned16(x) || !aligned16(trellis) || (suh && !aligned16(suh)) || (svh && !aligned16(svh)) || (y && !aligned16(y)))
+        return T3_BadArgs;
     if (x->ndim < 1 || trellis->ndim != 3) return T3_BadExl3Shape;
     const int64_t in = trellis->shape[0] * 16, out = trellis->shape[1] * 16, n = trellis->shape[2];
     if (!rate_ok(n)) return T3_BadExl3Shape;
@@ -177,7 +179,7 @@ int32_t t3_linear_stages(t3_stream stream, const t3_array* x, const t3_array* tr
     if (stages == 0u || stages > 7u) return T3_BadArgs;
     t3::DenseCall call;
     if (const int32_t st = t3::check_dense(x, trellis, suh, svh, dec, y, 32, &call); st != T3_OK) return st;
-    if (!workspace) return T3_BadArgs;
+    if (!t3::workspace_ok(workspace)) return T3_BadArgs;
     t3::carve_dense(&call, workspace);
     if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
     return t3::run_chain(call, static_cast<hipStream_t>(stream), stages);
@@ -188,7 +190,7 @@ int32_t t3_linear(t3_stream stream, const t3_array* x, const t3_array* trellis, 
     if (!suh || !svh || !y) return T3_BadArgs;
     t3::DenseCall call;
     if (const int32_t st = t3::check_dense(x, trellis, suh, svh, dec, y, 0, &call); st != T3_OK) return st;
-    if (!workspace) return T3_BadArgs;
+    if (!t3::workspace_ok(workspace)) return T3_BadArgs;
     if (call.launch.rows > t3::kGemvRowsMax) {
         if (!t3::config().prefill) return T3_Exl3EngineNotImplemented;
         if (t3::takes_w_hat(call.launch)) {
@@ -254,7 +256,7 @@ int32_t t3_unrot_workspace_bytes(const t3_array* trellis, size_t* bytes) {
 int32_t t3_unrot_weight(t3_stream stream, const t3_array* trellis, const t3_array* suh, const t3_array* svh,
                         t3_decode dec, t3_array* w_std, int64_t col0, uint32_t* nonfinite, void* workspace,
                         size_t workspace_bytes) {
-    if (!t3::array_ok(trellis) || !t3::array_ok(suh) || !t3::array_ok(svh) || !t3::array_ok(w_std) || !workspace)
+    if (!t3::array_ok(trellis) || !t3::array_ok(suh) || !t3::array_ok(svh) || !t3::array_ok(w_std) || !t3::workspace_ok(workspace))
         return T3_BadArgs;
     if (trellis->ndim != 3 || w_std->ndim != 2 || suh->ndim != 1 || svh->ndim != 1) return T3_BadExl3Shape;
     const int64_t in = trellis->shape[0] * 16, out = trellis->shape[1] * 16, n = trellis->shape[2];

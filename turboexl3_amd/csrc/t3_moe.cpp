@@ -15,6 +15,7 @@ struct MoeCall {
 // One projection's arrays against the geometry (src/root.zig:87-102).
 int32_t check_proj(const t3_proj& p, int64_t experts, int64_t in, int64_t out, int64_t* n) {
     if (!array_ok(&p.trellis) || !array_ok(&p.suh) || !array_ok(&p.svh)) return T3_BadArgs;
+    if (!aligned16(&p.trellis) || !aligned16(&p.suh) || !aligned16(&p.svh)) return T3_BadArgs;
     const t3_array& t = p.trellis;
     if (in <= 0 || out <= 0 || in % 128 != 0 || out % 128 != 0 || t.ndim != 4 || t.shape[0] != experts ||
         t.shape[1] != in / 16 || t.shape[2] != out / 16 || !rate_ok(t.shape[3]) || p.suh.ndim != 2 ||
@@ -62,6 +63,7 @@ int32_t check_moe(const t3_array* x, const t3_bank* bank, const t3_array* inds, 
     if (!array_ok(x) || !array_ok(inds) || (scores && !array_ok(scores)) || (y && !array_ok(y)) ||
         (shared_add && !array_ok(shared_add)))
         return T3_BadArgs;
+    if (!aligned16(x) || (y && !aligned16(y)) || (shared_add && !aligned16(shared_add))) return T3_BadArgs;
     if (x->ndim != 3 || inds->ndim != 3 || x->shape[0] <= 0 || x->shape[1] <= 0 || x->shape[0] != inds->shape[0] ||
         x->shape[1] != inds->shape[1] || inds->shape[2] <= 0 || inds->shape[2] > T3_REDUCE_MAX_TOPK)
         return T3_BadExl3Shape;
@@ -198,7 +200,7 @@ int32_t run_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const 
     if (const int32_t st = check_moe(x, bank, inds, scores, shared_bank, shared_add, dec, limit, y, &call, clamp_at);
         st != T3_OK)
         return st;
-    if (!workspace) return T3_BadArgs;
+    if (!workspace_ok(workspace)) return T3_BadArgs;
     // rows above the decode chain's take the prefill GEMM chain (src/root.zig:850-853)
     if (call.rows > T3_DECODE_ROWS_MAX) {
         if (const int32_t st = admit_prefill(call); st != T3_OK) return st;
@@ -293,7 +295,7 @@ int32_t t3_moe_fused_shared(t3_stream stream, const t3_array* x, const t3_bank* 
     if (call.rows > T3_SHARED_ROWS_MAX || l.shared_slots != 1u || (x->dtype != T3_F16 && x->dtype != T3_BF16) ||
         sigtab->dtype != x->dtype || tab != 65536 || logit->dtype != x->dtype || lg != static_cast<int64_t>(call.rows))
         return T3_Exl3EngineNotImplemented;
-    if (!workspace) return T3_BadArgs;
+    if (!t3::workspace_ok(workspace)) return T3_BadArgs;
     t3::carve_moe(&call, workspace);
     if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
     l.sigtab = sigtab->data;
