@@ -79,6 +79,27 @@ def test_config5_dense_4096_rows_w_hat_form(oracle, t3):
             assert oracle.compare(got[i, 128 * blk:128 * blk + 128], ref[i]) <= BF16_DENSE_BAR, (blk, sample[i])
 
 
+def test_config5_shape_few_rows_on_the_trellis_gemm(oracle, t3):
+    # few rows decode the matrix once: the launch shares the tile rows out into K parts (eight at 64 rows here, two at
+    # 600) and one item's column blocks go round all the dies; sampled blocks against the oracle either way
+    in_f, out_f, n = 4096, 14336, 64
+    rng = np.random.default_rng(0xC56)
+    trellis, suh, svh = oracle.synth_linear(rng, in_f, out_f, n)
+    d_t, d_suh, d_svh = dev_u16(trellis), dev_f16_bits(suh), dev_f16_bits(svh)
+    x_dev, x_f32 = make_x(rng, 600, in_f, torch.bfloat16)
+    t3.configure(dense_gemm_rows=0)  # keep 600 rows on the trellis GEMM
+    try:
+        for rows, sample in ((64, [0, 33, 63]), (600, [0, 300, 599])):
+            got = to_f32(t3.linear(x_dev[:rows], d_t, d_suh, d_svh, t3.Decode.mcg)[sample])
+            for blk in (0, 57, out_f // 128 - 1):
+                ref = block_ref(oracle, trellis, suh, svh, x_f32[sample], in_f, n, MCG, blk)
+                for i in range(len(sample)):
+                    e = oracle.compare(got[i, 128 * blk:128 * blk + 128], ref[i])
+                    assert e <= BF16_DENSE_BAR, (rows, blk, sample[i], e)
+    finally:
+        t3.configure()
+
+
 def routing_softmax(rng, tokens, topk, experts):
     logits = rng.standard_normal((tokens, experts)).astype(np.float32)
     slots = np.argsort(-logits, axis=1)[:, :topk].astype(np.int32)

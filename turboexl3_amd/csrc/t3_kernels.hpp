@@ -98,6 +98,16 @@ hipError_t launch_moe_decode(const MoeLaunch& a, int form, hipStream_t s);
 hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s);
 // One dense projection above 32 rows: prepare (f16, pair-quad order), the trellis GEMM, finish. xq holds plain f16; ks = 1.
 hipError_t launch_dense_prefill(const DenseLaunch& d, hipStream_t s);
+// Its K parts (d.ks; z then holds that many planes, summed in part order by the finish): a call of few rows decodes the
+// matrix once, and a workgroup per 256 columns alone would leave most of the GPU idle, so the tile rows are shared out
+// until the launch has two workgroups a compute unit. Each part keeps an even number of K = 32 steps, at least eight.
+inline uint32_t dense_prefill_kparts(uint32_t rows, uint32_t in, uint32_t out) {
+    const uint32_t item_rows = rows <= 64u ? 64u : 128u, items = (rows + item_rows - 1u) / item_rows;
+    const uint32_t nblk = (out + 255u) / 256u, steps = in / 32u;
+    uint32_t k = 1;
+    while (items * nblk * k < 512u && k < 16u && steps % (4u * k) == 0u && steps / (2u * k) >= 8u) k *= 2u;
+    return k;
+}
 
 // The W_hat form's own stages: the prepare in natural order (plain f16 [rows][in], what a plain GEMM multiplies), and the
 // finish of an f16 z [rows][out].

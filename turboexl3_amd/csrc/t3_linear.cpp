@@ -79,15 +79,15 @@ void carve_dense(DenseCall* call, void* workspace) {
     call->workspace = c.used;
 }
 
-// Above 32 rows: xq plain f16 [rows][in], xs f32 [rows][in / 128], z one f32 plane [rows][out].
+// Above 32 rows: xq plain f16 [rows][in], xs f32 [rows][in / 128], z f32 [K parts][rows][out].
 void carve_dense_prefill(DenseCall* call, void* workspace) {
     DenseLaunch& l = call->launch;
-    l.ks = 1;
+    l.ks = dense_prefill_kparts(l.rows, l.in, l.out);
     Carver c(workspace);
     l.arrive = c.take<uint32_t>(kCounterBytes);
     l.xq = c.take<uint32_t>(static_cast<size_t>(l.rows) * l.in * 2u);
     l.xs = c.take<float>(static_cast<size_t>(l.rows) * (l.in / 128u) * 4u);
-    l.z = c.take<float>(static_cast<size_t>(l.rows) * l.out * 4u);
+    l.z = c.take<float>(static_cast<size_t>(l.ks) * l.rows * l.out * 4u);
     call->workspace = c.used;
 }
 

@@ -33,6 +33,9 @@ struct PfGemm {
     const uint32_t* items;   // {expert, first position, rows, 0} an item; null: dense, item i = rows i RB 16 ...
     const uint32_t* n_items; // the route's item count (device)
     uint32_t in, out, n, wbits, positions, experts, nblk;  // nblk: workgroup columns (256 output columns each)
+    uint32_t spread;  // dies one item's column blocks go round: 1 with eight items or more a launch, up to 8 with one
+    uint32_t kparts;  // K parts (grid z): part k multiplies its share of the tile rows into plane k of z
+    uint32_t plane;   // elements between z's planes
 };
 
 // The weight a GEMM feeds the matrix core as one f16: exact, or MUL1's h = 1024 + t when its map is deferred.
@@ -87,9 +90,10 @@ __device__ __forceinline__ void wait_loads() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-// Grid (8 * nblk * ceil(max_items / 8), projections), 256 threads. Consecutive workgroup ids go round the eight dies,
-// so the workgroups that share an item's activations (its nblk column blocks) are given ids 8 apart: one die's L2
-// serves them all.
+// Grid (8 * ceil(nblk / spread) * ceil(max_items / (8 / spread)), projections, kparts), 256 threads. Consecutive
+// workgroup ids go round the eight dies, so the workgroups that share an item's activations (its nblk column blocks)
+// are given ids 8 apart: one die's L2 serves them all. With fewer than eight items that would leave dies idle (one item:
+// seven of eight), so an item's column blocks then go round `spread` dies.
 //
 // Shapes: RB 16-row blocks an item, four adjacent tiles a wave, 256 columns a workgroup. RB 4: 64 rows. RB 8: 128 rows:
 // a decoded weight feeds twice the MFMAs, and an expert with 65-128 rows stays one item (a second, short item would
@@ -113,8 +117,10 @@ __global__ void __launch_bounds__(256) pf_gemm(const PfGemm a) {
     __shared__ __attribute__((aligned(16))) unsigned char smem[D * kAStep + 4u * D * kPfWaveStep];
     static_assert(sizeof(smem) <= 65536u, "the LDS addresses of the loads are 16 bits");
 
-    const uint32_t id = blockIdx.x, proj = blockIdx.y;
-    const uint32_t j = id >> 3, blk = j % a.nblk, item_i = (j / a.nblk) * 8u + (id & 7u);
+    const uint32_t id = blockIdx.x, proj = blockIdx.y, kpart = blockIdx.z;
+    const uint32_t die = id & 7u, j = id >> 3, nbs = (a.nblk + a.spread - 1u) / a.spread;
+    const uint32_t blk = (j % nbs) * a.spread + die % a.spread, item_i = (j / nbs) * (8u / a.spread) + die / a.spread;
+    if (blk >= a.nblk) return;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
     uint32_t e = 0, first, count;
     if (a.items) {
@@ -155,13 +161,17 @@ __global__ void __launch_bounds__(256) pf_gemm(const PfGemm a) {
         const uint32_t row = (4u * i + wq) * 16u + (lane >> 2), piece = (lane & 3u) ^ ((row >> 1) & 3u);
         a_voff[i] = row < count ? ((first + row) * a.in + piece * 8u) * 2u : 0x80000000u;
     }
+    // this part's steps: the host gives every part an even number of them (in is a multiple of 128)
+    const uint32_t steps = (in_tiles >> 1) / a.kparts, step0 = kpart * steps;
+    float* z = a.z[proj] + static_cast<size_t>(kpart) * a.plane;
     auto issue = [&](uint32_t step, uint32_t slot) {
 #pragma unroll
         for (uint32_t i = 0; i < kALoads; ++i)
-            load_to_lds(xdesc, a_lds + slot * kAStep + (4u * i + wq) * 1024u, a_voff[i], step * 64u);
+            load_to_lds(xdesc, a_lds + slot * kAStep + (4u * i + wq) * 1024u, a_voff[i], (step0 + step) * 64u);
 #pragma unroll
         for (uint32_t r = 0; r < 2u; ++r)
-            load_to_lds(wdesc, w_lds + slot * kPfWaveStep + r * (kPfTiles * kPfSlot), w_voff, (2u * step + r) * wstep);
+            load_to_lds(wdesc, w_lds + slot * kPfWaveStep + r * (kPfTiles * kPfSlot), w_voff,
+                        (2u * (step0 + step) + r) * wstep);
     };
 
     const QuadPlan<WIDE> plan = quad_plan<WIDE>(a.n, lane);
@@ -185,8 +195,6 @@ __global__ void __launch_bounds__(256) pf_gemm(const PfGemm a) {
     // the B fragment of block mb: row 16 mb + lane % 16, K slots 8 (lane / 16) ..: its swizzled piece
     const uint32_t b_at = (lane & 15u) * 64u + (((lane >> 4) ^ ((lane >> 1) & 3u)) * 16u);
 
-    const uint32_t steps = in_tiles >> 1;  // a multiple of 4: in is a multiple of 128
-    float* z = a.z[proj];
 
     // The K loop and the stores for an item of LB live 16-row blocks: no branch inside the loop.
     auto run = [&]<int LB>() {
@@ -537,11 +545,12 @@ __global__ void __launch_bounds__(256) pf_dense_prep(const void* x, const uint16
     if (xs && q == 0u) xs[static_cast<size_t>(row) * nb + b] = sum;
 }
 
-// the dense finish of one plane: z f32 [rows][out] with xs [rows][in / 128] for MUL1's deferred map, or (HALF) z
-// already rounded to f16 (format.innerGemv's rounding point) by a plain GEMM
+// the dense finish: z f32 [ks][rows][out], the planes summed in part order, with xs [rows][in / 128] for MUL1's deferred
+// map; or (HALF) one plane already rounded to f16 (format.innerGemv's rounding point) by a plain GEMM
 template <int DT, bool HALF>
 __global__ void __launch_bounds__(256) pf_dense_finish(const void* z, const float* xs, const uint16_t* svh, void* y,
-                                                       uint32_t out, uint32_t rows, uint32_t inblk, int defer) {
+                                                       uint32_t out, uint32_t rows, uint32_t inblk, int defer,
+                                                       uint32_t ks) {
     const uint32_t nb = out / 128u, groups = (nb + kPfUnit - 1u) / kPfUnit;
     const uint32_t u0 = wave_unit(), row = u0 / groups, lane = threadIdx.x & 63u, q = lane & 15u;
     if (row >= rows) return;
@@ -551,8 +560,18 @@ __global__ void __launch_bounds__(256) pf_dense_finish(const void* z, const floa
     const Row16 g16 = row16(lane);
     const size_t at = static_cast<size_t>(row) * out + i;
     float v[8], sv[8];
-    if constexpr (HALF) load8_half(static_cast<const uint16_t*>(z), at, v);
-    else load8_f32(static_cast<const float*>(z), at, v);
+    if constexpr (HALF) {
+        load8_half(static_cast<const uint16_t*>(z), at, v);
+    } else {
+        load8_f32(static_cast<const float*>(z), at, v);
+        const size_t plane = static_cast<size_t>(rows) * out;
+        for (uint32_t k = 1; k < ks; ++k) {
+            float part[8];
+            load8_f32(static_cast<const float*>(z) + k * plane, at, part);
+#pragma unroll
+            for (uint32_t r = 0; r < 8u; ++r) v[r] += part[r];
+        }
+    }
     load8_half(svh, i, sv);
     if (!HALF && defer) {
         float xsum = 0.0f;
@@ -583,9 +602,10 @@ hipError_t launch_pf_dense_finish(const DenseLaunch& d, const void* z, hipStream
     const dim3 grid = unit_grid(d.rows, d.out), block(256);
     const uint32_t inblk = d.in / 128u;
     const int defer = d.codebook == kMul1Defer ? 1 : 0;
-    if (d.dtype == kF32) hipLaunchKernelGGL((pf_dense_finish<kF32, HALF>), grid, block, 0, s, z, d.xs, d.svh, d.y, d.out, d.rows, inblk, defer);
-    else if (d.dtype == kF16) hipLaunchKernelGGL((pf_dense_finish<kF16, HALF>), grid, block, 0, s, z, d.xs, d.svh, d.y, d.out, d.rows, inblk, defer);
-    else hipLaunchKernelGGL((pf_dense_finish<kBf16, HALF>), grid, block, 0, s, z, d.xs, d.svh, d.y, d.out, d.rows, inblk, defer);
+    const uint32_t ks = HALF ? 1u : d.ks;
+    if (d.dtype == kF32) hipLaunchKernelGGL((pf_dense_finish<kF32, HALF>), grid, block, 0, s, z, d.xs, d.svh, d.y, d.out, d.rows, inblk, defer, ks);
+    else if (d.dtype == kF16) hipLaunchKernelGGL((pf_dense_finish<kF16, HALF>), grid, block, 0, s, z, d.xs, d.svh, d.y, d.out, d.rows, inblk, defer, ks);
+    else hipLaunchKernelGGL((pf_dense_finish<kBf16, HALF>), grid, block, 0, s, z, d.xs, d.svh, d.y, d.out, d.rows, inblk, defer, ks);
     return hipGetLastError();
 }
 
@@ -598,7 +618,11 @@ inline uint32_t gemm_nblk(uint32_t out, uint32_t item_rows) {
 template <int CB, bool WIDE>
 hipError_t launch_gemm_rb(PfGemm g, uint32_t max_items, uint32_t nproj, uint32_t item_rows, hipStream_t s) {
     g.nblk = gemm_nblk(g.out, item_rows);
-    const dim3 grid(8u * g.nblk * ((max_items + 7u) / 8u), nproj), block(256);
+    g.spread = 8u;
+    while (g.spread > 1u && 8u / g.spread < max_items) g.spread >>= 1;  // 8 / spread items share the dies
+    if (g.kparts == 0u) g.kparts = 1u;
+    const uint32_t nbs = (g.nblk + g.spread - 1u) / g.spread, group = 8u / g.spread;
+    const dim3 grid(8u * nbs * ((max_items + group - 1u) / group), nproj, g.kparts), block(256);
     if (item_rows == 32u) hipLaunchKernelGGL((pf_gemm<CB, WIDE, 2>), grid, block, 0, s, g);
     else if (item_rows == 128u) hipLaunchKernelGGL((pf_gemm<CB, WIDE, 8>), grid, block, 0, s, g);
     else hipLaunchKernelGGL((pf_gemm<CB, WIDE, 4>), grid, block, 0, s, g);
@@ -701,6 +725,8 @@ hipError_t launch_dense_prefill(const DenseLaunch& d, hipStream_t s) {
     g.wbits = d.wbits;
     g.positions = d.rows;
     g.experts = 1u;
+    g.kparts = d.ks;
+    g.plane = d.rows * d.out;
     const uint32_t item_rows = d.rows <= 64u ? 64u : 128u;
     if ((e = launch_gemm(g, d.codebook, (d.rows + item_rows - 1u) / item_rows, 1u, item_rows, s)) != hipSuccess) return e;
     return launch_pf_dense_finish<false>(d, d.z, s);
