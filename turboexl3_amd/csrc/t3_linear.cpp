@@ -137,14 +137,17 @@ int32_t run_chain(const DenseCall& call, hipStream_t s, uint32_t stages) {
     return T3_OK;
 }
 
-// The served form (src/core/dense.zig:1229-1242 takes DEC-ONE up to 4 rows the same way). Up to 4 rows: one launch
-// where a wave's K part is whole 128-blocks and small enough to prepare in LDS, else the prepare launch and the
-// arriving GEMV. More rows: the chain (measured: with 16 and 32 rows the planes' coherent traffic costs the arriving
-// form more than the finish launch it saves).
+// The served form (src/core/dense.zig:1229-1242 takes DEC-ONE at its fewest rows the same way). One row (two at up to
+// four bits a weight, where a wave takes eight tiles a step): one launch where a wave's K part is whole 128-blocks and small enough to prepare
+// in LDS, else the prepare launch and the arriving GEMV. More rows: the chain. Measured at 4096 x 12288: the one launch
+// takes 14.8-17.1 us at one row against the chain's 16.7-18.0, but every further row adds 1-2 us to it (each workgroup
+// prepares every row and the last arriver finishes them one after the other) and nothing to the chain, and with 16 and
+// 32 rows the planes' coherent traffic costs the arriving form more than the finish launch it saves. The forms give the
+// same bytes.
 int32_t run_fused(const DenseCall& call, hipStream_t s) {
     const DenseLaunch& l = call.launch;
     const uint32_t per = (l.in / 16u) / (4u * l.ks);
-    if (l.rows > 4u) return run_chain(call, s, 7u);
+    if (l.rows > (l.bt == 8u ? 2u : 1u)) return run_chain(call, s, 7u);
     if (per % 8u == 0u && per <= 16u) return hip_status(launch_dense_gemv(l, kFuseOne, s));
     if (const int32_t st = hip_status(launch_dense_prep(l, s)); st != T3_OK) return st;
     return hip_status(launch_dense_gemv(l, kFuseArrive, s));
