@@ -225,6 +225,19 @@ int32_t t3_moe_shared_expert(t3_stream stream, const t3_array* x, const t3_bank*
 int32_t t3_moe_fused_shared(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
                             const t3_array* scores, t3_decode dec, const t3_bank* shared_bank, const t3_array* sigtab,
                             const t3_array* logit, t3_array* y, void* workspace, size_t workspace_bytes);
+/* `t3_moe_fused_shared` with the routing inside (src/models/qwen38/api.zig:386-395 `moeFusedSharedRouted`): logits
+ * [B, S, E] in x's dtype is the router gemv's output and k the experts a token (1..31, E <= 2048); one more launch
+ * in front picks each row's top-k by logit (ties to the lowest id) and their softmax weights renormalised over the k,
+ * with the statements of the host's router kernel as the reference restates it (src/models/qwen38/kernels/shared/
+ * router_softmax_1..6.metal): the softmax over all experts in f32, each weight rounded to the dtype, their total added
+ * up in ascending slot order in the dtype, each weight divided by it. The slots and weights live in the workspace's
+ * tail. The reference's `gate_vec` form (the shared gate's logit computed in the launch in MLX's gemv order) is not
+ * carried: pass `logit`. */
+int32_t t3_moe_fused_shared_routed_workspace_bytes(const t3_array* x, const t3_bank* bank, const t3_array* logits,
+                                                   int64_t k, const t3_bank* shared_bank, size_t* bytes);
+int32_t t3_moe_fused_shared_routed(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* logits,
+                                   int64_t k, t3_decode dec, const t3_bank* shared_bank, const t3_array* sigtab,
+                                   const t3_array* logit, t3_array* y, void* workspace, size_t workspace_bytes);
 /* shared_bank: NULL, or the bank `t3_moe_shared_expert` will take (its slots need scratch too). */
 int32_t t3_moe_workspace_bytes(const t3_array* x, const t3_bank* bank, const t3_array* inds,
                                const t3_bank* shared_bank, size_t* bytes);

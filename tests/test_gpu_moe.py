@@ -351,3 +351,56 @@ def test_fused_gated_shared_expert(oracle, t3, codebook, n, dtype):
                             torch.from_numpy(w5).cuda().reshape(1, 5, topk), dec, dshared, table.cuda(),
                             torch.zeros(5, dtype=dtype, device="cuda"))
     assert err.value.name == "Exl3EngineNotImplemented"
+
+
+def router_reference(logits_f32, k, dtype):
+    """The host's softmax router as src/models/qwen38/kernels/shared/router_softmax_*.metal restates it: top-k by logit
+    (ties to the lowest id), weights = dtype(softmax over all experts), renormalised by their total added up in slot
+    order in the dtype."""
+    rows = logits_f32.shape[0]
+    inds = np.zeros((rows, k), dtype=np.int32)
+    scores = np.zeros((rows, k), dtype=np.float32)
+    for r in range(rows):
+        row = logits_f32[r]
+        pick = np.argsort(-row, kind="stable")[:k]
+        smax = row.max()
+        snorm = np.float32(1.0) / np.exp(row - smax, dtype=np.float32).sum(dtype=np.float32)
+        w = _to(dtype, np.exp(row[pick] - smax, dtype=np.float32) * snorm)
+        tot = np.float32(0.0)
+        for j in range(k):
+            tot = _to(dtype, np.array([w[j] + tot]))[0]
+        inds[r] = pick
+        scores[r] = _to(dtype, w / tot)
+    return inds, scores
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fused_gated_shared_expert_with_the_router_inside(oracle, t3, dtype):
+    # src/models/qwen38/api.zig:386-395: the same call with the top-k and the renormalised softmax weights made from the
+    # router's logits by one launch in front
+    rng = np.random.default_rng(0x5A7)
+    hidden, inter, experts, k, n = 512, 256, 70, 6, 64
+    bank, shared = oracle.synth_bank(rng, experts, hidden, inter, n), oracle.synth_bank(rng, 1, hidden, inter, n)
+    dbank, dshared = dev_bank(t3, bank), dev_bank(t3, shared)
+    dec = t3.Decode(MCG, 16)
+    rows = 3
+    x_dev, _ = make_x(rng, rows, hidden, dtype)
+    logits = torch.from_numpy(rng.standard_normal((rows, experts)).astype(np.float32)).to(dtype)
+    logits[1, 5] = logits[1, 40] = 9.0  # a tie at the top: the lowest id first
+    logit = torch.from_numpy(rng.standard_normal(rows).astype(np.float32)).to(dtype)
+    table = sigmoid_table(dtype).cuda()
+    y, inds, scores = t3.moe_fused_shared_routed(x_dev.reshape(1, rows, hidden), dbank, logits.cuda().reshape(1, rows, experts),
+                                                 k, dec, dshared, table, logit.cuda(), return_routing=True)
+    want_i, want_s = router_reference(logits.to(torch.float32).numpy(), k, dtype)
+    assert np.array_equal(inds.cpu().numpy(), want_i), "the router picked other experts"
+    assert want_i[1, 0] == 5 and want_i[1, 1] == 40
+    step = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
+    assert np.abs(to_f32(scores) - want_s).max() <= step * want_s.max() * 2, "weights further than a step of the dtype"
+    # and the call is the unrouted one on the router's own slots and weights, byte for byte
+    same = t3.moe_fused_shared(x_dev.reshape(1, rows, hidden), dbank, inds.reshape(1, rows, k), scores.reshape(1, rows, k),
+                               dec, dshared, table, logit.cuda())
+    assert bytes_of(y) == bytes_of(same)
+    with pytest.raises(t3.T3Error) as err:  # more experts a token than the router carries
+        t3.moe_fused_shared_routed(x_dev.reshape(1, rows, hidden), dbank, logits.cuda().reshape(1, rows, experts), 32, dec,
+                                   dshared, table, logit.cuda())
+    assert err.value.name == "Exl3EngineNotImplemented"

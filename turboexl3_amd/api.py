@@ -304,6 +304,33 @@ def moe_fused_shared(x, bank: Bank, inds, scores, dec: Decode, shared_bank: Bank
     return y
 
 
+def moe_fused_shared_routed(x, bank: Bank, logits, k: int, dec: Decode, shared_bank: Bank, sigtab, logit, stream=None,
+                            return_routing: bool = False):
+    """qwen38's moeFusedSharedRouted: `moe_fused_shared` with the top-k and the renormalised softmax weights computed
+    from the router's logits [B, S, E] by one launch in front. return_routing: also the slots and weights it made."""
+    L = _lib.lib()
+    ax, al = _arr(x), _arr(logits)
+    cb, _keep = _cbank(bank)
+    sb, _keep2 = _cbank(shared_bank)
+    need = C.c_size_t(0)
+    _check(L.t3_moe_fused_shared_routed_workspace_bytes(C.byref(ax), C.byref(cb), C.byref(al), int(k), C.byref(sb),
+                                                        C.byref(need)))
+    ws = torch.zeros(max(need.value, 256), dtype=torch.uint8, device=x.device)
+    y = torch.empty_like(x)
+    ay, at, ag = _arr(y), _arr(sigtab), _arr(logit)
+    _check(L.t3_moe_fused_shared_routed(_stream_ptr(stream), C.byref(ax), C.byref(cb), C.byref(al), int(k), dec.c(),
+                                        C.byref(sb), C.byref(at), C.byref(ag), C.byref(ay), ws.data_ptr(), ws.numel()))
+    if not return_routing:
+        return y
+    rows = x.shape[0] * x.shape[1]
+    slots = rows * k
+    pad = lambda b: (b + 255) & ~255
+    tail = need.value - pad(slots * 4) - pad(slots * 2)
+    inds = ws[tail:tail + slots * 4].view(torch.int32).reshape(rows, k).clone()
+    scores = ws[tail + pad(slots * 4):tail + pad(slots * 4) + slots * 2].view(x.dtype).reshape(rows, k).clone()
+    return y, inds, scores
+
+
 # ---- device self-tests -------------------------------------------------------------------------------------
 
 def test_codebooks(device="cuda"):

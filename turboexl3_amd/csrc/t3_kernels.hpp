@@ -92,6 +92,9 @@ struct MoeLaunch {
 // or two (gate|up + mid, down + combine: the last workgroup to arrive at a block runs the next stage). The same bytes.
 enum MoeForm : int { kMoeFiveLaunches = 0, kMoeFourLaunches = 1, kMoeTwoLaunches = 2 };
 hipError_t launch_moe_decode(const MoeLaunch& a, int form, hipStream_t s);
+// a row's top-k experts by logit (ties to the lowest id) and their renormalised softmax weights in the logits' dtype
+hipError_t launch_route_softmax(const void* logits, int32_t* inds, void* scores, uint32_t rows, uint32_t experts, uint32_t k,
+                                int dtype, hipStream_t s);
 
 // The same call above the decode rows: route, prepare, gate|up GEMM, mid, down GEMM, combine. xg, xu, hd hold plain f16
 // here (pair-quad order), zg, zu, zd one plane each, all by sorted position.

@@ -280,24 +280,69 @@ int32_t t3_moe_shared_expert(t3_stream stream, const t3_array* x, const t3_bank*
     return t3::run_moe(stream, x, bank, inds, scores, shared_bank, nullptr, dec, limit, y, workspace, workspace_bytes);
 }
 
-int32_t t3_moe_fused_shared(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
-                            const t3_array* scores, t3_decode dec, const t3_bank* shared_bank, const t3_array* sigtab,
-                            const t3_array* logit, t3_array* y, void* workspace, size_t workspace_bytes) {
-    if (!shared_bank || !scores || !y || !t3::array_ok(sigtab) || !t3::array_ok(logit)) return T3_BadArgs;
+namespace {
+// `moeFusedShared`; with `logits` [.., rows, E] and k, `moeFusedSharedRouted`: the slots and weights come from the
+// router kernel, into the workspace's tail. bytes non-null: only the workspace size is wanted.
+int32_t fused_shared(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
+                     const t3_array* scores, const t3_array* logits, int64_t k, t3_decode dec, const t3_bank* shared_bank,
+                     const t3_array* sigtab, const t3_array* logit, t3_array* y, void* workspace, size_t workspace_bytes,
+                     size_t* bytes) {
+    if (!shared_bank || !t3::array_ok(x)) return T3_BadArgs;
+    t3_array routed_inds{}, routed_scores{};
+    if (logits) {
+        // src/models/qwen38/api.zig:396-407
+        if (!t3::array_ok(logits)) return T3_BadArgs;
+        if (x->ndim != 3 || logits->ndim != 3 || x->shape[0] != logits->shape[0] || x->shape[1] != logits->shape[1])
+            return T3_BadExl3Shape;
+        if (k <= 0 || k > 31 || logits->dtype != x->dtype || logits->shape[2] > 2048 || logits->shape[2] < k)
+            return T3_Exl3EngineNotImplemented;
+        routed_inds = *x;  // the shape [B, S, k]; the data pointer only has to be one until the workspace is carved
+        routed_inds.dtype = T3_I32;
+        routed_inds.shape[2] = k;
+        routed_scores = routed_inds;
+        routed_scores.dtype = x->dtype;
+        inds = &routed_inds;
+        scores = &routed_scores;
+    }
+    if (!scores) return T3_BadArgs;
     t3::MoeCall call;
-    if (const int32_t st = t3::check_moe(x, bank, inds, scores, shared_bank, nullptr, dec, 0, y, &call, 0); st != T3_OK)
+    if (const int32_t st = t3::check_moe(x, bank, inds, scores, shared_bank, nullptr, dec, 0, bytes ? nullptr : y, &call, 0);
+        st != T3_OK)
         return st;
-    // what the fused launches do not carry stays with the caller's chain (src/models/qwen38/api.zig:312-322)
     t3::MoeLaunch& l = call.launch;
+    if (logits && logits->shape[2] != static_cast<int64_t>(l.bank.experts)) return T3_Exl3EngineNotImplemented;
+    // what the fused launches do not carry stays with the caller's chain (src/models/qwen38/api.zig:312-322)
+    if (call.rows > T3_SHARED_ROWS_MAX || l.shared_slots != 1u || (x->dtype != T3_F16 && x->dtype != T3_BF16))
+        return T3_Exl3EngineNotImplemented;
+    t3::carve_moe(&call, workspace);
+    const size_t slots = static_cast<size_t>(call.rows) * l.topk;
+    const size_t inds_at = call.workspace, scores_at = inds_at + ((slots * 4u + 255u) & ~static_cast<size_t>(255u));
+    const size_t total = logits ? scores_at + ((slots * 2u + 255u) & ~static_cast<size_t>(255u)) : call.workspace;
+    if (bytes) {
+        *bytes = total;
+        return T3_OK;
+    }
+    if (!y || !t3::array_ok(sigtab) || !t3::array_ok(logit)) return T3_BadArgs;
     int64_t tab = 1, lg = 1;
     for (int i = 0; i < sigtab->ndim; ++i) tab *= sigtab->shape[i];
     for (int i = 0; i < logit->ndim; ++i) lg *= logit->shape[i];
-    if (call.rows > T3_SHARED_ROWS_MAX || l.shared_slots != 1u || (x->dtype != T3_F16 && x->dtype != T3_BF16) ||
-        sigtab->dtype != x->dtype || tab != 65536 || logit->dtype != x->dtype || lg != static_cast<int64_t>(call.rows))
+    if (sigtab->dtype != x->dtype || tab != 65536 || logit->dtype != x->dtype || lg != static_cast<int64_t>(call.rows))
         return T3_Exl3EngineNotImplemented;
     if (!t3::workspace_ok(workspace)) return T3_BadArgs;
-    t3::carve_moe(&call, workspace);
-    if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
+    if (workspace_bytes < total) return T3_WorkspaceTooSmall;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (logits) {
+        int32_t* d_inds = reinterpret_cast<int32_t*>(static_cast<unsigned char*>(workspace) + inds_at);
+        void* d_scores = static_cast<unsigned char*>(workspace) + scores_at;
+        if (const int32_t st = t3::hip_status(t3::launch_route_softmax(logits->data, d_inds, d_scores,
+                                                                       static_cast<uint32_t>(call.rows), l.bank.experts,
+                                                                       l.topk, x->dtype, s));
+            st != T3_OK)
+            return st;
+        l.slots = d_inds;
+        l.scores = d_scores;
+        l.score_dt = x->dtype;
+    }
     l.sigtab = sigtab->data;
     l.slogit = logit->data;
     const size_t widest = (l.hidden > l.inter ? l.hidden : l.inter) / 128u;
@@ -305,7 +350,32 @@ int32_t t3_moe_fused_shared(t3_stream stream, const t3_array* x, const t3_bank* 
     const int form = t3::config().decode_form == 3 ? t3::kMoeFiveLaunches
                      : t3::config().decode_form == 4 || counters * 4u > t3::kCounterBytes ? t3::kMoeFourLaunches
                                                                                           : t3::kMoeTwoLaunches;
-    return t3::hip_status(t3::launch_moe_decode(l, form, static_cast<hipStream_t>(stream)));
+    return t3::hip_status(t3::launch_moe_decode(l, form, s));
+}
+}  // namespace
+
+int32_t t3_moe_fused_shared(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
+                            const t3_array* scores, t3_decode dec, const t3_bank* shared_bank, const t3_array* sigtab,
+                            const t3_array* logit, t3_array* y, void* workspace, size_t workspace_bytes) {
+    if (!inds || !scores || !y) return T3_BadArgs;
+    return fused_shared(stream, x, bank, inds, scores, nullptr, 0, dec, shared_bank, sigtab, logit, y, workspace,
+                        workspace_bytes, nullptr);
+}
+
+int32_t t3_moe_fused_shared_routed_workspace_bytes(const t3_array* x, const t3_bank* bank, const t3_array* logits,
+                                                   int64_t k, const t3_bank* shared_bank, size_t* bytes) {
+    if (!bytes || !logits) return T3_BadArgs;
+    const t3_decode dec = {0, 16};
+    return fused_shared(nullptr, x, bank, nullptr, nullptr, logits, k, dec, shared_bank, nullptr, nullptr, nullptr, nullptr,
+                        0, bytes);
+}
+
+int32_t t3_moe_fused_shared_routed(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* logits,
+                                   int64_t k, t3_decode dec, const t3_bank* shared_bank, const t3_array* sigtab,
+                                   const t3_array* logit, t3_array* y, void* workspace, size_t workspace_bytes) {
+    if (!logits || !y) return T3_BadArgs;
+    return fused_shared(stream, x, bank, nullptr, nullptr, logits, k, dec, shared_bank, sigtab, logit, y, workspace,
+                        workspace_bytes, nullptr);
 }
 
 }  // extern "C"

@@ -285,4 +285,96 @@ hipError_t launch_moe_decode(const MoeLaunch& a, int form, hipStream_t s) {
     return hipGetLastError();
 }
 
+
+namespace {
+
+// The softmax router of the gated shared expert's routed form (turboexl3 src/models/qwen38/kernels/shared/
+// router_softmax_1..6.metal, a copy of the host's "mlxserve_moe_router_softmax"): a row's top-k experts by logit, ties
+// to the lowest id, and their softmax weights renormalised over the k. The statements' order is the host kernel's: the
+// softmax over all experts in f32; each selected weight rounded to the dtype; their total added up in ascending slot
+// order in the dtype, rounding after every add; each weight divided by it and rounded. (The f32 sum over the experts is
+// a wave reduction whose order no source fixes.) One wave a row: lane L holds experts L + 64 i, i < 32.
+// Grid (rows), 64 threads.
+template <int DT>
+__global__ void __launch_bounds__(64) route_softmax(const void* logits, int32_t* inds, void* scores, uint32_t experts,
+                                                     uint32_t k) {
+    const uint32_t row = blockIdx.x, lane = threadIdx.x;
+    const size_t base = static_cast<size_t>(row) * experts;
+    constexpr float kNone = -__builtin_inff();
+    float mine[32];
+#pragma unroll
+    for (uint32_t i = 0; i < 32u; ++i) {
+        const uint32_t e = lane + 64u * i;
+        mine[i] = e < experts ? load_act<DT>(logits, base + e) : kNone;
+    }
+    auto wave_max = [](float v) {
+#pragma unroll
+        for (int m = 32; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
+        return v;
+    };
+    float lane_max = kNone;
+#pragma unroll
+    for (uint32_t i = 0; i < 32u; ++i) lane_max = fmaxf(lane_max, mine[i]);
+    const float smax = wave_max(lane_max);
+    float sum = 0.0f;
+#pragma unroll
+    for (uint32_t i = 0; i < 32u; ++i) sum += lane + 64u * i < experts ? __expf(mine[i] - smax) : 0.0f;
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) sum += __shfl_xor(sum, m, 64);
+    const float snorm = 1.0f / sum;
+
+    auto round_dt = [](float v) {
+        if constexpr (DT == kF16) return round_half(v);
+        else if constexpr (DT == kBf16) return bf16_value(bf16_bits(v));
+        else return v;
+    };
+    // k rounds of "max, then mask"
+    uint32_t my_sel = 0;   // lane j < k keeps round j's pick
+    float my_w = 0.0f;
+    for (uint32_t r = 0; r < k; ++r) {
+        float best = kNone;
+        uint32_t slot = 0xFFFFFFFFu;
+#pragma unroll
+        for (uint32_t i = 0; i < 32u; ++i)
+            if (mine[i] > best) {
+                best = mine[i];
+                slot = i;
+            }
+        const float gmax = wave_max(best);
+        uint32_t cand = (best == gmax && slot != 0xFFFFFFFFu) ? lane + 64u * slot : 0xFFFFFFFFu;
+#pragma unroll
+        for (int m = 32; m > 0; m >>= 1) {
+            const uint32_t o = static_cast<uint32_t>(__shfl_xor(static_cast<int>(cand), m, 64));
+            cand = o < cand ? o : cand;
+        }
+        const uint32_t pick = cand < experts - 1u ? cand : experts - 1u;
+        if ((pick & 63u) == lane) {
+#pragma unroll
+            for (uint32_t i = 0; i < 32u; ++i)
+                if (i == pick >> 6) mine[i] = kNone;
+        }
+        if (lane == r) {
+            my_sel = pick;
+            my_w = round_dt(__expf(load_act<DT>(logits, base + pick) - smax) * snorm);
+        }
+    }
+    float tot = 0.0f;
+    for (uint32_t j = 0; j < k; ++j)
+        tot = round_dt(__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_w), static_cast<int>(j))) + tot);
+    if (lane < k) {
+        inds[static_cast<size_t>(row) * k + lane] = static_cast<int32_t>(my_sel);
+        store_act<DT>(scores, static_cast<size_t>(row) * k + lane, my_w / round_dt(tot));
+    }
+}
+
+}  // namespace
+
+hipError_t launch_route_softmax(const void* logits, int32_t* inds, void* scores, uint32_t rows, uint32_t experts, uint32_t k,
+                                int dtype, hipStream_t s) {
+    if (dtype == kF16) hipLaunchKernelGGL(route_softmax<kF16>, dim3(rows), dim3(64), 0, s, logits, inds, scores, experts, k);
+    else if (dtype == kBf16) hipLaunchKernelGGL(route_softmax<kBf16>, dim3(rows), dim3(64), 0, s, logits, inds, scores, experts, k);
+    else hipLaunchKernelGGL(route_softmax<kF32>, dim3(rows), dim3(64), 0, s, logits, inds, scores, experts, k);
+    return hipGetLastError();
+}
+
 }  // namespace t3
