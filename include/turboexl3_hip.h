@@ -238,6 +238,14 @@ int32_t t3_moe_fused_shared_routed_workspace_bytes(const t3_array* x, const t3_b
 int32_t t3_moe_fused_shared_routed(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* logits,
                                    int64_t k, t3_decode dec, const t3_bank* shared_bank, const t3_array* sigtab,
                                    const t3_array* logit, t3_array* y, void* workspace, size_t workspace_bytes);
+/* The routed experts under GLM's rounding profile (src/hip/plan.zig:219-247,396-403 `Profile.glm`;
+ * src/kernels/hip/decode/decode.hip:8-13): x BF16 times suh in f32 (no f16 rounding of x), the inner products stay f32,
+ * gate and up round to bf16 and are limited (limit 0: not), the SiLU rounds to bf16, the product rounds to bf16; y F32
+ * [B, S, K, D]: each routed slot's own down finish, no score (the host combines a row's slots and its shared expert). A
+ * slot whose id is outside [0, E) is skipped and its output left as it is. Any row count: the decode chain's five
+ * launches up to 16 rows, the prefill chain above. Workspace: t3_moe_workspace_bytes (shared_bank NULL). */
+int32_t t3_moe_glm(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds, t3_decode dec,
+                   int32_t limit, t3_array* y, void* workspace, size_t workspace_bytes);
 /* shared_bank: NULL, or the bank `t3_moe_shared_expert` will take (its slots need scratch too). */
 int32_t t3_moe_workspace_bytes(const t3_array* x, const t3_bank* bank, const t3_array* inds,
                                const t3_bank* shared_bank, size_t* bytes);

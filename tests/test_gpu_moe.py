@@ -404,3 +404,55 @@ def test_fused_gated_shared_expert_with_the_router_inside(oracle, t3, dtype):
         t3.moe_fused_shared_routed(x_dev.reshape(1, rows, hidden), dbank, logits.cuda().reshape(1, rows, experts), 32, dec,
                                    dshared, table, logit.cuda())
     assert err.value.name == "Exl3EngineNotImplemented"
+
+
+def _bf16_round64(v):
+    return torch.from_numpy(np.asarray(v, dtype=np.float32)).to(torch.bfloat16).to(torch.float64).numpy()
+
+
+def _w_std64(oracle, trellis, suh, svh, in_f, out_f, n, codebook):
+    """diag(suh) H W_hat H diag(svh) in f64 (src/hip_tests.zig:546-554 dequant64)."""
+    import scipy.linalg
+    w = oracle.reconstruct_inner(trellis, in_f, out_f, n, codebook, 0xFFFF).view(np.float16).astype(np.float64).reshape(in_f, out_f)
+    h = scipy.linalg.hadamard(128).astype(np.float64) / np.sqrt(128.0)
+    w = (h @ w.reshape(in_f // 128, 128, out_f)).reshape(in_f, out_f)          # rotate the input side, block by block
+    w = w * suh.view(np.float16).astype(np.float64)[:, None]
+    w = (w.reshape(in_f, out_f // 128, 128) @ h).reshape(in_f, out_f)           # and the output side
+    return w * svh.view(np.float16).astype(np.float64)[None, :]
+
+
+@pytest.mark.parametrize("rows", [1, 4, 8, 40])
+def test_glm_profile_slots_against_float64(oracle, t3, rows):
+    # src/hip_tests.zig:576-671: every routed slot's f32 output within sum |a w| / 64 + 1e-6 of float64 under GLM's
+    # roundings, the slot past the experts (the host's shared expert) left alone; 40 rows take the prefill chain
+    rng = np.random.default_rng(0x61A)
+    hidden, inter, experts, topk, n, limit = 512, 256, 12, 8, 64, 7.0
+    bank = oracle.synth_bank(rng, experts, hidden, inter, n)
+    dbank = dev_bank(t3, bank)
+    k = topk + 1
+    x_dev, x_f32 = make_x(rng, rows, hidden, torch.bfloat16)
+    slots = np.stack([np.concatenate([rng.permutation(experts)[:topk], [experts]]) for _ in range(rows)]).astype(np.int32)
+    y = t3.moe_glm(x_dev.reshape(1, rows, hidden), dbank, torch.from_numpy(slots).cuda().reshape(1, rows, k),
+                   t3.Decode(MCG, 16), int(limit), fill=float("nan"))
+    got = y.cpu().numpy().reshape(rows, k, hidden).astype(np.float64)
+    assert np.isnan(got[:, topk]).all(), "the slot past the experts was written"
+    worst = 0.0
+    w64 = {}
+    for r in range(rows if rows <= 8 else 6):
+        xr = x_f32[r].astype(np.float64)
+        for j in range(topk):
+            e = int(slots[r, j])
+            if e not in w64:
+                w64[e] = (_w_std64(oracle, bank.gate_t[e], bank.gate_suh[e], bank.gate_svh[e], hidden, inter, n, MCG),
+                          _w_std64(oracle, bank.up_t[e], bank.up_suh[e], bank.up_svh[e], hidden, inter, n, MCG),
+                          _w_std64(oracle, bank.down_t[e], bank.down_suh[e], bank.down_svh[e], inter, hidden, n, MCG))
+            wg, wu, wd = w64[e]
+            gg, uu = _bf16_round64(xr @ wg), _bf16_round64(xr @ wu)
+            gg, uu = np.minimum(gg, limit), np.clip(uu, -limit, limit)
+            act = _bf16_round64(_bf16_round64(gg / (1.0 + np.exp(-gg))) * uu)
+            want = act @ wd
+            tol = np.abs(act[:, None] * wd).sum(axis=0) / 64.0 + 1e-6
+            q = (np.abs(got[r, j] - want) / tol).max()
+            assert q <= 1.0, f"rows {rows} row {r} slot {j}: {q:.3f} of its tolerance"
+            worst = max(worst, q)
+    print(f"GLM profile rows {rows}: worst {worst:.3f} of the float64 tolerance")

@@ -331,6 +331,20 @@ def moe_fused_shared_routed(x, bank: Bank, logits, k: int, dec: Decode, shared_b
     return y, inds, scores
 
 
+def moe_glm(x, bank: Bank, inds, dec: Decode, limit: int = 0, stream=None, fill: float = 0.0) -> torch.Tensor:
+    """The routed experts under GLM's rounding profile: x bf16 [B, S, D] -> f32 [B, S, K, D], a slot's own output each
+    (a skipped slot keeps `fill`)."""
+    L = _lib.lib()
+    ax, ai = _arr(x), _arr(inds)
+    cb, _keep = _cbank(bank)
+    ws = _moe_workspace(L, ax, cb, ai, x.device)
+    y = torch.full((x.shape[0], x.shape[1], inds.shape[2], x.shape[2]), fill, dtype=torch.float32, device=x.device)
+    ay = _arr(y)
+    _check(L.t3_moe_glm(_stream_ptr(stream), C.byref(ax), C.byref(cb), C.byref(ai), dec.c(), int(limit), C.byref(ay),
+                        ws.data_ptr(), ws.numel()))
+    return y
+
+
 # ---- device self-tests -------------------------------------------------------------------------------------
 
 def test_codebooks(device="cuda"):

@@ -60,6 +60,8 @@ struct MoeLaunch {
     // pattern, slogit [rows] in dtype = the shared gate's logit; null: the shared slots are summed at weight 1
     const void* sigtab = nullptr;
     const void* slogit = nullptr;
+    // GLM's rounding profile (src/hip/plan.zig:219-221): x bf16, y f32 [rows][topk][hidden] a slot, no scores
+    int glm = 0;
     void* y = nullptr;
     uint32_t* arrive = nullptr;  // the two-launch form's arrival counters
     uint32_t* xg = nullptr;      // u32 [RKT][hidden]

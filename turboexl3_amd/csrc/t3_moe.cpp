@@ -192,6 +192,16 @@ int32_t admit_prefill(const MoeCall& call) {
     return T3_OK;
 }
 
+// decode_form 3: the five-launch chain; 4: four launches; 9: two launches while a counter a (row-slot, 128-block) fits
+// the workspace's counter area, else four
+int decode_form_of(const MoeLaunch& l) {
+    const size_t widest = (l.hidden > l.inter ? l.hidden : l.inter) / 128u;
+    const size_t counters = static_cast<size_t>(l.rows) * (l.topk + l.shared_slots) * widest;
+    return config().decode_form == 3 ? kMoeFiveLaunches
+           : config().decode_form == 4 || counters * 4u > kCounterBytes ? kMoeFourLaunches
+                                                                         : kMoeTwoLaunches;
+}
+
 int32_t run_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
                 const t3_array* scores, const t3_bank* shared_bank, const t3_array* shared_add, t3_decode dec,
                 int32_t limit, t3_array* y, void* workspace, size_t workspace_bytes, int32_t clamp_at = 0) {
@@ -210,15 +220,7 @@ int32_t run_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const 
     }
     carve_moe(&call, workspace);
     if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
-    // decode_form 3: the five-launch chain; 4: four launches; 9: two launches while a counter a (row-slot, 128-block)
-    // fits the workspace's counter area, else four
-    const MoeLaunch& l = call.launch;
-    const size_t widest = (l.hidden > l.inter ? l.hidden : l.inter) / 128u;
-    const size_t counters = static_cast<size_t>(l.rows) * (l.topk + l.shared_slots) * widest;
-    const int form = config().decode_form == 3 ? kMoeFiveLaunches
-                     : config().decode_form == 4 || counters * 4u > kCounterBytes ? kMoeFourLaunches
-                                                                                   : kMoeTwoLaunches;
-    return hip_status(launch_moe_decode(l, form, static_cast<hipStream_t>(stream)));
+    return hip_status(launch_moe_decode(call.launch, decode_form_of(call.launch), static_cast<hipStream_t>(stream)));
 }
 
 }  // namespace
@@ -278,6 +280,36 @@ int32_t t3_moe_shared_expert(t3_stream stream, const t3_array* x, const t3_bank*
                              t3_array* y, void* workspace, size_t workspace_bytes) {
     if (!shared_bank) return T3_BadArgs;
     return t3::run_moe(stream, x, bank, inds, scores, shared_bank, nullptr, dec, limit, y, workspace, workspace_bytes);
+}
+
+/* GLM's rounding profile of the routed experts (src/hip/plan.zig:219-247 `Profile.glm`): x bf16, each routed slot's own
+ * f32 output, no scores; the slots of a row are the host's to combine. */
+int32_t t3_moe_glm(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds, t3_decode dec,
+                   int32_t limit, t3_array* y, void* workspace, size_t workspace_bytes) {
+    if (!t3::array_ok(y)) return T3_BadArgs;
+    if (limit < 0 || limit > 128) return T3_InvalidExl3Clamp;
+    t3::MoeCall call;
+    if (const int32_t st = t3::check_moe(x, bank, inds, nullptr, nullptr, nullptr, dec, limit, nullptr, &call, 0); st != T3_OK)
+        return st;
+    t3::MoeLaunch& l = call.launch;
+    if (x->dtype != T3_BF16) return T3_BadExl3Shape;  // plan.zig:244
+    if (y->dtype != T3_F32) return T3_BadExl3Dtype;
+    if (y->ndim != 4 || y->shape[0] != x->shape[0] || y->shape[1] != x->shape[1] || y->shape[2] != inds->shape[2] ||
+        y->shape[3] != x->shape[2] || !t3::aligned16(y))
+        return T3_BadExl3Shape;
+    if (!t3::workspace_ok(workspace)) return T3_BadArgs;
+    l.y = y->data;
+    l.glm = 1;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (call.rows > T3_DECODE_ROWS_MAX) {
+        if (const int32_t st = t3::admit_prefill(call); st != T3_OK) return st;
+        t3::carve_moe_prefill(&call, workspace);
+        if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
+        return t3::hip_status(t3::launch_moe_prefill(l, s));
+    }
+    t3::carve_moe(&call, workspace);
+    if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
+    return t3::hip_status(t3::launch_moe_decode(l, t3::kMoeFiveLaunches, s));
 }
 
 namespace {
@@ -345,12 +377,7 @@ int32_t fused_shared(t3_stream stream, const t3_array* x, const t3_bank* bank, c
     }
     l.sigtab = sigtab->data;
     l.slogit = logit->data;
-    const size_t widest = (l.hidden > l.inter ? l.hidden : l.inter) / 128u;
-    const size_t counters = static_cast<size_t>(l.rows) * (l.topk + l.shared_slots) * widest;
-    const int form = t3::config().decode_form == 3 ? t3::kMoeFiveLaunches
-                     : t3::config().decode_form == 4 || counters * 4u > t3::kCounterBytes ? t3::kMoeFourLaunches
-                                                                                          : t3::kMoeTwoLaunches;
-    return t3::hip_status(t3::launch_moe_decode(l, form, s));
+    return t3::hip_status(t3::launch_moe_decode(l, t3::decode_form_of(l), s));
 }
 }  // namespace
 

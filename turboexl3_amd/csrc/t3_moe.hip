@@ -23,8 +23,9 @@ namespace t3 {
 namespace {
 
 // Grid (hidden / 128, RKT), 64 threads: the five-launch form's prepare.
+template <int PROF>
 __global__ void __launch_bounds__(64) moe_prep(const MoeLaunch a) {
-    routed_prep_block<false>(a, blockIdx.y, blockIdx.y, blockIdx.x, threadIdx.x);
+    routed_prep_block<false, PROF>(a, blockIdx.y, blockIdx.y, blockIdx.x, threadIdx.x);
 }
 
 // Grid (out / 16 / BT, RKT * NPROJ, KS), 256 threads. NPROJ 2: gate (proj 0) and up (proj 1), hidden -> inter;
@@ -222,13 +223,16 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ?
 }
 
 // Grid (inter / 128, RKT), 64 threads.
+template <int PROF>
 __global__ void __launch_bounds__(64) moe_mid(const MoeLaunch a) {
-    routed_mid_block<false>(a, resolve_slot(a, blockIdx.y), blockIdx.y, blockIdx.x, threadIdx.x);
+    routed_mid_block<false, false, PROF>(a, resolve_slot(a, blockIdx.y), blockIdx.y, blockIdx.x, threadIdx.x);
 }
 
-// Grid (hidden / 128, rows), 64 threads.
+// Grid (hidden / 128, rows), 64 threads. PROF 1 (GLM's): the slots' own f32 outputs instead of their weighted sum.
+template <int PROF>
 __global__ void __launch_bounds__(64) moe_combine(const MoeLaunch a) {
-    routed_combine_block<false>(a, blockIdx.y, blockIdx.x, threadIdx.x);
+    if constexpr (PROF == 0) routed_combine_block<false>(a, blockIdx.y, blockIdx.x, threadIdx.x);
+    else routed_slots_block<false>(a, blockIdx.y, blockIdx.x, threadIdx.x);
 }
 
 template <int CB, bool WIDE, int NPROJ, bool XLDS, bool ARRIVE>
@@ -267,21 +271,32 @@ hipError_t launch_gemv_cb(const MoeLaunch& a, hipStream_t s) {
 hipError_t launch_moe_decode(const MoeLaunch& a, int form, hipStream_t s) {
     const uint32_t rkt = a.rows * (a.topk + a.shared_slots);
     hipError_t e;
-    if (form == kMoeTwoLaunches) {
+    if (form == kMoeTwoLaunches && !a.glm) {
         if ((e = launch_gemv_cb<2, true, true>(a, s)) != hipSuccess) return e;
         return launch_gemv_cb<1, false, true>(a, s);
     }
+    if (a.glm) {
+        // GLM's profile runs the five launches with its own roundings in the stages between the GEMVs
+        hipLaunchKernelGGL(moe_prep<1>, dim3(a.hidden / 128u, rkt), dim3(64), 0, s, a);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        if ((e = launch_gemv_cb<2, false, false>(a, s)) != hipSuccess) return e;
+        hipLaunchKernelGGL(moe_mid<1>, dim3(a.inter / 128u, rkt), dim3(64), 0, s, a);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        if ((e = launch_gemv_cb<1, false, false>(a, s)) != hipSuccess) return e;
+        hipLaunchKernelGGL(moe_combine<1>, dim3(a.hidden / 128u, a.rows), dim3(64), 0, s, a);
+        return hipGetLastError();
+    }
     if (form == kMoeFiveLaunches) {
-        hipLaunchKernelGGL(moe_prep, dim3(a.hidden / 128u, rkt), dim3(64), 0, s, a);
+        hipLaunchKernelGGL(moe_prep<0>, dim3(a.hidden / 128u, rkt), dim3(64), 0, s, a);
         if ((e = hipGetLastError()) != hipSuccess) return e;
         if ((e = launch_gemv_cb<2, false, false>(a, s)) != hipSuccess) return e;
     } else {
         if ((e = launch_gemv_cb<2, true, false>(a, s)) != hipSuccess) return e;
     }
-    hipLaunchKernelGGL(moe_mid, dim3(a.inter / 128u, rkt), dim3(64), 0, s, a);
+    hipLaunchKernelGGL(moe_mid<0>, dim3(a.inter / 128u, rkt), dim3(64), 0, s, a);
     if ((e = hipGetLastError()) != hipSuccess) return e;
     if ((e = launch_gemv_cb<1, false, false>(a, s)) != hipSuccess) return e;
-    hipLaunchKernelGGL(moe_combine, dim3(a.hidden / 128u, a.rows), dim3(64), 0, s, a);
+    hipLaunchKernelGGL(moe_combine<0>, dim3(a.hidden / 128u, a.rows), dim3(64), 0, s, a);
     return hipGetLastError();
 }
 

@@ -395,7 +395,7 @@ constexpr uint32_t kPfUnit = 4;
 
 __device__ __forceinline__ uint32_t wave_unit() { return blockIdx.x * 4u + (threadIdx.x >> 6); }
 
-template <int DT>
+template <int DT, int PROF>
 __global__ void __launch_bounds__(256) pf_prep(const MoeLaunch a) {
     const uint32_t nb = a.hidden / 128u, groups = (nb + kPfUnit - 1u) / kPfUnit;
     const uint32_t u0 = wave_unit(), pos = u0 / groups, lane = threadIdx.x & 63u, q = lane & 15u;
@@ -414,7 +414,7 @@ __global__ void __launch_bounds__(256) pf_prep(const MoeLaunch a) {
     for (uint32_t proj = 0; proj < 2u; ++proj) {
         float v[8];
 #pragma unroll
-        for (uint32_t r = 0; r < 8u; ++r) v[r] = round_half(xv[r]) * sc[proj][r];
+        for (uint32_t r = 0; r < 8u; ++r) v[r] = (PROF == 0 ? round_half(xv[r]) : xv[r]) * sc[proj][r];
         uint32_t hv[4];
         float sum;
         prep_row16(v, g16, hv, sum, a.defer != 0);
@@ -425,6 +425,7 @@ __global__ void __launch_bounds__(256) pf_prep(const MoeLaunch a) {
 }
 
 // gate and up finishes, the (clamped) SwiGLU, the down's prepare (routed_mid_block's statements)
+template <int PROF>
 __global__ void __launch_bounds__(256) pf_mid(const MoeLaunch a) {
     const uint32_t nb = a.inter / 128u, nbh = a.hidden / 128u, groups = (nb + kPfUnit - 1u) / kPfUnit;
     const uint32_t u0 = wave_unit(), pos = u0 / groups, lane = threadIdx.x & 63u, q = lane & 15u;
@@ -454,17 +455,49 @@ __global__ void __launch_bounds__(256) pf_mid(const MoeLaunch a) {
             up[r] = __builtin_fmaf(up[r], mul1_a(), mul1_b() * xu);
         }
     }
-    finish_row16(gt, svg, g16);
-    finish_row16(up, svu, g16);
     float d[8];
+    if constexpr (PROF == 0) {
+        finish_row16(gt, svg, g16);
+        finish_row16(up, svu, g16);
 #pragma unroll
-    for (uint32_t r = 0; r < 8u; ++r) d[r] = round_half(swiglu_clamped(gt[r], up[r], a.limit, a.clamp_at)) * sdn[r];
+        for (uint32_t r = 0; r < 8u; ++r) d[r] = round_half(swiglu_clamped(gt[r], up[r], a.limit, a.clamp_at)) * sdn[r];
+    } else {
+        finish_row16_glm(gt, svg, g16, true);
+        finish_row16_glm(up, svu, g16, true);
+#pragma unroll
+        for (uint32_t r = 0; r < 8u; ++r) d[r] = swiglu_glm(gt[r], up[r], a.limit) * sdn[r];
+    }
     uint32_t hv[4];
     float sum;
     prep_row16(d, g16, hv, sum, a.defer != 0);
     if (!live) return;
     store_pair_quad(reinterpret_cast<uint16_t*>(a.hd), qo, b, q, hv);
     if (q == 0u) a.hs[static_cast<size_t>(pos) * nb + b] = sum;
+}
+
+// GLM's profile: each placed row-slot's down finish as f32 [row-slot][hidden] (routed_slots_block's statements), by
+// sorted position
+__global__ void __launch_bounds__(256) pf_slots(const MoeLaunch a) {
+    const uint32_t nb = a.hidden / 128u, nbi = a.inter / 128u, groups = (nb + kPfUnit - 1u) / kPfUnit;
+    const uint32_t u0 = wave_unit(), pos = u0 / groups, lane = threadIdx.x & 63u, q = lane & 15u;
+    if (pos >= a.counts[a.bank.experts + a.shared_slots + 1u]) return;
+    const uint32_t b1 = (u0 % groups) * kPfUnit + (lane >> 4);
+    const bool live = b1 < nb;
+    const uint32_t b = live ? b1 : nb - 1u, i = b * 128u + 8u * q;
+    const uint32_t rk = a.order[pos];
+    const SlotRef s = resolve_slot(a, rk);
+    const Row16 g16 = row16(lane);
+    float v[8], sv[8];
+    load8_f32(a.zd, static_cast<size_t>(pos) * a.hidden + i, v);
+    load8_half(a.bank.down_svh, static_cast<size_t>(s.e) * a.hidden + i, sv);
+    if (a.defer) {
+        float xsum = 0.0f;
+        for (uint32_t t = 0; t < nbi; ++t) xsum += a.hs[static_cast<size_t>(pos) * nbi + t];
+#pragma unroll
+        for (uint32_t r = 0; r < 8u; ++r) v[r] = __builtin_fmaf(v[r], mul1_a(), mul1_b() * xsum);
+    }
+    finish_row16_glm(v, sv, g16, false);
+    if (live) store8_act<kF32>(a.y, static_cast<size_t>(rk) * a.hidden + i, v);
 }
 
 // every slot's down finish, then the score-weighted sum in slot order (routed_combine_block's statements)
@@ -659,9 +692,10 @@ hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s) {
     if ((e = hipGetLastError()) != hipSuccess) return e;
     hipLaunchKernelGGL(pf_place, dim3((p + 255u) / 256u), dim3(256), 0, s, a);
     if ((e = hipGetLastError()) != hipSuccess) return e;
-    if (a.dtype == kF32) hipLaunchKernelGGL(pf_prep<kF32>, unit_grid(p, a.hidden), dim3(256), 0, s, a);
-    else if (a.dtype == kF16) hipLaunchKernelGGL(pf_prep<kF16>, unit_grid(p, a.hidden), dim3(256), 0, s, a);
-    else hipLaunchKernelGGL(pf_prep<kBf16>, unit_grid(p, a.hidden), dim3(256), 0, s, a);
+    if (a.glm) hipLaunchKernelGGL((pf_prep<kBf16, 1>), unit_grid(p, a.hidden), dim3(256), 0, s, a);
+    else if (a.dtype == kF32) hipLaunchKernelGGL((pf_prep<kF32, 0>), unit_grid(p, a.hidden), dim3(256), 0, s, a);
+    else if (a.dtype == kF16) hipLaunchKernelGGL((pf_prep<kF16, 0>), unit_grid(p, a.hidden), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((pf_prep<kBf16, 0>), unit_grid(p, a.hidden), dim3(256), 0, s, a);
     if ((e = hipGetLastError()) != hipSuccess) return e;
 
     PfGemm g{};
@@ -683,7 +717,8 @@ hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s) {
     g.experts = a.bank.experts;
     if ((e = launch_gemm(g, a.codebook, a.max_items, 2u, a.item_rows, s)) != hipSuccess) return e;
 
-    hipLaunchKernelGGL(pf_mid, unit_grid(p, a.inter), dim3(256), 0, s, a);
+    if (a.glm) hipLaunchKernelGGL(pf_mid<1>, unit_grid(p, a.inter), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(pf_mid<0>, unit_grid(p, a.inter), dim3(256), 0, s, a);
     if ((e = hipGetLastError()) != hipSuccess) return e;
 
     g.w[0] = a.bank.down_t;
@@ -698,7 +733,8 @@ hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s) {
     g.n = a.n_dn;
     if ((e = launch_gemm(g, a.codebook, a.max_items, 1u, a.item_rows, s)) != hipSuccess) return e;
 
-    hipLaunchKernelGGL(pf_combine, unit_grid(a.rows, a.hidden), dim3(256), 0, s, a);
+    if (a.glm) hipLaunchKernelGGL(pf_slots, unit_grid(p, a.hidden), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(pf_combine, unit_grid(a.rows, a.hidden), dim3(256), 0, s, a);
     return hipGetLastError();
 }
 

@@ -142,7 +142,7 @@ __device__ __forceinline__ void store_prepared(uint32_t* base, size_t row_at, ui
 }
 
 // the gate's and the up's prepare of block b of row-slot rk: xg, xu [.][hidden], sg, su [.][hidden / 128]
-template <bool PF>
+template <bool PF, int PROF = 0>
 __device__ __forceinline__ void routed_prep_block(const MoeLaunch& a, uint32_t rk, uint32_t q, uint32_t b,
                                                   uint32_t lane) {
     const SlotRef s = resolve_slot(a, rk);
@@ -154,7 +154,7 @@ __device__ __forceinline__ void routed_prep_block(const MoeLaunch& a, uint32_t r
         const uint16_t* suh = (proj ? bank.up_suh : bank.gate_suh) + static_cast<size_t>(s.e) * a.hidden;
         uint32_t hv[2];
         float sum;
-        prep_values(a.dtype, a.x, suh, a.hidden, s.row, b, lane, hv, sum);
+        prep_values(a.dtype, a.x, suh, a.hidden, s.row, b, lane, hv, sum, PROF == 0);
 #pragma unroll
         for (uint32_t j = 0; j < 2u; ++j)
             store_prepared<PF>(proj ? a.xu : a.xg, static_cast<size_t>(q) * a.hidden, b * 128u + lane + 64u * j, hv[j]);
@@ -164,7 +164,7 @@ __device__ __forceinline__ void routed_prep_block(const MoeLaunch& a, uint32_t r
 
 // gate and up finishes, the (clamped) SwiGLU in f32 on their f16 values, and the down's prepare: hd [.][inter],
 // hs f32 [.][inter / 128]
-template <bool PF, bool COH = false>
+template <bool PF, bool COH = false, int PROF = 0>
 __device__ __forceinline__ void routed_mid_block(const MoeLaunch& a, const SlotRef& s, uint32_t q, uint32_t b,
                                                  uint32_t lane) {
     if (!s.live) return;
@@ -194,13 +194,20 @@ __device__ __forceinline__ void routed_mid_block(const MoeLaunch& a, const SlotR
             u[j] = __builtin_fmaf(u[j], mul1_a(), mul1_b() * xu);
         }
     }
-    finish_core(g, svg, lane);
-    finish_core(u, svu, lane);
     float d[2];
+    if constexpr (PROF == 0) {
+        finish_core(g, svg, lane);
+        finish_core(u, svu, lane);
 #pragma unroll
-    for (uint32_t j = 0; j < 2u; ++j) {
-        const float h = s.shared && a.sigtab ? swiglu_table(a, g[j], u[j]) : swiglu_clamped(g[j], u[j], a.limit, a.clamp_at);
-        d[j] = round_half(h) * sdn[j];
+        for (uint32_t j = 0; j < 2u; ++j) {
+            const float h = s.shared && a.sigtab ? swiglu_table(a, g[j], u[j]) : swiglu_clamped(g[j], u[j], a.limit, a.clamp_at);
+            d[j] = round_half(h) * sdn[j];
+        }
+    } else {
+        finish_core_glm(g, svg, lane, true);
+        finish_core_glm(u, svu, lane, true);
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j) d[j] = swiglu_glm(g[j], u[j], a.limit) * sdn[j];
     }
     h128_wave(d, lane);
     float sum = 0.0f;
@@ -217,7 +224,7 @@ __device__ __forceinline__ void routed_mid_block(const MoeLaunch& a, const SlotR
 
 // One slot's finished down outputs of block b (f16-valued), false for a skipped slot. COH: only the planes cross
 // workgroups inside the launch; the block sums hs came from the launch before.
-template <bool COH, bool HS_COH = false>
+template <bool COH, bool HS_COH = false, int PROF = 0>
 __device__ __forceinline__ bool routed_down_finish(const MoeLaunch& a, const SlotRef& s, uint32_t q, uint32_t b,
                                                    uint32_t lane, float (&v)[2], uint32_t ks) {
     if (!s.live) return false;  // uniform over the wave
@@ -235,7 +242,8 @@ __device__ __forceinline__ bool routed_down_finish(const MoeLaunch& a, const Slo
 #pragma unroll
         for (uint32_t j = 0; j < 2u; ++j) v[j] = __builtin_fmaf(v[j], mul1_a(), mul1_b() * xsum);
     }
-    finish_core(v, sv, lane);
+    if constexpr (PROF == 0) finish_core(v, sv, lane);
+    else finish_core_glm(v, sv, lane, false);
     return true;
 }
 
@@ -289,6 +297,22 @@ __device__ __forceinline__ void routed_store_row(const MoeLaunch& a, uint32_t ro
         } else {
             store_act_rt(a.dtype, a.y, o, acc[j]);
         }
+    }
+}
+
+// GLM's profile ends here: each routed slot's down finish as f32 [row-slot][hidden], no score, a skipped slot's output
+// left as it is (the host combines the slots and its shared expert; src/kernels/hip/decode/decode.hip:11-13)
+template <bool PF>
+__device__ __forceinline__ void routed_slots_block(const MoeLaunch& a, uint32_t row, uint32_t b, uint32_t lane) {
+    for (uint32_t k = 0; k < a.topk; ++k) {
+        const uint32_t rk = row * a.topk + k;
+        const SlotRef s = resolve_slot(a, rk);
+        if (!s.live) continue;  // uniform over the wave
+        float v[2];
+        routed_down_finish<false, false, 1>(a, s, PF ? a.inv[rk] : rk, b, lane, v, PF ? 1u : a.ks_dn);
+#pragma unroll
+        for (uint32_t j = 0; j < 2u; ++j)
+            static_cast<float*>(a.y)[static_cast<size_t>(rk) * a.hidden + b * 128u + lane + 64u * j] = v[j];
     }
 }
 

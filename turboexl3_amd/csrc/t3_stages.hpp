@@ -39,13 +39,16 @@ __device__ __forceinline__ void prep_core(float (&v)[2], uint32_t lane, uint32_t
 }
 
 // One 128-block of one row, one wave: loads, then prep_core.
+// round_x false: GLM's profile, x times suh in f32 without the f16 rounding of x.
 __device__ __forceinline__ void prep_values(int dt, const void* x, const uint16_t* suh, uint32_t in, uint32_t row,
-                                            uint32_t b, uint32_t lane, uint32_t (&hv)[2], float& sum) {
+                                            uint32_t b, uint32_t lane, uint32_t (&hv)[2], float& sum,
+                                            bool round_x = true) {
     float v[2];
 #pragma unroll
     for (uint32_t j = 0; j < 2u; ++j) {
         const uint32_t i = b * 128u + lane + 64u * j;
-        v[j] = round_half(load_act_rt(dt, x, static_cast<size_t>(row) * in + i)) * half_value(suh[i]);
+        const float xr = load_act_rt(dt, x, static_cast<size_t>(row) * in + i);
+        v[j] = (round_x ? round_half(xr) : xr) * half_value(suh[i]);
     }
     prep_core(v, lane, hv, sum);
 }
@@ -62,6 +65,27 @@ __device__ __forceinline__ void finish_core(float (&s)[2], const float (&sv)[2],
 __device__ __forceinline__ void finish_values(float (&s)[2], const uint16_t* svh, uint32_t b, uint32_t lane) {
     const float sv[2] = {half_value(svh[b * 128u + lane]), half_value(svh[b * 128u + lane + 64u])};
     finish_core(s, sv, lane);
+}
+
+// GLM's rounding profile (turboexl3 src/kernels/hip/decode/decode.hip:8-13, routed.hpp:89-98,120-133): the inner
+// products stay f32 (no f16 rounding before a finish); gate and up round to bf16 and are limited, the SiLU rounds to
+// bf16, the product rounds to bf16; a down finish stays f32.
+__device__ __forceinline__ float round_bf16(float v) { return bf16_value(bf16_bits(v)); }
+__device__ __forceinline__ void finish_core_glm(float (&s)[2], const float (&sv)[2], uint32_t lane, bool to_bf16) {
+    h128_wave(s, lane);
+#pragma unroll
+    for (uint32_t j = 0; j < 2u; ++j) {
+        s[j] = s[j] * kHadScale * sv[j];
+        if (to_bf16) s[j] = round_bf16(s[j]);
+    }
+}
+// g, u: bf16 values. limit 0: none; a NaN stays a NaN (torch.clamp).
+__device__ __forceinline__ float swiglu_glm(float g, float u, float limit) {
+    if (limit > 0.0f) {
+        g = g > limit ? limit : g;
+        u = u > limit ? limit : (u < -limit ? -limit : u);
+    }
+    return round_bf16(round_bf16(g / (1.0f + expf(-g))) * u);
 }
 
 // One element's SwiGLU in f32 on the f16-valued gate and up, with the clamp (turboexl3 src/core/ref.zig:119-140): limit 0
@@ -197,6 +221,15 @@ __device__ __forceinline__ void finish_row16(float (&s)[8], const float (&sv)[8]
     h128_row16(v, g);
 #pragma unroll
     for (uint32_t r = 0; r < 8u; ++r) s[r] = round_half(v[r] * g.scale * sv[r]);
+}
+
+__device__ __forceinline__ void finish_row16_glm(float (&s)[8], const float (&sv)[8], const Row16& g, bool to_bf16) {
+    h128_row16(s, g);
+#pragma unroll
+    for (uint32_t r = 0; r < 8u; ++r) {
+        s[r] = s[r] * g.scale * sv[r];
+        if (to_bf16) s[r] = round_bf16(s[r]);
+    }
 }
 
 // 8 adjacent values from element i (a multiple of 8) of an array whose base is 16-byte aligned
