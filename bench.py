@@ -287,6 +287,9 @@ def main() -> int:
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run one 256 MiB device copy, the known-size kernel that scales the profiler's "
                          "FETCH_SIZE / WRITE_SIZE readings")
+    ap.add_argument("--dense-rows", default="",
+                    help="comma-separated row counts above 32: time the dense projection --in-f x --out-f at --k on the "
+                         "trellis GEMM and on the W_hat form (dense_gemm_rows forced either way)")
     ap.add_argument("--in-f", type=int, default=4096)
     ap.add_argument("--out-f", type=int, default=12288)
     args = ap.parse_args()
@@ -394,6 +397,30 @@ def main() -> int:
                                       "tflops": 2 * rows * in_f * out_f / t / 1e12,
                                       "frac_of_f16_mfma_peak": 2 * rows * in_f * out_f / t / 2.5e15,
                                       "ms_to_make_w_std_once": once, "nonfinite": bad}
+    if args.dense_rows:
+        g = torch.Generator(device="cuda")
+        g.manual_seed(5)
+        tr = torch.randint(-32768, 32768, (IN_F // 16, OUT_F // 16, 16 * args.k), dtype=torch.int16, device="cuda",
+                           generator=g)
+        suh = (0.5 + torch.rand(IN_F, device="cuda", generator=g)).to(torch.float16)
+        svh = ((0.5 + torch.rand(OUT_F, device="cuda", generator=g)) / IN_F ** 0.5).to(torch.float16)
+
+        def dense_us(rows, gemm_rows):
+            api.configure(dense_gemm_rows=gemm_rows)
+            x = torch.randn(rows, IN_F, device="cuda", generator=g).to(torch.bfloat16)
+            api.linear(x, tr, suh, svh, dec)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(5):
+                api.linear(x, tr, suh, svh, dec)
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e3 / 5
+
+        out["dense_rows"] = [{"rows": r, "trellis_gemm_us": dense_us(r, 1 << 30), "w_hat_form_us": dense_us(r, 33)}
+                             for r in (int(v) for v in args.dense_rows.split(","))]
+        api.configure()
     if args.sweep:
         out["sweep"] = [measure(k, r, max(50, args.steps // 4), 10) for k in (3, 4, 5) for r in (1, 4, 16, 32)]
     if not args.no_cpu:
