@@ -12,6 +12,14 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_sessionstart(session):
+    """The tests load the in-tree library and call it only; a tree where nothing is built yet gets built once."""
+    from turboexl3_amd import _lib, build
+
+    if not os.path.exists(_lib.LIB_PATH):
+        build.build()
+
+
 def has_gpu() -> bool:
     try:
         import torch
