@@ -397,6 +397,20 @@ def main() -> int:
                                       "tflops": 2 * rows * in_f * out_f / t / 1e12,
                                       "frac_of_f16_mfma_peak": 2 * rows * in_f * out_f / t / 2.5e15,
                                       "ms_to_make_w_std_once": once, "nonfinite": bad}
+        # and with the W_hat of the trellis kept (decoded once a weight): the call above without its decode
+        w_hat = api.dequant(tr, dec)
+        api.linear_resident(x, w_hat, suh, svh)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(5):
+            api.linear_resident(x, w_hat, suh, svh)
+        e1.record()
+        torch.cuda.synchronize()
+        t = e0.elapsed_time(e1) * 1e-3 / 5
+        out["dense_prefill_resident"] = {"workload": "the same, W_hat f16 resident (117 MB)", "ms_per_call": t * 1e3,
+                                         "tflops": 2 * rows * in_f * out_f / t / 1e12,
+                                         "frac_of_f16_mfma_peak": 2 * rows * in_f * out_f / t / 2.5e15}
+        del w_hat, w_std
     if args.dense_rows:
         g = torch.Generator(device="cuda")
         g.manual_seed(5)
@@ -418,7 +432,22 @@ def main() -> int:
             torch.cuda.synchronize()
             return e0.elapsed_time(e1) * 1e3 / 5
 
-        out["dense_rows"] = [{"rows": r, "trellis_gemm_us": dense_us(r, 1 << 30), "w_hat_form_us": dense_us(r, 33)}
+        w_hat = api.dequant(tr, dec)
+
+        def resident_us(rows):
+            x = torch.randn(rows, IN_F, device="cuda", generator=g).to(torch.bfloat16)
+            api.linear_resident(x, w_hat, suh, svh)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(5):
+                api.linear_resident(x, w_hat, suh, svh)
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e3 / 5
+
+        out["dense_rows"] = [{"rows": r, "trellis_gemm_us": dense_us(r, 1 << 30), "w_hat_form_us": dense_us(r, 33),
+                              "resident_w_hat_us": resident_us(r)}
                              for r in (int(v) for v in args.dense_rows.split(","))]
         api.configure()
     if args.sweep:

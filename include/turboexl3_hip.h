@@ -158,6 +158,15 @@ int32_t t3_linear_bias(t3_stream stream, const t3_array* x, const t3_array* trel
  * (src/core/format.zig:276-291; the role of src/core/dense.zig:909-922 `dequantize`). */
 int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_array* w_hat);
 
+/* The resident W_hat (src/core/dense.zig:1323-1345, a host's opt-in: memory for compute): `t3_linear` above
+ * t3_config.dense_gemm_rows rows decodes the whole trellis to W_hat on every call; a host that keeps the W_hat of
+ * `t3_dequant` calls this instead: prepare, one plain f16 GEMM (rocBLAS, opened at run time), finish, the same launches
+ * on the same operands, so y is `t3_linear`'s W_hat form byte for byte. w_hat F16 [in, out]. Up to 32 rows, and without
+ * rocBLAS, it refuses with T3_Exl3EngineNotImplemented: decode and verify rows never read a W_hat (dense.zig:1309). */
+int32_t t3_linear_resident_workspace_bytes(const t3_array* x, const t3_array* w_hat, size_t* bytes);
+int32_t t3_linear_resident(t3_stream stream, const t3_array* x, const t3_array* w_hat, const t3_array* suh,
+                           const t3_array* svh, t3_array* y, void* workspace, size_t workspace_bytes);
+
 /* The un-rotated weight of a dense linear, made once a weight (src/core/dense.zig:1600-1676 `unrotCols`, `unrotRows`,
  * `unrotWeight`; src/root.zig:392-505 `trunkUnrot` installs it): W_std = act(((H' W_hat H)[i, o] / 128) suh[i] svh[o]),
  * one rounding, written to columns [col0, col0 + out) of w_std [in, N] (F16 or BF16: the activation dtype). A join of up

@@ -192,6 +192,45 @@ def test_dense_w_hat_form_from_512_rows(oracle, t3, in_f, out_f, n, codebook, dt
     print(f"dense W_hat form {in_f}x{out_f} n={n} {dtype}: worst {worst:.3e} (bar {bar})")
 
 
+@pytest.mark.parametrize("in_f,out_f,n,codebook,wbits,dtype", [
+    (512, 384, 64, MCG, 16, torch.float32),
+    (1024, 512, 48, MUL1, 16, torch.float16),
+    (512, 256, 128, MCG, 12, torch.bfloat16),
+])
+def test_dense_over_a_resident_w_hat(oracle, t3, in_f, out_f, n, codebook, wbits, dtype):
+    """The reference's resident trunk (src/core/dense.zig:1323-1345): the W_hat decoded once and kept serves every later
+    call's GEMM; "the kept W_hat is the per-call one byte for byte, and so is every output". Held that way against
+    `linear`'s own W_hat form at 40 and 530 rows (and so to the oracle's bars, which that form is held to), with the
+    reference's refusals: decode rows never read a W_hat."""
+    case = DenseCase(oracle, t3, 0x4E5 + in_f + n, in_f, out_f, n, codebook, wbits)
+    w_hat = t3.dequant(case.d_trellis, case.dec)
+    x_dev, x_f32 = make_x(case.rng, 530, in_f, dtype, outliers=True)
+    bar = F32_BAR if dtype == torch.float32 else BF16_DENSE_BAR
+    t3.configure(dense_gemm_rows=33)
+    try:
+        for rows in (40, 530):
+            per_call = t3.linear(x_dev[:rows], case.d_trellis, case.d_suh, case.d_svh, case.dec)
+            kept = t3.linear_resident(x_dev[:rows], w_hat, case.d_suh, case.d_svh)
+            assert bytes_of(kept) == bytes_of(per_call), f"{rows} rows: the kept W_hat's output differs"
+        yref = case.ref(x_f32[:40])
+        got = to_f32(kept[:40])
+        assert max(oracle.compare(got[r], yref[r]) for r in range(40)) <= bar
+    finally:
+        t3.configure()
+    # a 3-d x, as `linear` takes it
+    y3 = t3.linear_resident(x_dev[:80].reshape(2, 40, in_f), w_hat, case.d_suh, case.d_svh)
+    assert y3.shape == (2, 40, out_f) and bytes_of(y3[1]) == bytes_of(kept[40:80])
+    for bad, name in (
+        (lambda: t3.linear_resident(x_dev[:32], w_hat, case.d_suh, case.d_svh), "Exl3EngineNotImplemented"),
+        (lambda: t3.linear_resident(x_dev[:40], w_hat[:, :out_f - 64].contiguous(), case.d_suh, case.d_svh), "BadExl3Shape"),
+        (lambda: t3.linear_resident(x_dev[:40], w_hat.to(torch.bfloat16), case.d_suh, case.d_svh), "BadExl3Dtype"),
+        (lambda: t3.linear_resident(x_dev[:40, :in_f - 128].contiguous(), w_hat, case.d_suh, case.d_svh), "BadExl3Shape"),
+    ):
+        with pytest.raises(t3.T3Error) as err:
+            bad()
+        assert err.value.name == name
+
+
 def test_trellis_gemm_every_live_block_count(oracle, t3):
     """The GEMM's K loop is specialised by the item's live 16-row blocks (1..4 in the 64-row shape, 1..8 in the 128-row
     shape): row counts that end an item at every block count, both codebooks."""

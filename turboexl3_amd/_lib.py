@@ -69,6 +69,8 @@ SYMBOLS = {
     "t3_linear_stages": (C.c_int32, [C.c_void_p, _AP, _AP, _AP, _AP, Decode, _AP, C.c_void_p, C.c_size_t, C.c_uint32]),
     "t3_linear_bias": (C.c_int32, [C.c_void_p, _AP, _AP, _AP, _AP, _AP, Decode, _AP, C.c_void_p, C.c_size_t]),
     "t3_dequant": (C.c_int32, [C.c_void_p, _AP, Decode, _AP]),
+    "t3_linear_resident_workspace_bytes": (C.c_int32, [_AP, _AP, C.POINTER(C.c_size_t)]),
+    "t3_linear_resident": (C.c_int32, [C.c_void_p, _AP, _AP, _AP, _AP, _AP, C.c_void_p, C.c_size_t]),
     "t3_unrot_workspace_bytes": (C.c_int32, [_AP, C.POINTER(C.c_size_t)]),
     "t3_unrot_weight": (C.c_int32, [C.c_void_p, _AP, _AP, _AP, Decode, _AP, C.c_int64, C.c_void_p, C.c_void_p,
                                     C.c_size_t]),

@@ -155,6 +155,20 @@ def dequant(trellis, dec: Decode = Decode.mul1, stream=None) -> torch.Tensor:
     return w
 
 
+def linear_resident(x, w_hat, suh, svh, stream=None) -> torch.Tensor:
+    """`linear` above 32 rows over a kept W_hat (`dequant`'s output): prepare, one plain f16 GEMM, finish."""
+    L = _lib.lib()
+    ax, aw, asu, asv = _arr(x), _arr(w_hat), _arr(suh), _arr(svh)
+    need = C.c_size_t(0)
+    _check(L.t3_linear_resident_workspace_bytes(C.byref(ax), C.byref(aw), C.byref(need)))
+    y = torch.empty(*x.shape[:-1], w_hat.shape[1], dtype=x.dtype, device=x.device)
+    ay = _arr(y)
+    ws = _workspace(x.device, need.value)
+    _check(L.t3_linear_resident(_stream_ptr(stream), C.byref(ax), C.byref(aw), C.byref(asu), C.byref(asv), C.byref(ay),
+                                ws.data_ptr(), ws.numel()))
+    return y
+
+
 def unrot_weight(trellis, suh, svh, dec: Decode = Decode.mul1, dtype=torch.bfloat16, into=None, col0: int = 0,
                  stream=None):
     """The un-rotated weight W_std [in, out] in `dtype` (dense.unrotWeight), or written into columns col0.. of `into`

@@ -118,14 +118,73 @@ WhatScratch carve_dense_w_hat(DenseCall* call, void* workspace) {
     return w;
 }
 
+// prepare (natural order) -> z = f16(xp W_hat) -> finish, over a W_hat that is already there
+int32_t run_over_w_hat(const DenseLaunch& l, const uint16_t* w_hat, uint16_t* xp, uint16_t* z, hipStream_t s) {
+    if (const int32_t st = hip_status(launch_dense_prep_natural(l, xp, s)); st != T3_OK) return st;
+    if (const int32_t st = blas_gemm_f16(s, xp, w_hat, z, l.rows, l.in, l.out); st != T3_OK) return st;
+    return hip_status(launch_dense_finish_half(l, z, s));
+}
+
 int32_t run_w_hat(const DenseCall& call, const WhatScratch& w, int codebook, hipStream_t s) {
     const DenseLaunch& l = call.launch;
     if (const int32_t st = hip_status(launch_dequant(l.trellis, w.w_hat, l.in, l.out, l.n, l.wbits, codebook, s));
         st != T3_OK)
         return st;
-    if (const int32_t st = hip_status(launch_dense_prep_natural(l, w.xp, s)); st != T3_OK) return st;
-    if (const int32_t st = blas_gemm_f16(s, w.xp, w.w_hat, w.z, l.rows, l.in, l.out); st != T3_OK) return st;
-    return hip_status(launch_dense_finish_half(l, w.z, s));
+    return run_over_w_hat(l, w.w_hat, w.xp, w.z, s);
+}
+
+// The operand checks of a call over a kept W_hat f16 [in, out]: `check_dense`'s, with the W_hat in the trellis's place.
+int32_t check_resident(const t3_array* x, const t3_array* w_hat, const t3_array* suh, const t3_array* svh,
+                       const t3_array* y, DenseCall* call) {
+    if (!array_ok(x) || !array_ok(w_hat) || (suh && !array_ok(suh)) || (svh && !array_ok(svh)) || (y && !array_ok(y)))
+        return T3_BadArgs;
+    if (!aligned16(x) || !aligned16(w_hat) || (suh && !aligned16(suh)) || (svh && !aligned16(svh)) || (y && !aligned16(y)))
+        return T3_BadArgs;
+    if (x->ndim < 1 || w_hat->ndim != 2) return T3_BadExl3Shape;
+    const int64_t in = w_hat->shape[0], out = w_hat->shape[1];
+    if (in <= 0 || out <= 0 || in % 128 != 0 || out % 128 != 0 || in > (1ll << 30) || out > (1ll << 30))
+        return T3_BadExl3Shape;
+    if (x->shape[x->ndim - 1] != in) return T3_BadExl3Shape;
+    if (suh && (suh->ndim < 1 || suh->shape[0] != in)) return T3_BadExl3Shape;
+    if (svh && (svh->ndim < 1 || svh->shape[0] != out)) return T3_BadExl3Shape;
+    if (!is_act_dtype(x->dtype) || w_hat->dtype != T3_F16) return T3_BadExl3Dtype;
+    if ((suh && suh->dtype != T3_F16) || (svh && svh->dtype != T3_F16)) return T3_BadExl3Dtype;
+    int64_t rows = 1;
+    for (int i = 0; i + 1 < x->ndim; ++i) {
+        rows *= x->shape[i];
+        if (rows > (1ll << 30)) return T3_BadExl3Shape;
+    }
+    if (rows < 1) return T3_BadExl3Shape;
+    if (y) {
+        if (y->ndim != x->ndim || y->shape[y->ndim - 1] != out) return T3_BadExl3Shape;
+        for (int i = 0; i + 1 < x->ndim; ++i)
+            if (y->shape[i] != x->shape[i]) return T3_BadExl3Shape;
+        if (y->dtype != x->dtype) return T3_BadExl3Dtype;
+    }
+    // decode and verify rows never read a W_hat (src/core/dense.zig:1309 `prefillOperands`), and the GEMM is rocBLAS's
+    if (rows <= kGemvRowsMax || !blas_available()) return T3_Exl3EngineNotImplemented;
+    if (rows * in * 4 >= (1ll << 31)) return T3_Exl3EngineNotImplemented;
+    DenseLaunch& l = call->launch;
+    l.x = x->data;
+    l.suh = suh ? static_cast<const uint16_t*>(suh->data) : nullptr;
+    l.svh = svh ? static_cast<const uint16_t*>(svh->data) : nullptr;
+    l.y = y ? y->data : nullptr;
+    l.in = static_cast<uint32_t>(in);
+    l.out = static_cast<uint32_t>(out);
+    l.rows = static_cast<uint32_t>(rows);
+    l.codebook = 1;  // an exact codebook (MCG's number): the W_hat holds finished weights, no deferred map
+    l.dtype = x->dtype;
+    l.ks = 1u;
+    return T3_OK;
+}
+
+// xp f16 [rows][in] (natural order), z f16 [rows][out]
+void carve_resident(DenseCall* call, void* workspace, uint16_t** xp, uint16_t** z) {
+    const DenseLaunch& l = call->launch;
+    Carver c(workspace);
+    *xp = c.take<uint16_t>(static_cast<size_t>(l.rows) * l.in * 2u);
+    *z = c.take<uint16_t>(static_cast<size_t>(l.rows) * l.out * 2u);
+    call->workspace = c.used;
 }
 
 int32_t run_chain(const DenseCall& call, hipStream_t s, uint32_t stages) {
@@ -242,6 +301,29 @@ int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_
                                              static_cast<uint16_t*>(w_hat->data), static_cast<uint32_t>(in),
                                              static_cast<uint32_t>(out), static_cast<uint32_t>(n), d.wbits, d.codebook,
                                              static_cast<hipStream_t>(stream)));
+}
+
+int32_t t3_linear_resident_workspace_bytes(const t3_array* x, const t3_array* w_hat, size_t* bytes) {
+    if (!bytes) return T3_BadArgs;
+    t3::DenseCall call;
+    if (const int32_t st = t3::check_resident(x, w_hat, nullptr, nullptr, nullptr, &call); st != T3_OK) return st;
+    uint16_t *xp, *z;
+    t3::carve_resident(&call, nullptr, &xp, &z);
+    *bytes = call.workspace;
+    return T3_OK;
+}
+
+int32_t t3_linear_resident(t3_stream stream, const t3_array* x, const t3_array* w_hat, const t3_array* suh,
+                           const t3_array* svh, t3_array* y, void* workspace, size_t workspace_bytes) {
+    if (!suh || !svh || !y) return T3_BadArgs;
+    t3::DenseCall call;
+    if (const int32_t st = t3::check_resident(x, w_hat, suh, svh, y, &call); st != T3_OK) return st;
+    if (!t3::workspace_ok(workspace)) return T3_BadArgs;
+    uint16_t *xp, *z;
+    t3::carve_resident(&call, workspace, &xp, &z);
+    if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
+    return t3::run_over_w_hat(call.launch, static_cast<const uint16_t*>(w_hat->data), xp, z,
+                              static_cast<hipStream_t>(stream));
 }
 
 int32_t t3_unrot_workspace_bytes(const t3_array* trellis, size_t* bytes) {
