@@ -240,13 +240,17 @@ int32_t t3_moe_fused_shared(t3_stream stream, const t3_array* x, const t3_bank* 
  * with the statements of the host's router kernel as the reference restates it (src/models/qwen38/kernels/shared/
  * router_softmax_1..6.metal): the softmax over all experts in f32, each weight rounded to the dtype, their total added
  * up in ascending slot order in the dtype, each weight divided by it. The slots and weights live in the workspace's
- * tail. The reference's `gate_vec` form (the shared gate's logit computed in the launch in MLX's gemv order) is not
- * carried: pass `logit`. */
+ * tail. Exactly one of `logit` and `gate_vec` (else T3_BadExl3Shape, api.zig:399): logit [rows] as `t3_moe_fused_shared`
+ * takes it, or gate_vec BF16 [D], the shared gate's weight vector: the router's launch then also takes each row's logit
+ * x[row] . gate_vec, in the summation order the reference states for MLX's gemv (src/core/kernels/sources/
+ * gate_gemv.metal, gate_sum.metal) and rounded to bf16, at the rows and widths that gemv runs at (x BF16, 2..4 rows,
+ * D > 64, D >= 16 rows; else T3_Exl3EngineNotImplemented, api.zig:412-416). */
 int32_t t3_moe_fused_shared_routed_workspace_bytes(const t3_array* x, const t3_bank* bank, const t3_array* logits,
                                                    int64_t k, const t3_bank* shared_bank, size_t* bytes);
 int32_t t3_moe_fused_shared_routed(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* logits,
                                    int64_t k, t3_decode dec, const t3_bank* shared_bank, const t3_array* sigtab,
-                                   const t3_array* logit, t3_array* y, void* workspace, size_t workspace_bytes);
+                                   const t3_array* logit, const t3_array* gate_vec, t3_array* y, void* workspace,
+                                   size_t workspace_bytes);
 /* The routed experts under GLM's rounding profile (src/hip/plan.zig:219-247,396-403 `Profile.glm`;
  * src/kernels/hip/decode/decode.hip:8-13): x BF16 times suh in f32 (no f16 rounding of x), the inner products stay f32,
  * gate and up round to bf16 and are limited (limit 0: not), the SiLU rounds to bf16, the product rounds to bf16; y F32

@@ -406,6 +406,71 @@ def test_fused_gated_shared_expert_with_the_router_inside(oracle, t3, dtype):
     assert err.value.name == "Exl3EngineNotImplemented"
 
 
+def gate_logit_reference(x, gv):
+    """x [rows, D], gv [D] (bf16 values in f32) -> bf16 logits, summed as src/core/kernels/sources/gate_gemv.metal and
+    gate_sum.metal state MLX's gemv: lane t of 256 adds columns 4 t + 1024 i + tn in order, each group of 32 lanes folds
+    a shuffle-down tree, the 8 partials are added in order. Every operation in f32."""
+    rows, d = x.shape
+    out = np.zeros(rows, dtype=np.float32)
+    for r in range(rows):
+        res = np.zeros(256, dtype=np.float32)
+        for i in range(0, d, 1024):
+            for tn in range(4):
+                c = 4 * np.arange(256) + i + tn
+                ok = c < d
+                prod = np.zeros(256, dtype=np.float32)
+                prod[ok] = x[r, c[ok]] * gv[c[ok]]
+                res = (res + prod).astype(np.float32)
+        v = res.reshape(8, 32).copy()
+        for off in (16, 8, 4, 2, 1):
+            nxt = v.copy()
+            nxt[:, :32 - off] = v[:, :32 - off] + v[:, off:]
+            v = nxt
+        total = v[0, 0]
+        for g in range(1, 8):
+            total = np.float32(total + v[g, 0])
+        out[r] = total
+    return torch.from_numpy(out).to(torch.bfloat16)
+
+
+@pytest.mark.parametrize("hidden,rows", [(512, 2), (2560, 3), (2048, 4)])
+def test_fused_gated_shared_expert_with_the_gate_vector(oracle, t3, hidden, rows):
+    # src/models/qwen38/api.zig:386-416: with the shared gate's weight vector in the logit's place the router's launch
+    # also takes each row's logit, in the order the reference states for MLX's gemv. That order is a fixed sequence of f32
+    # operations (a product of two bf16 values is exact in f32), so the logits are held to their bytes against a numpy
+    # statement of it, which in turn sits within a bf16 step of the float64 dot; the call then equals the one given
+    # those logits, byte for byte.
+    rng = np.random.default_rng(0x6A7E + hidden)
+    inter, experts, k, n = 256, 12, 4, 48
+    bank, shared = oracle.synth_bank(rng, experts, hidden, inter, n), oracle.synth_bank(rng, 1, hidden, inter, n)
+    dbank, dshared = dev_bank(t3, bank), dev_bank(t3, shared)
+    dec = t3.Decode(MCG, 16)
+    dtype = torch.bfloat16
+    x_dev, x_f32 = make_x(rng, rows, hidden, dtype)
+    logits = torch.from_numpy(rng.standard_normal((rows, experts)).astype(np.float32)).to(dtype).cuda()
+    gv = torch.from_numpy((rng.standard_normal(hidden) * 0.05).astype(np.float32)).to(dtype)
+    table = sigmoid_table(dtype).cuda()
+    x3, l3 = x_dev.reshape(1, rows, hidden), logits.reshape(1, rows, experts)
+    y, inds, scores, glogit = t3.moe_fused_shared_routed(x3, dbank, l3, k, dec, dshared, table, None, return_routing=True,
+                                                         gate_vec=gv.cuda())
+    want = gate_logit_reference(x_f32, gv.to(torch.float32).numpy())
+    assert bytes_of(glogit.cpu()) == bytes_of(want), "the gate's logits differ from the stated order's"
+    exact = x_f32.astype(np.float64) @ gv.to(torch.float64).numpy()
+    assert np.all(np.abs(want.to(torch.float64).numpy() - exact) <= 2.0 ** -8 * np.maximum(np.abs(exact), 2.0 ** -6))
+    same = t3.moe_fused_shared_routed(x3, dbank, l3, k, dec, dshared, table, glogit)
+    assert bytes_of(y) == bytes_of(same)
+    for kwargs, logit, xs, name in (
+        ({"gate_vec": gv.cuda()}, glogit, x3, "BadExl3Shape"),                     # both
+        ({}, None, x3, "BadExl3Shape"),                                             # neither
+        ({"gate_vec": gv.cuda()}, None, x3[:, :1], "Exl3EngineNotImplemented"),     # one row: not that gemv
+        ({"gate_vec": gv[:hidden - 128].contiguous().cuda()}, None, x3, "Exl3EngineNotImplemented"),
+        ({"gate_vec": gv.to(torch.float16).cuda()}, None, x3, "Exl3EngineNotImplemented"),
+    ):
+        with pytest.raises(t3.T3Error) as err:
+            t3.moe_fused_shared_routed(xs, dbank, l3[:, :xs.shape[1]], k, dec, dshared, table, logit, **kwargs)
+        assert err.value.name == name, (kwargs.keys(), name)
+
+
 def _bf16_round64(v):
     return torch.from_numpy(np.asarray(v, dtype=np.float32)).to(torch.bfloat16).to(torch.float64).numpy()
 

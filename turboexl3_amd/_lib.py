@@ -86,7 +86,7 @@ SYMBOLS = {
     "t3_moe_fused_shared": (C.c_int32, [C.c_void_p, _AP, _BP, _AP, _AP, Decode, _BP, _AP, _AP, _AP, C.c_void_p,
                                         C.c_size_t]),
     "t3_moe_fused_shared_routed_workspace_bytes": (C.c_int32, [_AP, _BP, _AP, C.c_int64, _BP, C.POINTER(C.c_size_t)]),
-    "t3_moe_fused_shared_routed": (C.c_int32, [C.c_void_p, _AP, _BP, _AP, C.c_int64, Decode, _BP, _AP, _AP, _AP,
+    "t3_moe_fused_shared_routed": (C.c_int32, [C.c_void_p, _AP, _BP, _AP, C.c_int64, Decode, _BP, _AP, _AP, _AP, _AP,
                                                C.c_void_p, C.c_size_t]),
     "t3_moe_glm": (C.c_int32, [C.c_void_p, _AP, _BP, _AP, Decode, C.c_int32, _AP, C.c_void_p, C.c_size_t]),
     "t3_moe_workspace_bytes": (C.c_int32, [_AP, _BP, _AP, _BP, C.POINTER(C.c_size_t)]),

@@ -319,9 +319,11 @@ def moe_fused_shared(x, bank: Bank, inds, scores, dec: Decode, shared_bank: Bank
 
 
 def moe_fused_shared_routed(x, bank: Bank, logits, k: int, dec: Decode, shared_bank: Bank, sigtab, logit, stream=None,
-                            return_routing: bool = False):
+                            return_routing: bool = False, gate_vec=None):
     """qwen38's moeFusedSharedRouted: `moe_fused_shared` with the top-k and the renormalised softmax weights computed
-    from the router's logits [B, S, E] by one launch in front. return_routing: also the slots and weights it made."""
+    from the router's logits [B, S, E] by one launch in front. `logit` [rows], or None with `gate_vec` bf16 [D]: the
+    shared gate's logit is then taken in the same launch. return_routing: also the slots and weights it made (and, with
+    gate_vec, the logits)."""
     L = _lib.lib()
     ax, al = _arr(x), _arr(logits)
     cb, _keep = _cbank(bank)
@@ -331,18 +333,24 @@ def moe_fused_shared_routed(x, bank: Bank, logits, k: int, dec: Decode, shared_b
                                                         C.byref(need)))
     ws = torch.zeros(max(need.value, 256), dtype=torch.uint8, device=x.device)
     y = torch.empty_like(x)
-    ay, at, ag = _arr(y), _arr(sigtab), _arr(logit)
+    ay, at = _arr(y), _arr(sigtab)
+    ag = _arr(logit) if logit is not None else None
+    av = _arr(gate_vec) if gate_vec is not None else None
     _check(L.t3_moe_fused_shared_routed(_stream_ptr(stream), C.byref(ax), C.byref(cb), C.byref(al), int(k), dec.c(),
-                                        C.byref(sb), C.byref(at), C.byref(ag), C.byref(ay), ws.data_ptr(), ws.numel()))
+                                        C.byref(sb), C.byref(at), C.byref(ag) if ag is not None else None,
+                                        C.byref(av) if av is not None else None, C.byref(ay), ws.data_ptr(), ws.numel()))
     if not return_routing:
         return y
     rows = x.shape[0] * x.shape[1]
     slots = rows * k
     pad = lambda b: (b + 255) & ~255
-    tail = need.value - pad(slots * 4) - pad(slots * 2)
+    tail = need.value - pad(slots * 4) - pad(slots * 2) - 256
     inds = ws[tail:tail + slots * 4].view(torch.int32).reshape(rows, k).clone()
     scores = ws[tail + pad(slots * 4):tail + pad(slots * 4) + slots * 2].view(x.dtype).reshape(rows, k).clone()
-    return y, inds, scores
+    if gate_vec is None:
+        return y, inds, scores
+    glogit = ws[need.value - 256:need.value - 256 + rows * 2].view(torch.bfloat16).clone()
+    return y, inds, scores, glogit
 
 
 def moe_glm(x, bank: Bank, inds, dec: Decode, limit: int = 0, stream=None, fill: float = 0.0) -> torch.Tensor:

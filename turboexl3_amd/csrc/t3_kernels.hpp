@@ -97,6 +97,10 @@ hipError_t launch_moe_decode(const MoeLaunch& a, int form, hipStream_t s);
 // a row's top-k experts by logit (ties to the lowest id) and their renormalised softmax weights in the logits' dtype
 hipError_t launch_route_softmax(const void* logits, int32_t* inds, void* scores, uint32_t rows, uint32_t experts, uint32_t k,
                                 int dtype, hipStream_t s);
+// the same launch with the shared gate's logit of every row beside it: glogit bf16 [rows] = x [rows][hidden] . gate_vec
+hipError_t launch_route_softmax_gate(const void* logits, int32_t* inds, void* scores, uint32_t rows, uint32_t experts,
+                                     uint32_t k, const uint16_t* x, const uint16_t* gate_vec, uint16_t* glogit,
+                                     uint32_t hidden, hipStream_t s);
 
 // The same call above the decode rows: route, prepare, gate|up GEMM, mid, down GEMM, combine. xg, xu, hd hold plain f16
 // here (pair-quad order), zg, zu, zd one plane each, all by sorted position.

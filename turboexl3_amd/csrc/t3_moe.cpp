@@ -317,8 +317,8 @@ namespace {
 // router kernel, into the workspace's tail. bytes non-null: only the workspace size is wanted.
 int32_t fused_shared(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
                      const t3_array* scores, const t3_array* logits, int64_t k, t3_decode dec, const t3_bank* shared_bank,
-                     const t3_array* sigtab, const t3_array* logit, t3_array* y, void* workspace, size_t workspace_bytes,
-                     size_t* bytes) {
+                     const t3_array* sigtab, const t3_array* logit, const t3_array* gate_vec, t3_array* y, void* workspace,
+                     size_t workspace_bytes, size_t* bytes) {
     if (!shared_bank || !t3::array_ok(x)) return T3_BadArgs;
     t3_array routed_inds{}, routed_scores{};
     if (logits) {
@@ -349,34 +349,55 @@ int32_t fused_shared(t3_stream stream, const t3_array* x, const t3_bank* bank, c
     t3::carve_moe(&call, workspace);
     const size_t slots = static_cast<size_t>(call.rows) * l.topk;
     const size_t inds_at = call.workspace, scores_at = inds_at + ((slots * 4u + 255u) & ~static_cast<size_t>(255u));
-    const size_t total = logits ? scores_at + ((slots * 2u + 255u) & ~static_cast<size_t>(255u)) : call.workspace;
+    // the tail: slots, weights, and the shared gate's logit a row where the router's launch makes it
+    const size_t glogit_at = scores_at + ((slots * 2u + 255u) & ~static_cast<size_t>(255u));
+    const size_t total = logits ? glogit_at + 256u : call.workspace;
     if (bytes) {
         *bytes = total;
         return T3_OK;
     }
-    if (!y || !t3::array_ok(sigtab) || !t3::array_ok(logit)) return T3_BadArgs;
-    int64_t tab = 1, lg = 1;
+    if (!y || !t3::array_ok(sigtab)) return T3_BadArgs;
+    // the logit, or (routed form only) the gate's vector: one of the two (src/models/qwen38/api.zig:399)
+    if ((logit == nullptr) == (gate_vec == nullptr) || (gate_vec && !logits)) return T3_BadExl3Shape;
+    int64_t tab = 1;
     for (int i = 0; i < sigtab->ndim; ++i) tab *= sigtab->shape[i];
-    for (int i = 0; i < logit->ndim; ++i) lg *= logit->shape[i];
-    if (sigtab->dtype != x->dtype || tab != 65536 || logit->dtype != x->dtype || lg != static_cast<int64_t>(call.rows))
-        return T3_Exl3EngineNotImplemented;
+    if (sigtab->dtype != x->dtype || tab != 65536) return T3_Exl3EngineNotImplemented;
+    if (logit) {
+        if (!t3::array_ok(logit)) return T3_BadArgs;
+        int64_t lg = 1;
+        for (int i = 0; i < logit->ndim; ++i) lg *= logit->shape[i];
+        if (logit->dtype != x->dtype || lg != static_cast<int64_t>(call.rows)) return T3_Exl3EngineNotImplemented;
+    } else {
+        // the rows and widths MLX's matmul takes its 8-group gemv at (src/models/qwen38/api.zig:412-416)
+        if (!t3::array_ok(gate_vec) || !t3::aligned16(gate_vec)) return T3_BadArgs;
+        int64_t gv = 1;
+        for (int i = 0; i < gate_vec->ndim; ++i) gv *= gate_vec->shape[i];
+        const int64_t d = x->shape[2], rows = static_cast<int64_t>(call.rows);
+        if (x->dtype != T3_BF16 || gate_vec->dtype != T3_BF16 || gv != d || rows < 2 || rows > 4 || d <= 64 || d < 16 * rows)
+            return T3_Exl3EngineNotImplemented;
+    }
     if (!t3::workspace_ok(workspace)) return T3_BadArgs;
     if (workspace_bytes < total) return T3_WorkspaceTooSmall;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (logits) {
         int32_t* d_inds = reinterpret_cast<int32_t*>(static_cast<unsigned char*>(workspace) + inds_at);
         void* d_scores = static_cast<unsigned char*>(workspace) + scores_at;
-        if (const int32_t st = t3::hip_status(t3::launch_route_softmax(logits->data, d_inds, d_scores,
-                                                                       static_cast<uint32_t>(call.rows), l.bank.experts,
-                                                                       l.topk, x->dtype, s));
-            st != T3_OK)
-            return st;
+        uint16_t* d_glogit = reinterpret_cast<uint16_t*>(static_cast<unsigned char*>(workspace) + glogit_at);
+        const uint32_t rows = static_cast<uint32_t>(call.rows);
+        const hipError_t e =
+            gate_vec ? t3::launch_route_softmax_gate(logits->data, d_inds, d_scores, rows, l.bank.experts, l.topk,
+                                                     static_cast<const uint16_t*>(x->data),
+                                                     static_cast<const uint16_t*>(gate_vec->data), d_glogit,
+                                                     static_cast<uint32_t>(x->shape[2]), s)
+                     : t3::launch_route_softmax(logits->data, d_inds, d_scores, rows, l.bank.experts, l.topk, x->dtype, s);
+        if (const int32_t st = t3::hip_status(e); st != T3_OK) return st;
         l.slots = d_inds;
         l.scores = d_scores;
         l.score_dt = x->dtype;
+        if (gate_vec) l.slogit = d_glogit;
     }
     l.sigtab = sigtab->data;
-    l.slogit = logit->data;
+    if (logit) l.slogit = logit->data;
     return t3::hip_status(t3::launch_moe_decode(l, t3::decode_form_of(l), s));
 }
 }  // namespace
@@ -385,7 +406,8 @@ int32_t t3_moe_fused_shared(t3_stream stream, const t3_array* x, const t3_bank* 
                             const t3_array* scores, t3_decode dec, const t3_bank* shared_bank, const t3_array* sigtab,
                             const t3_array* logit, t3_array* y, void* workspace, size_t workspace_bytes) {
     if (!inds || !scores || !y) return T3_BadArgs;
-    return fused_shared(stream, x, bank, inds, scores, nullptr, 0, dec, shared_bank, sigtab, logit, y, workspace,
+    if (!logit) return T3_BadArgs;
+    return fused_shared(stream, x, bank, inds, scores, nullptr, 0, dec, shared_bank, sigtab, logit, nullptr, y, workspace,
                         workspace_bytes, nullptr);
 }
 
@@ -394,15 +416,16 @@ int32_t t3_moe_fused_shared_routed_workspace_bytes(const t3_array* x, const t3_b
     if (!bytes || !logits) return T3_BadArgs;
     const t3_decode dec = {0, 16};
     return fused_shared(nullptr, x, bank, nullptr, nullptr, logits, k, dec, shared_bank, nullptr, nullptr, nullptr, nullptr,
-                        0, bytes);
+                        nullptr, 0, bytes);
 }
 
 int32_t t3_moe_fused_shared_routed(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* logits,
                                    int64_t k, t3_decode dec, const t3_bank* shared_bank, const t3_array* sigtab,
-                                   const t3_array* logit, t3_array* y, void* workspace, size_t workspace_bytes) {
+                                   const t3_array* logit, const t3_array* gate_vec, t3_array* y, void* workspace,
+                                   size_t workspace_bytes) {
     if (!logits || !y) return T3_BadArgs;
-    return fused_shared(stream, x, bank, nullptr, nullptr, logits, k, dec, shared_bank, sigtab, logit, y, workspace,
-                        workspace_bytes, nullptr);
+    return fused_shared(stream, x, bank, nullptr, nullptr, logits, k, dec, shared_bank, sigtab, logit, gate_vec, y,
+                        workspace, workspace_bytes, nullptr);
 }
 
 }  // extern "C"

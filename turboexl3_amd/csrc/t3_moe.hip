@@ -310,10 +310,42 @@ namespace {
 // order in the dtype, rounding after every add; each weight divided by it and rounded. (The f32 sum over the experts is
 // a wave reduction whose order no source fixes.) One wave a row: lane L holds experts L + 64 i, i < 32.
 // Grid (rows), 64 threads.
-template <int DT>
-__global__ void __launch_bounds__(64) route_softmax(const void* logits, int32_t* inds, void* scores, uint32_t experts,
-                                                     uint32_t k) {
-    const uint32_t row = blockIdx.x, lane = threadIdx.x;
+//
+// GATE: four more waves take the shared gate's logit of the row, x[row] . gate_vec in bf16, in the order the reference
+// states for it (src/core/kernels/sources/gate_gemv.metal, gate_sum.metal: MLX's gemv at 2..4 rows): 8 groups of 32
+// lanes, lane t of 256 adds the products of columns 4 t + 1024 i + {0, 1, 2, 3} in that order in f32 (a product of two
+// bf16 values is exact in f32, so fused or not is the same sum), each group folds a shuffle-down tree (16, 8, 4, 2, 1),
+// the 8 partials are added in group order, and the total rounds to bf16. Columns past `hidden` add nothing. 320 threads.
+template <int DT, bool GATE>
+__global__ void __launch_bounds__(GATE ? 320 : 64) route_softmax(const void* logits, int32_t* inds, void* scores,
+                                                                 uint32_t experts, uint32_t k, const uint16_t* gx,
+                                                                 const uint16_t* gw, uint16_t* glogit, uint32_t hidden) {
+    const uint32_t row = blockIdx.x, lane = threadIdx.x & 63u;
+    if constexpr (GATE) {
+        __shared__ float gp[8];
+        if (threadIdx.x >= 64u) {
+            const uint32_t t = threadIdx.x - 64u;
+            const uint16_t* xr = gx + static_cast<size_t>(row) * hidden;
+            float res = 0.0f;
+            for (uint32_t c = 4u * t; c < hidden; c += 1024u) {
+                const uint2 xv = *reinterpret_cast<const uint2*>(xr + c), wv = *reinterpret_cast<const uint2*>(gw + c);
+                res += bf16_value(static_cast<uint16_t>(xv.x)) * bf16_value(static_cast<uint16_t>(wv.x));
+                res += bf16_value(static_cast<uint16_t>(xv.x >> 16)) * bf16_value(static_cast<uint16_t>(wv.x >> 16));
+                res += bf16_value(static_cast<uint16_t>(xv.y)) * bf16_value(static_cast<uint16_t>(wv.y));
+                res += bf16_value(static_cast<uint16_t>(xv.y >> 16)) * bf16_value(static_cast<uint16_t>(wv.y >> 16));
+            }
+#pragma unroll
+            for (int off = 16; off >= 1; off >>= 1) res += __shfl_down(res, off, 32);
+            if ((t & 31u) == 0u) gp[t >> 5] = res;
+        }
+        __syncthreads();
+        if (threadIdx.x == 64u) {
+            float total = gp[0];
+            for (uint32_t g = 1; g < 8u; ++g) total += gp[g];
+            glogit[row] = bf16_bits(total);
+        }
+        if (threadIdx.x >= 64u) return;
+    }
     const size_t base = static_cast<size_t>(row) * experts;
     constexpr float kNone = -__builtin_inff();
     float mine[32];
@@ -386,9 +418,19 @@ __global__ void __launch_bounds__(64) route_softmax(const void* logits, int32_t*
 
 hipError_t launch_route_softmax(const void* logits, int32_t* inds, void* scores, uint32_t rows, uint32_t experts, uint32_t k,
                                 int dtype, hipStream_t s) {
-    if (dtype == kF16) hipLaunchKernelGGL(route_softmax<kF16>, dim3(rows), dim3(64), 0, s, logits, inds, scores, experts, k);
-    else if (dtype == kBf16) hipLaunchKernelGGL(route_softmax<kBf16>, dim3(rows), dim3(64), 0, s, logits, inds, scores, experts, k);
-    else hipLaunchKernelGGL(route_softmax<kF32>, dim3(rows), dim3(64), 0, s, logits, inds, scores, experts, k);
+    const uint16_t* none = nullptr;
+    uint16_t* out = nullptr;
+    if (dtype == kF16) hipLaunchKernelGGL((route_softmax<kF16, false>), dim3(rows), dim3(64), 0, s, logits, inds, scores, experts, k, none, none, out, 0u);
+    else if (dtype == kBf16) hipLaunchKernelGGL((route_softmax<kBf16, false>), dim3(rows), dim3(64), 0, s, logits, inds, scores, experts, k, none, none, out, 0u);
+    else hipLaunchKernelGGL((route_softmax<kF32, false>), dim3(rows), dim3(64), 0, s, logits, inds, scores, experts, k, none, none, out, 0u);
+    return hipGetLastError();
+}
+
+hipError_t launch_route_softmax_gate(const void* logits, int32_t* inds, void* scores, uint32_t rows, uint32_t experts,
+                                     uint32_t k, const uint16_t* x, const uint16_t* gate_vec, uint16_t* glogit,
+                                     uint32_t hidden, hipStream_t s) {
+    hipLaunchKernelGGL((route_softmax<kBf16, true>), dim3(rows), dim3(320), 0, s, logits, inds, scores, experts, k, x,
+                       gate_vec, glogit, hidden);
     return hipGetLastError();
 }
 
