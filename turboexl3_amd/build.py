@@ -41,19 +41,18 @@ def _headers_mtime() -> float:
     return max(os.path.getmtime(p) for p in paths)
 
 
-# Kernels that count their own loads in flight (they issue them from inline asm and wait with s_waitcnt vmcnt(N)): a
-# register spill would put the compiler's scratch loads and stores into the same counter, so these must not spill.
-NO_SCRATCH = {"t3_prefill.hip": "pf_gemm"}
-
-
+# No kernel here may use scratch memory (a register spill, or a local array the compiler could not keep in registers):
+# the GEMM that issues its loads from inline asm and waits with s_waitcnt vmcnt(N) counts them itself, and a spill would
+# put the compiler's scratch loads and stores into the same counter; everywhere else scratch means a slower wave launch
+# and memory traffic in a latency-bound chain. The build reads the compiler's resource remarks and fails on any.
 def _check_no_scratch(src: str, remarks: str) -> None:
     name = None
     for line in remarks.splitlines():
         if "Function Name:" in line:
             name = line.split("Function Name:")[1].split()[0]
-        elif name and NO_SCRATCH[src] in name and ("ScratchSize" in line or "VGPRs Spill" in line):
+        elif name and ("ScratchSize" in line or "VGPRs Spill" in line):
             if int(line.split(":")[-1].split()[0]) != 0:
-                raise RuntimeError(f"{src}: {name} uses scratch memory ({line.strip()}); it counts its own loads in flight")
+                raise RuntimeError(f"{src}: {name} uses scratch memory ({line.strip()})")
 
 
 def _compile(src: str, force: bool) -> str:
@@ -62,15 +61,13 @@ def _compile(src: str, force: bool) -> str:
     if not force and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(path), _headers_mtime()):
         return obj
     cmd = [hipcc(), "-x", "hip", *COMMON, *HIP_FLAGS, "-c", path, "-o", obj]
-    if src in NO_SCRATCH:
-        cmd[-4:-4] = ["-Rpass-analysis=kernel-resource-usage", "-fno-caret-diagnostics"]  # remarks without source lines
+    cmd[-4:-4] = ["-Rpass-analysis=kernel-resource-usage", "-fno-caret-diagnostics"]  # remarks without source lines
     res = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in res.stderr.splitlines()
                     if "packed-fp32-ops" not in l and "kernel-resource-usage" not in l)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{err}")
-    if src in NO_SCRATCH:
-        _check_no_scratch(src, res.stderr)
+    _check_no_scratch(src, res.stderr)
     if err.strip():
         sys.stderr.write(err + "\n")
     return obj

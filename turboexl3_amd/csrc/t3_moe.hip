@@ -208,7 +208,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
                     }
                 __syncthreads();
             }
-            if (sg == 0u) routed_store_row(a, s.row, b128, lane, acc2, a.sigtab ? gated : nullptr);
+            if (sg == 0u) routed_store_row(a, s.row, b128, lane, acc2, gated);
         }
     }
 }

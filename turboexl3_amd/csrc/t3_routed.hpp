@@ -284,16 +284,17 @@ __device__ __forceinline__ void routed_down_finish_many(const MoeLaunch& a, cons
 }
 
 // a row's block b from its f32 sums: y's dtype; or two roundings: the routed output rounds to x's dtype, then the add
-// of `moeWithShared`'s tensor (src/root.zig:976-984) or of the gated shared expert's term (`gated`, null: none) rounds
-// again
+// of `moeWithShared`'s tensor (src/root.zig:976-984) or of the gated shared expert's term (`gated`, where the call has
+// a sigmoid table) rounds again
 __device__ __forceinline__ void routed_store_row(const MoeLaunch& a, uint32_t row, uint32_t b, uint32_t lane,
-                                                 const float (&acc)[2], const float* gated = nullptr) {
+                                                 const float (&acc)[2], const float (&gated)[2]) {
+    const bool has_gate = a.sigtab != nullptr;
 #pragma unroll
     for (uint32_t j = 0; j < 2u; ++j) {
         const size_t o = static_cast<size_t>(row) * a.hidden + b * 128u + lane + 64u * j;
-        if (a.shared_add || gated) {
+        if (a.shared_add || has_gate) {
             const float r = round_act(a.dtype, acc[j]);
-            store_act_rt(a.dtype, a.y, o, r + (gated ? gated[j] : load_act_rt(a.dtype, a.shared_add, o)));
+            store_act_rt(a.dtype, a.y, o, r + (has_gate ? gated[j] : load_act_rt(a.dtype, a.shared_add, o)));
         } else {
             store_act_rt(a.dtype, a.y, o, acc[j]);
         }
@@ -336,7 +337,7 @@ __device__ __forceinline__ void routed_combine_block(const MoeLaunch& a, uint32_
 #pragma unroll
         for (uint32_t j = 0; j < 2u; ++j) acc[j] = __builtin_fmaf(w, v[j], acc[j]);
     }
-    routed_store_row(a, row, b, lane, acc, a.sigtab ? gated : nullptr);
+    routed_store_row(a, row, b, lane, acc, gated);
 }
 
 }  // namespace t3
