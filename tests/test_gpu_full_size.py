@@ -26,6 +26,28 @@ def block_ref(oracle, trellis, suh, svh, x_f32, in_f, n, codebook, blk):
                                codebook, 0xFFFF, threads=8)
 
 
+def test_config1_cpu_case_2048_k4_one_row(oracle, t3):
+    # the reference's own CPU-runnable case: in = out = 2048 at K4, scale vectors sign x N(1, 0.1), one f16 row; the whole
+    # output against format.project, both codebooks, and W_hat to the bit
+    in_f = out_f = 2048
+    n = 64
+    rng = np.random.default_rng(0xC1)
+    trellis = rng.integers(0, 65536, (in_f // 16, out_f // 16, n), dtype=np.uint16)
+    sign = lambda m: rng.choice(np.array([-1.0, 1.0], dtype=np.float32), m)
+    suh = (sign(in_f) * rng.normal(1.0, 0.1, in_f)).astype(np.float16).view(np.uint16)
+    svh = (sign(out_f) * rng.normal(1.0, 0.1, out_f) / np.sqrt(in_f)).astype(np.float16).view(np.uint16)
+    d_t, d_suh, d_svh = dev_u16(trellis), dev_f16_bits(suh), dev_f16_bits(svh)
+    x_dev, x_f32 = make_x(rng, 1, in_f, torch.float16)
+    for codebook, dec in ((MCG, t3.Decode.mcg), (MUL1, t3.Decode.mul1)):
+        w_hat = oracle.reconstruct_inner(trellis, in_f, out_f, n, codebook)
+        assert np.array_equal(host_u16(t3.dequant(d_t, dec)), w_hat)
+        ref = oracle.project_rows(x_f32, trellis, suh, svh, in_f, out_f, n, codebook, 0xFFFF, threads=8, w_hat=w_hat)
+        y = t3.linear(x_dev, d_t, d_suh, d_svh, dec)
+        e = oracle.compare(to_f32(y)[0], ref[0], 2.0 ** -11)
+        assert e <= F32_BAR, f"codebook {codebook}: {e:.3e}"
+        assert bytes_of(y) == bytes_of(t3.linear_chain(x_dev, d_t, d_suh, d_svh, dec)), "one launch differs from the chain"
+
+
 @pytest.mark.parametrize("k", [3, 4, 5])
 def test_config2_qkv_shape_rows_1_4_16_32(oracle, t3, k):
     in_f, out_f, n = 4096, 12288, 16 * k

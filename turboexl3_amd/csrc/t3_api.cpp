@@ -4,14 +4,12 @@
 
 #include "../../include/turboexl3_hip.h"
 
-#include <atomic>
 #include <cstring>
 
 #include "t3_host.hpp"
 
 namespace {
 
-std::atomic<bool> g_configured{false};
 t3_config g_config = {9, 1, 1, 1, 1, 512};
 
 }  // namespace
@@ -65,7 +63,6 @@ int32_t t3_configure(const t3_config* cfg) {
                           cfg->dense_gemm_rows >= 0;
     if ((cfg->decode_form != 3 && cfg->decode_form != 4 && cfg->decode_form != 9) || !flags_ok) return T3_InvalidTurboexl3Config;
     g_config = *cfg;
-    g_configured.store(true);
     return T3_OK;
 }
 
