@@ -170,8 +170,8 @@ int32_t t3_linear_resident(t3_stream stream, const t3_array* x, const t3_array* 
 /* The un-rotated weight of a dense linear, made once a weight (src/core/dense.zig:1600-1676 `unrotCols`, `unrotRows`,
  * `unrotWeight`; src/root.zig:392-505 `trunkUnrot` installs it): W_std = act(((H' W_hat H)[i, o] / 128) suh[i] svh[o]),
  * one rounding, written to columns [col0, col0 + out) of w_std [in, N] (F16 or BF16: the activation dtype). A join of up
- * to four linears reading one x is one w_std with the members side by side (dense.zig:1613). Workspace: six bytes a
- * weight (the W_hat and pass 1's f32 copy), as in the reference. `nonfinite` (device, may be null): a u32 the kernels
+ * to four linears reading one x is one w_std with the members side by side (dense.zig:1613). Workspace: its head, then
+ * six bytes a weight (the W_hat and pass 1's f32 copy), as in the reference. `nonfinite` (device, may be null): a u32 the kernels
  * add the number of weights that left the dtype's range to; the reference keeps such a group on its trellis path
  * (root.zig:456-468). The caller zeroes it before and reads it after the stream has run. */
 int32_t t3_unrot_workspace_bytes(const t3_array* trellis, size_t* bytes);

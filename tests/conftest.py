@@ -35,3 +35,18 @@ def oracle():
 
     o.build()
     return o
+
+
+@pytest.fixture(autouse=True)
+def workspace_head_stays_zero(request):
+    """The C ABI's workspace contract: the first T3_WORKSPACE_COUNTER_BYTES bytes (the fused launches' arrival counters)
+    are zero when a workspace is first passed and every call leaves them zero, whichever entry points share it. The
+    harness keeps one workspace a device; after every GPU test its head must still be zero."""
+    yield
+    if request.node.get_closest_marker("gpu") is None:
+        return
+    api = sys.modules.get("turboexl3_amd.api")
+    if api is None:
+        return
+    for ws in api._workspaces.values():
+        assert not ws[:65536].any().item(), "a call left the workspace's counter area nonzero"

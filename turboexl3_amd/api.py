@@ -181,7 +181,7 @@ def unrot_weight(trellis, suh, svh, dec: Decode = Decode.mul1, dtype=torch.bfloa
     w = into if into is not None else torch.empty(in_f, out_f, dtype=dtype, device=trellis.device)
     need = C.c_size_t(0)
     _check(L.t3_unrot_workspace_bytes(C.byref(at), C.byref(need)))
-    ws = torch.empty(max(need.value, 256), dtype=torch.uint8, device=trellis.device)
+    ws = _workspace(trellis.device, need.value)
     bad = torch.zeros(1, dtype=torch.int32, device=trellis.device)
     asu, asv, aw = _arr(suh), _arr(svh), _arr(w)
     _check(L.t3_unrot_weight(_stream_ptr(stream), C.byref(at), C.byref(asu), C.byref(asv), dec.c(), C.byref(aw), col0,
@@ -331,7 +331,7 @@ def moe_fused_shared_routed(x, bank: Bank, logits, k: int, dec: Decode, shared_b
     need = C.c_size_t(0)
     _check(L.t3_moe_fused_shared_routed_workspace_bytes(C.byref(ax), C.byref(cb), C.byref(al), int(k), C.byref(sb),
                                                         C.byref(need)))
-    ws = torch.zeros(max(need.value, 256), dtype=torch.uint8, device=x.device)
+    ws = _workspace(x.device, need.value)
     y = torch.empty_like(x)
     ay, at = _arr(y), _arr(sigtab)
     ag = _arr(logit) if logit is not None else None

@@ -178,10 +178,12 @@ int32_t check_resident(const t3_array* x, const t3_array* w_hat, const t3_array*
     return T3_OK;
 }
 
-// xp f16 [rows][in] (natural order), z f16 [rows][out]
+// arrival counters (untouched here: a workspace's head stays zero whoever is called with it), xp f16 [rows][in]
+// (natural order), z f16 [rows][out]
 void carve_resident(DenseCall* call, void* workspace, uint16_t** xp, uint16_t** z) {
-    const DenseLaunch& l = call->launch;
+    DenseLaunch& l = call->launch;
     Carver c(workspace);
+    l.arrive = c.take<uint32_t>(kCounterBytes);
     *xp = c.take<uint16_t>(static_cast<size_t>(l.rows) * l.in * 2u);
     *z = c.take<uint16_t>(static_cast<size_t>(l.rows) * l.out * 2u);
     call->workspace = c.used;
@@ -332,6 +334,7 @@ int32_t t3_unrot_workspace_bytes(const t3_array* trellis, size_t* bytes) {
     const int64_t in = trellis->shape[0] * 16, out = trellis->shape[1] * 16;
     if (in <= 0 || out <= 0) return T3_BadExl3Shape;
     t3::Carver c(nullptr);
+    c.take<uint32_t>(t3::kCounterBytes);
     c.take<uint16_t>(static_cast<size_t>(in) * out * 2u);
     c.take<float>(static_cast<size_t>(in) * out * 4u);
     *bytes = c.used;
@@ -357,6 +360,7 @@ int32_t t3_unrot_weight(t3_stream stream, const t3_array* trellis, const t3_arra
     t3::Dec d;
     if (const int32_t st = t3::resolve_decode(dec, &d); st != T3_OK) return st;
     t3::Carver c(workspace);
+    c.take<uint32_t>(t3::kCounterBytes);  // a workspace's head: the fused launches' counters, left alone
     uint16_t* w_hat = c.take<uint16_t>(static_cast<size_t>(in) * out * 2u);
     float* r = c.take<float>(static_cast<size_t>(in) * out * 4u);
     if (workspace_bytes < c.used) return T3_WorkspaceTooSmall;
