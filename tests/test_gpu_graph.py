@@ -1,0 +1,74 @@
+"""The entry points under HIP graph capture: they allocate nothing, synchronise nothing and leave their arrival
+counters as they found them, so a serving loop can hold a decode step (or a prefill chunk) as one graph. A captured
+sequence of calls is replayed several times, with new inputs and eager work between the replays, and every replay must
+give the bytes of the same calls made eagerly."""
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_util import MCG, MUL1, bytes_of, dev_f16_bits, dev_u16, make_x
+from tests.test_gpu_moe import dev_bank, routing
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def t3():
+    from turboexl3_amd import api
+    return api
+
+
+def test_captured_calls_replay_to_the_eager_bytes(oracle, t3):
+    rng = np.random.default_rng(0x64A9)
+    in_f, out_f, n = 1024, 512, 64
+    trellis, suh, svh = oracle.synth_linear(rng, in_f, out_f, n)
+    d_t, d_suh, d_svh = dev_u16(trellis), dev_f16_bits(suh), dev_f16_bits(svh)
+    hidden, inter, experts, topk = 512, 256, 8, 4
+    bank = dev_bank(t3, oracle.synth_bank(rng, experts, hidden, inter, 48))
+    dec = t3.Decode(MCG, 16)
+
+    # static inputs, as a captured step keeps them; the rows of each call are views of one buffer a kind
+    x_dense = torch.zeros(40, in_f, dtype=torch.float16, device="cuda")
+    x_moe = torch.zeros(1, 20, hidden, dtype=torch.bfloat16, device="cuda")
+    slots = torch.zeros(1, 20, topk, dtype=torch.int32, device="cuda")
+    scores = torch.zeros(1, 20, topk, dtype=torch.float32, device="cuda")
+
+    def step():
+        return [
+            t3.linear(x_dense[:1], d_t, d_suh, d_svh, dec),          # one launch, its finish by the last arriver
+            t3.linear(x_dense[:8], d_t, d_suh, d_svh, dec),          # the three-launch chain
+            t3.linear(x_dense, d_t, d_suh, d_svh, dec),              # 40 rows: the trellis GEMM
+            t3.moe_clamped(x_moe[:, :2], bank, slots[:, :2], scores[:, :2], dec, 7),   # two arriving launches
+            t3.moe_clamped(x_moe, bank, slots, scores, dec, 7),      # 20 rows: route, GEMMs, combine
+            t3.linear(x_dense[:1], d_t, d_suh, d_svh, t3.Decode(MUL1, 16)),
+        ]
+
+    def new_inputs(seed):
+        r = np.random.default_rng(seed)
+        xd, _ = make_x(r, 40, in_f, torch.float16, outliers=True)
+        xm, _ = make_x(r, 20, hidden, torch.bfloat16)
+        s, w = routing(r, 20, topk, experts)
+        x_dense.copy_(xd)
+        x_moe.copy_(xm.reshape(1, 20, hidden))
+        slots.copy_(torch.from_numpy(s).reshape(1, 20, topk))
+        scores.copy_(torch.from_numpy(w).reshape(1, 20, topk))
+
+    new_inputs(1)
+    step()  # sizes the harness's workspace before anything is captured
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            captured = step()
+    torch.cuda.synchronize()
+    for seed in (2, 3, 4, 5):
+        new_inputs(seed)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [bytes_of(y) for y in captured]
+        want = [bytes_of(y) for y in step()]  # the program's own eager work between the replays
+        torch.cuda.synchronize()
+        for i, (g, w) in enumerate(zip(got, want)):
+            assert g == w, f"replay with inputs {seed}: call {i} differs from the eager call"
