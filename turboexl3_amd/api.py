@@ -6,6 +6,7 @@ libturboexl3_hip.so through the C ABI."""
 from __future__ import annotations
 
 import ctypes as C
+import threading
 from dataclasses import dataclass
 
 import torch
@@ -95,8 +96,9 @@ _workspaces: dict = {}
 
 
 def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    """A grow-only scratch buffer per device (the caller of the C ABI owns scratch; this harness keeps one)."""
-    key = (device.type, device.index)
+    """A grow-only scratch buffer per device and host thread (the caller of the C ABI owns scratch; calls that share a
+    workspace must be ordered on one stream, so every thread of this harness keeps its own)."""
+    key = (device.type, device.index, threading.get_ident())
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         # zero-filled once: the head of a workspace holds the fused launches' arrival counters
