@@ -320,7 +320,10 @@ def main() -> int:
         run = DenseRunner(torch, api, trellis, suh, svh, x, dec)
         t_call = run.time(steps, warmup)
         t_gemv = run.time(steps, warmup, stages=2)
+        plan = api.linear_plan(x, trellis[0], dec)
         return {"k": k, "rows": rows, "code_bytes": cb, "copies": copies, "us_per_call": t_call * 1e6,
+                "plan": {key: plan[key] for key in ("path", "launches", "tiles_a_load", "k_slices", "tiles_a_wave",
+                                                    "workgroups")},
                 "call_gbps": cb / t_call / 1e9, "gemv_us": t_gemv * 1e6, "gemv_gbps": cb / t_gemv / 1e9,
                 "gemv_frac_of_hbm": cb / t_gemv / HBM_PEAK}
 
@@ -338,7 +341,7 @@ def main() -> int:
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": f"dense decode-row GEMV in={IN_F} out={OUT_F} K={args.k} rows={args.rows} MCG w16, "
                                f"f16 activations, {head['copies']} rotating weight copies",
-                   "pct_of_8TBps": 100.0 * head["call_gbps"] * 1e9 / HBM_PEAK},
+                   "pct_of_8TBps": 100.0 * head["call_gbps"] * 1e9 / HBM_PEAK, "plan": head["plan"]},
         "roofline": {"bound": "hbm", "achieved": head["gemv_gbps"], "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": head["gemv_frac_of_hbm"],
                      "traffic": MEASURED_TRAFFIC.get((IN_F, OUT_F, args.k, args.rows)), "kernel": "t3::dense_gemv",

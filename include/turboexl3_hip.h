@@ -154,6 +154,29 @@ int32_t t3_linear_bias(t3_stream stream, const t3_array* x, const t3_array* trel
                        const t3_array* svh, const t3_array* bias, t3_decode dec, t3_array* y, void* workspace,
                        size_t workspace_bytes);
 
+/* How `t3_linear` would run a call, without launching anything: the partition a host or a profiler can read where the
+ * reference publishes its launch plans (src/hip/plan.zig:112-204 `dense`). The K slices and tiles a wave depend on the
+ * matrix alone, never on the rows of a call: a row's bytes are those of the row alone. Status as `t3_linear`'s checks. */
+enum {
+    T3_DENSE_ONE_LAUNCH = 0,   /* prepare + GEMV + finish in one kernel */
+    T3_DENSE_ARRIVE = 1,       /* prepare launch, then the GEMV whose last workgroup a block runs the finish */
+    T3_DENSE_CHAIN = 2,        /* prepare, GEMV, finish */
+    T3_DENSE_TRELLIS_GEMM = 3, /* above 32 rows: prepare, the GEMM that decodes in registers, finish */
+    T3_DENSE_W_HAT_GEMM = 4    /* from dense_gemm_rows rows: W_hat decode, prepare, plain f16 GEMM, finish */
+};
+typedef struct t3_linear_plan {
+    int32_t path;            /* T3_DENSE_* */
+    int32_t launches;
+    uint32_t rows, in, out, n;
+    uint32_t tiles_a_load;   /* adjacent output tiles one 128-bit load a lane covers (GEMV paths) */
+    uint32_t k_slices;       /* planes z [k_slices][rows][out] summed in slice order by the finish */
+    uint32_t tiles_a_wave;   /* input tiles a wave walks (GEMV paths; 0 on the GEMM paths) */
+    uint32_t workgroups;     /* of the GEMV or GEMM launch */
+    uint64_t code_bytes;     /* (in/16)(out/16) n 2: what one call reads of the trellis */
+    size_t workspace_bytes;
+} t3_linear_plan;
+int32_t t3_linear_plan_of(const t3_array* x, const t3_array* trellis, t3_decode dec, t3_linear_plan* plan);
+
 /* W_hat f16 [in, out] from trellis [in/16, out/16, n], bit-exact to format.reconstructInner
  * (src/core/format.zig:276-291; the role of src/core/dense.zig:909-922 `dequantize`). */
 int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_array* w_hat);
@@ -251,6 +274,28 @@ int32_t t3_moe_fused_shared_routed(t3_stream stream, const t3_array* x, const t3
                                    int64_t k, t3_decode dec, const t3_bank* shared_bank, const t3_array* sigtab,
                                    const t3_array* logit, const t3_array* gate_vec, t3_array* y, void* workspace,
                                    size_t workspace_bytes);
+/* How the routed entry points would run a call, without launching anything (src/hip/plan.zig:283-371 `moe`'s plans):
+ * the partitions come from the bank's widths alone. shared_bank may be NULL. Status as `t3_moe`'s checks. */
+enum {
+    T3_MOE_TWO_LAUNCHES = 0,   /* gate|up + mid, down + combine */
+    T3_MOE_FOUR_LAUNCHES = 1,  /* gate|up (prepare inside), mid, down, combine */
+    T3_MOE_FIVE_LAUNCHES = 2,  /* prepare, gate|up, mid, down, combine */
+    T3_MOE_PREFILL = 3         /* above 16 rows: route (clear, histogram, scan, place), prepare, gate|up GEMM, mid, down
+                                * GEMM, combine */
+};
+typedef struct t3_moe_plan {
+    int32_t path;              /* T3_MOE_* */
+    int32_t launches;
+    uint32_t rows, row_slots;  /* row_slots = rows (topk + shared slots) */
+    uint32_t hidden, inter, topk, shared_slots;
+    uint32_t tiles_a_wave_gu, k_slices_gu, tiles_a_load_gu;  /* gate|up GEMV (decode rows) */
+    uint32_t tiles_a_wave_dn, k_slices_dn, tiles_a_load_dn;  /* down GEMV */
+    uint32_t item_rows, max_items;                           /* prefill: rows a GEMM item, items at most */
+    uint64_t expert_code_bytes;  /* one expert's three matrices */
+    size_t workspace_bytes;
+} t3_moe_plan;
+int32_t t3_moe_plan_of(const t3_array* x, const t3_bank* bank, const t3_array* inds, const t3_bank* shared_bank,
+                       t3_moe_plan* plan);
 /* The routed experts under GLM's rounding profile (src/hip/plan.zig:219-247,396-403 `Profile.glm`;
  * src/kernels/hip/decode/decode.hip:8-13): x BF16 times suh in f32 (no f16 rounding of x), the inner products stay f32,
  * gate and up round to bf16 and are limited (limit 0: not), the SiLU rounds to bf16, the product rounds to bf16; y F32

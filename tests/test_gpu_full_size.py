@@ -102,7 +102,7 @@ def test_config5_dense_4096_rows_w_hat_form(oracle, t3):
 
 
 def test_config5_shape_few_rows_on_the_trellis_gemm(oracle, t3):
-    # few rows decode the matrix once: the launch shares the tile rows out into K parts (eight at 64 rows here, two at
+    # few rows decode the matrix once: the launch shares the tile rows out into K parts (sixteen at 64 rows here, two at
     # 600) and one item's column blocks go round all the dies; sampled blocks against the oracle either way
     in_f, out_f, n = 4096, 14336, 64
     rng = np.random.default_rng(0xC56)

@@ -1,0 +1,142 @@
+"""The library's launch partitions, read through t3_linear_plan_of / t3_moe_plan_of without a GPU (nothing is launched
+and no pointer is followed): the benchmark configurations' partitions, the rule every byte equality rests on (the K
+split of a matrix never depends on the rows of a call), and the path a call takes by its rows."""
+import ctypes as C
+
+import pytest
+
+from turboexl3_amd import _lib
+from turboexl3_amd._lib import Array, Bank, Config, Decode, LinearPlan, MoePlan, Proj
+
+F32, F16, BF16, U16, I16, U32, I32 = range(7)
+FAKE = 0x10000  # an aligned non-null address: the plan queries read descriptors only
+
+
+def arr(dtype, *shape):
+    a = Array()
+    a.data, a.ndim, a.dtype = FAKE, len(shape), dtype
+    for i, d in enumerate(shape):
+        a.shape[i] = d
+    return a
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _lib.lib()
+
+
+def linear_plan(lib, rows, in_f, out_f, n, dtype=F16):
+    p = LinearPlan()
+    st = lib.t3_linear_plan_of(C.byref(arr(dtype, rows, in_f)), C.byref(arr(U16, in_f // 16, out_f // 16, n)),
+                               Decode(1, 16), C.byref(p))
+    assert st == 0, lib.t3_error_name(st)
+    return p
+
+
+def bank_of(experts, hidden, inter, n_gu, n_dn):
+    def proj(i, o, n):
+        return Proj(arr(U16, experts, i // 16, o // 16, n), arr(F16, experts, i), arr(F16, experts, o))
+    return Bank(proj(hidden, inter, n_gu), proj(hidden, inter, n_gu), proj(inter, hidden, n_dn))
+
+
+def moe_plan(lib, rows, experts, hidden, inter, topk, n_gu, n_dn, shared=None):
+    p = MoePlan()
+    bank = bank_of(experts, hidden, inter, n_gu, n_dn)
+    st = lib.t3_moe_plan_of(C.byref(arr(BF16, 1, rows, hidden)), C.byref(bank), C.byref(arr(I32, 1, rows, topk)),
+                            C.byref(shared) if shared is not None else None, C.byref(p))
+    assert st == 0, lib.t3_error_name(st)
+    return p
+
+
+def test_config2_qkv_partition(lib):
+    # in 4096, out 12288: K3 and K4 take eight tiles a load (a tile row's 8 x 2n bytes fit one 1 KB load), K5 four;
+    # 768 workgroups either way, one launch at one row
+    for k, bt, ks in ((3, 8, 8), (4, 8, 8), (5, 4, 4)):
+        p = linear_plan(lib, 1, 4096, 12288, 16 * k)
+        assert (p.path, p.launches) == (0, 1)
+        assert (p.tiles_a_load, p.k_slices, p.workgroups) == (bt, ks, 768), (k, p.tiles_a_load, p.k_slices)
+        assert p.tiles_a_wave * 4 * p.k_slices == 4096 // 16
+        assert p.code_bytes == (4096 // 16) * (12288 // 16) * 16 * k * 2
+    assert linear_plan(lib, 1, 4096, 12288, 64).code_bytes == 25165824
+
+
+def test_the_k_split_never_depends_on_the_rows(lib):
+    for in_f, out_f, n in ((4096, 12288, 64), (4096, 151936, 96), (2048, 2048, 64), (512, 256, 36), (7168, 2048, 32)):
+        one = linear_plan(lib, 1, in_f, out_f, n)
+        for rows in (2, 3, 4, 5, 16, 17, 32):
+            p = linear_plan(lib, rows, in_f, out_f, n)
+            assert (p.k_slices, p.tiles_a_load, p.tiles_a_wave) == (one.k_slices, one.tiles_a_load, one.tiles_a_wave)
+
+
+def test_dense_path_by_rows(lib):
+    paths = {rows: linear_plan(lib, rows, 4096, 12288, 64).path for rows in (1, 2, 3, 32, 33, 511)}
+    assert paths == {1: 0, 2: 0, 3: 2, 32: 2, 33: 3, 511: 3}
+    assert linear_plan(lib, 2, 4096, 12288, 80).path == 2          # above four bits a weight: one row only
+    assert linear_plan(lib, 1, 4096, 151936, 96).path == 1         # 64 tiles a wave: prepare launch + arriving GEMV
+    assert linear_plan(lib, 1, 4096, 151936, 96).code_bytes == 466747392
+    cfg = Config()
+    lib.t3_config_default(C.byref(cfg))
+    cfg.dec_one = 0
+    assert lib.t3_configure(C.byref(cfg)) == 0
+    try:
+        assert linear_plan(lib, 1, 4096, 12288, 64).path == 2
+    finally:
+        lib.t3_config_default(C.byref(cfg))
+        assert lib.t3_configure(C.byref(cfg)) == 0
+
+
+def test_few_rows_share_the_tile_rows_out(lib):
+    # the trellis GEMM at 64 rows: one item, 56 workgroup columns spread over the dies, sixteen K parts of eight steps
+    p = linear_plan(lib, 64, 4096, 14336, 64, BF16)
+    assert (p.path, p.launches, p.k_slices) == (3, 3, 16)
+    assert p.workgroups == 56 * 16
+    q = linear_plan(lib, 300, 4096, 14336, 64, BF16)   # three items
+    assert (q.path, q.k_slices) == (3, 4)
+    assert linear_plan(lib, 600, 4096, 14336, 64, BF16).k_slices == 2
+
+
+def test_config3_routed_partition(lib):
+    shared = bank_of(1, 2048, 512, 48, 48)
+    for rows in (1, 8, 16):
+        p = moe_plan(lib, rows, 512, 2048, 512, 10, 48, 48, shared)
+        assert (p.path, p.launches) == (0, 2)
+        assert p.row_slots == rows * 11 and p.shared_slots == 1
+        assert (p.tiles_a_wave_gu, p.k_slices_gu, p.tiles_a_load_gu) == (8, 4, 8)
+        assert (p.tiles_a_wave_dn, p.k_slices_dn, p.tiles_a_load_dn) == (4, 2, 8)
+        assert p.expert_code_bytes == 1179648
+    p = moe_plan(lib, 17, 512, 2048, 512, 10, 48, 48, shared)
+    assert (p.path, p.launches) == (3, 9)
+
+
+def test_config4_prefill_items(lib):
+    p = moe_plan(lib, 2048, 256, 7168, 2048, 8, 32, 48)
+    assert p.path == 3 and p.row_slots == 16384
+    assert p.item_rows == 128                      # 64 rows an expert on average: an expert stays one item
+    assert p.max_items == 256 + 16384 // 128
+    assert p.expert_code_bytes == 2 * 3670016 + 5505024
+
+
+def test_decode_forms_by_configuration(lib):
+    cfg = Config()
+    for form, path, launches in ((3, 2, 5), (4, 1, 4), (9, 0, 2)):
+        lib.t3_config_default(C.byref(cfg))
+        cfg.decode_form = form
+        assert lib.t3_configure(C.byref(cfg)) == 0
+        try:
+            p = moe_plan(lib, 4, 12, 512, 256, 4, 64, 64)
+            assert (p.path, p.launches) == (path, launches)
+        finally:
+            lib.t3_config_default(C.byref(cfg))
+            assert lib.t3_configure(C.byref(cfg)) == 0
+
+
+def test_plan_refusals(lib):
+    p = LinearPlan()
+    st = lib.t3_linear_plan_of(C.byref(arr(F16, 1, 4000)), C.byref(arr(U16, 256, 768, 64)), Decode(1, 16), C.byref(p))
+    assert lib.t3_error_name(st).decode() == "BadExl3Shape"
+    st = lib.t3_linear_plan_of(C.byref(arr(F16, 1, 4096)), C.byref(arr(U16, 256, 768, 64)), Decode(1, 16), None)
+    assert lib.t3_error_name(st).decode() == "BadArgs"
+    m = MoePlan()
+    bank = bank_of(8, 512, 256, 64, 64)
+    st = lib.t3_moe_plan_of(C.byref(arr(BF16, 1, 2, 512)), C.byref(bank), C.byref(arr(I32, 1, 2, 33)), None, C.byref(m))
+    assert st != 0

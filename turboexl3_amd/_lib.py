@@ -57,6 +57,22 @@ BLOCK_TRUNK, BLOCK_BANK = 0, 1
 # every symbol include/turboexl3_hip.h declares: name -> (restype, argtypes)
 _AP, _BP = C.POINTER(Array), C.POINTER(Bank)
 _KP, _WP, _SZP = C.POINTER(Block), C.POINTER(Weight), C.POINTER(C.c_size_t)
+class LinearPlan(C.Structure):
+    _fields_ = [("path", C.c_int32), ("launches", C.c_int32), ("rows", C.c_uint32), ("in_f", C.c_uint32),
+                ("out_f", C.c_uint32), ("n", C.c_uint32), ("tiles_a_load", C.c_uint32), ("k_slices", C.c_uint32),
+                ("tiles_a_wave", C.c_uint32), ("workgroups", C.c_uint32), ("code_bytes", C.c_uint64),
+                ("workspace_bytes", C.c_size_t)]
+
+
+class MoePlan(C.Structure):
+    _fields_ = [("path", C.c_int32), ("launches", C.c_int32), ("rows", C.c_uint32), ("row_slots", C.c_uint32),
+                ("hidden", C.c_uint32), ("inter", C.c_uint32), ("topk", C.c_uint32), ("shared_slots", C.c_uint32),
+                ("tiles_a_wave_gu", C.c_uint32), ("k_slices_gu", C.c_uint32), ("tiles_a_load_gu", C.c_uint32),
+                ("tiles_a_wave_dn", C.c_uint32), ("k_slices_dn", C.c_uint32), ("tiles_a_load_dn", C.c_uint32),
+                ("item_rows", C.c_uint32), ("max_items", C.c_uint32), ("expert_code_bytes", C.c_uint64),
+                ("workspace_bytes", C.c_size_t)]
+
+
 _u16p = C.POINTER(C.c_uint16)
 SYMBOLS = {
     "t3_error_name": (C.c_char_p, [C.c_int32]),
@@ -65,6 +81,8 @@ SYMBOLS = {
     "t3_release_engines": (None, []),
     "t3_linear": (C.c_int32, [C.c_void_p, _AP, _AP, _AP, _AP, Decode, _AP, C.c_void_p, C.c_size_t]),
     "t3_linear_workspace_bytes": (C.c_int32, [_AP, _AP, Decode, C.POINTER(C.c_size_t)]),
+    "t3_linear_plan_of": (C.c_int32, [_AP, _AP, Decode, C.POINTER(LinearPlan)]),
+    "t3_moe_plan_of": (C.c_int32, [_AP, _BP, _AP, _BP, C.POINTER(MoePlan)]),
     "t3_linear_chain": (C.c_int32, [C.c_void_p, _AP, _AP, _AP, _AP, Decode, _AP, C.c_void_p, C.c_size_t]),
     "t3_linear_stages": (C.c_int32, [C.c_void_p, _AP, _AP, _AP, _AP, Decode, _AP, C.c_void_p, C.c_size_t, C.c_uint32]),
     "t3_linear_bias": (C.c_int32, [C.c_void_p, _AP, _AP, _AP, _AP, _AP, Decode, _AP, C.c_void_p, C.c_size_t]),

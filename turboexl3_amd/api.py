@@ -136,6 +136,28 @@ def _linear(entry, x, trellis, suh, svh, dec: Decode, stream=None) -> torch.Tens
     return y
 
 
+def _plan_dict(p) -> dict:
+    return {name: getattr(p, name) for name, _ in p._fields_}
+
+
+def linear_plan(x, trellis, dec: Decode = Decode.mul1) -> dict:
+    """How `linear` would run this call (path, launches, K slices, tiles a wave, workgroups, bytes): nothing is launched."""
+    p = _lib.LinearPlan()
+    ax, at = _arr(x), _arr(trellis)
+    _check(_lib.lib().t3_linear_plan_of(C.byref(ax), C.byref(at), dec.c(), C.byref(p)))
+    return _plan_dict(p)
+
+
+def moe_plan(x, bank: "Bank", inds, shared_bank=None) -> dict:
+    """How the routed entry points would run this call: nothing is launched."""
+    p = _lib.MoePlan()
+    ax, ai = _arr(x), _arr(inds)
+    cb, _keep = _cbank(bank)
+    sb = _cbank(shared_bank) if shared_bank is not None else None
+    _check(_lib.lib().t3_moe_plan_of(C.byref(ax), C.byref(cb), C.byref(ai), C.byref(sb[0]) if sb else None, C.byref(p)))
+    return _plan_dict(p)
+
+
 def linear(x, trellis, suh, svh, dec: Decode = Decode.mul1, stream=None) -> torch.Tensor:
     """root.linear: y [..., out] in x's dtype for x [..., in]."""
     return _linear(_lib.lib().t3_linear, x, trellis, suh, svh, dec, stream)

@@ -118,6 +118,22 @@ inline uint32_t dense_prefill_kparts(uint32_t rows, uint32_t in, uint32_t out) {
     return k;
 }
 
+// The trellis GEMM's grid over `nblk` workgroup columns (256 output columns each) and up to `max_items` items.
+// Consecutive workgroup ids go round the eight dies, and an item's columns stay on `spread` of them (so the dies' L2s
+// each hold few items' activations): with fewer than eight items an item's columns spread over 8, 4 or 2 dies, else
+// they share one. Ids a die: nbs columns x the item groups.
+inline uint32_t gemm_spread(uint32_t max_items) {
+    uint32_t spread = 8u;
+    while (spread > 1u && 8u / spread < max_items) spread >>= 1;
+    return spread;
+}
+inline uint32_t gemm_grid_x(uint32_t nblk, uint32_t max_items) {
+    const uint32_t spread = gemm_spread(max_items), nbs = (nblk + spread - 1u) / spread, group = 8u / spread;
+    return 8u * nbs * ((max_items + group - 1u) / group);
+}
+// workgroups a K part of the dense trellis GEMM launches
+inline uint32_t dense_prefill_workgroups(uint32_t out, uint32_t items) { return gemm_grid_x((out + 255u) / 256u, items); }
+
 // The W_hat form's own stages: the prepare in natural order (plain f16 [rows][in], what a plain GEMM multiplies), and the
 // finish of an f16 z [rows][out].
 hipError_t launch_dense_prep_natural(const DenseLaunch& d, uint16_t* xp, hipStream_t s);

@@ -205,11 +205,18 @@ int32_t run_chain(const DenseCall& call, hipStream_t s, uint32_t stages) {
 // prepares every row and the last arriver finishes them one after the other) and nothing to the chain, and with 16 and
 // 32 rows the planes' coherent traffic costs the arriving form more than the finish launch it saves. The forms give the
 // same bytes.
+int dense_path(const DenseLaunch& l) {
+    if (l.rows > kGemvRowsMax) return takes_w_hat(l) ? T3_DENSE_W_HAT_GEMM : T3_DENSE_TRELLIS_GEMM;
+    const uint32_t per = (l.in / 16u) / (4u * l.ks);
+    if (!config().dec_one || l.rows > (l.bt == 8u ? 2u : 1u)) return T3_DENSE_CHAIN;
+    return per % 8u == 0u && per <= 16u ? T3_DENSE_ONE_LAUNCH : T3_DENSE_ARRIVE;
+}
+
 int32_t run_fused(const DenseCall& call, hipStream_t s) {
     const DenseLaunch& l = call.launch;
-    const uint32_t per = (l.in / 16u) / (4u * l.ks);
-    if (l.rows > (l.bt == 8u ? 2u : 1u)) return run_chain(call, s, 7u);
-    if (per % 8u == 0u && per <= 16u) return hip_status(launch_dense_gemv(l, kFuseOne, s));
+    const int path = dense_path(l);
+    if (path == T3_DENSE_CHAIN) return run_chain(call, s, 7u);
+    if (path == T3_DENSE_ONE_LAUNCH) return hip_status(launch_dense_gemv(l, kFuseOne, s));
     if (const int32_t st = hip_status(launch_dense_prep(l, s)); st != T3_OK) return st;
     return hip_status(launch_dense_gemv(l, kFuseArrive, s));
 }
@@ -227,6 +234,43 @@ int32_t t3_linear_workspace_bytes(const t3_array* x, const t3_array* trellis, t3
     else if (call.launch.rows > t3::kGemvRowsMax) t3::carve_dense_prefill(&call, nullptr);
     else t3::carve_dense(&call, nullptr);
     *bytes = call.workspace;
+    return T3_OK;
+}
+
+int32_t t3_linear_plan_of(const t3_array* x, const t3_array* trellis, t3_decode dec, t3_linear_plan* plan) {
+    if (!plan) return T3_BadArgs;
+    t3::DenseCall call;
+    if (const int32_t st = t3::check_dense(x, trellis, nullptr, nullptr, dec, nullptr, 0, &call); st != T3_OK) return st;
+    t3::DenseLaunch& l = call.launch;
+    if (l.rows > t3::kGemvRowsMax && !t3::config().prefill) return T3_Exl3EngineNotImplemented;
+    const int path = t3::dense_path(l);
+    if (path == T3_DENSE_W_HAT_GEMM) t3::carve_dense_w_hat(&call, nullptr);
+    else if (path == T3_DENSE_TRELLIS_GEMM) t3::carve_dense_prefill(&call, nullptr);
+    else t3::carve_dense(&call, nullptr);
+    t3_linear_plan p = {};
+    p.path = path;
+    p.rows = l.rows;
+    p.in = l.in;
+    p.out = l.out;
+    p.n = l.n;
+    p.code_bytes = static_cast<uint64_t>(l.in / 16u) * (l.out / 16u) * l.n * 2u;
+    p.workspace_bytes = call.workspace;
+    if (path <= T3_DENSE_CHAIN) {
+        p.launches = path == T3_DENSE_ONE_LAUNCH ? 1 : path == T3_DENSE_ARRIVE ? 2 : 3;
+        p.tiles_a_load = l.bt;
+        p.k_slices = l.ks;
+        p.tiles_a_wave = (l.in / 16u) / (4u * l.ks);
+        p.workgroups = (l.out / 16u) / l.bt * l.ks;
+    } else if (path == T3_DENSE_TRELLIS_GEMM) {
+        p.launches = 3;
+        p.k_slices = l.ks;  // carve_dense_prefill set the K parts
+        const uint32_t item_rows = l.rows <= 64u ? 64u : 128u, items = (l.rows + item_rows - 1u) / item_rows;
+        p.workgroups = t3::dense_prefill_workgroups(l.out, items) * l.ks;
+    } else {
+        p.launches = 4;
+        p.k_slices = 1;
+    }
+    *plan = p;
     return T3_OK;
 }
 
@@ -269,7 +313,6 @@ int32_t t3_linear(t3_stream stream, const t3_array* x, const t3_array* trellis, 
     }
     t3::carve_dense(&call, workspace);
     if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
-    if (!t3::config().dec_one) return t3::run_chain(call, static_cast<hipStream_t>(stream), 7u);
     return t3::run_fused(call, static_cast<hipStream_t>(stream));
 }
 

@@ -246,6 +246,48 @@ int32_t t3_moe_workspace_bytes(const t3_array* x, const t3_bank* bank, const t3_
     return T3_OK;
 }
 
+int32_t t3_moe_plan_of(const t3_array* x, const t3_bank* bank, const t3_array* inds, const t3_bank* shared_bank,
+                       t3_moe_plan* plan) {
+    if (!plan) return T3_BadArgs;
+    t3::MoeCall call;
+    const t3_decode dec = {0, 16};
+    if (const int32_t st = t3::check_moe(x, bank, inds, nullptr, shared_bank, nullptr, dec, 0, nullptr, &call);
+        st != T3_OK)
+        return st;
+    const t3::MoeLaunch& l = call.launch;
+    t3_moe_plan p = {};
+    p.rows = l.rows;
+    p.row_slots = l.rows * (l.topk + l.shared_slots);
+    p.hidden = l.hidden;
+    p.inter = l.inter;
+    p.topk = l.topk;
+    p.shared_slots = l.shared_slots;
+    p.expert_code_bytes = static_cast<uint64_t>(l.hidden / 16u) * (l.inter / 16u) * 2u * (2u * l.n_gu + l.n_dn);
+    if (call.rows > T3_DECODE_ROWS_MAX) {
+        if (const int32_t st = t3::admit_prefill(call); st != T3_OK) return st;
+        t3::carve_moe_prefill(&call, nullptr);
+        p.path = T3_MOE_PREFILL;
+        p.launches = 9;
+        p.item_rows = l.item_rows;
+        p.max_items = l.max_items;
+    } else {
+        t3::carve_moe(&call, nullptr);
+        const int form = t3::decode_form_of(l);
+        p.path = form == t3::kMoeTwoLaunches ? T3_MOE_TWO_LAUNCHES
+                 : form == t3::kMoeFourLaunches ? T3_MOE_FOUR_LAUNCHES : T3_MOE_FIVE_LAUNCHES;
+        p.launches = form == t3::kMoeTwoLaunches ? 2 : form == t3::kMoeFourLaunches ? 4 : 5;
+        p.tiles_a_wave_gu = l.per_gu;
+        p.k_slices_gu = l.ks_gu;
+        p.tiles_a_load_gu = l.bt_gu;
+        p.tiles_a_wave_dn = l.per_dn;
+        p.k_slices_dn = l.ks_dn;
+        p.tiles_a_load_dn = l.bt_dn;
+    }
+    p.workspace_bytes = call.workspace;
+    *plan = p;
+    return T3_OK;
+}
+
 int32_t t3_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
                const t3_array* scores, t3_decode dec, int32_t verify_rows, t3_array* y, void* workspace,
                size_t workspace_bytes) {

@@ -651,11 +651,9 @@ inline uint32_t gemm_nblk(uint32_t out, uint32_t item_rows) {
 template <int CB, bool WIDE>
 hipError_t launch_gemm_rb(PfGemm g, uint32_t max_items, uint32_t nproj, uint32_t item_rows, hipStream_t s) {
     g.nblk = gemm_nblk(g.out, item_rows);
-    g.spread = 8u;
-    while (g.spread > 1u && 8u / g.spread < max_items) g.spread >>= 1;  // 8 / spread items share the dies
+    g.spread = gemm_spread(max_items);  // 8 / spread items share the dies
     if (g.kparts == 0u) g.kparts = 1u;
-    const uint32_t nbs = (g.nblk + g.spread - 1u) / g.spread, group = 8u / g.spread;
-    const dim3 grid(8u * nbs * ((max_items + group - 1u) / group), nproj, g.kparts), block(256);
+    const dim3 grid(gemm_grid_x(g.nblk, max_items), nproj, g.kparts), block(256);
     if (item_rows == 32u) hipLaunchKernelGGL((pf_gemm<CB, WIDE, 2>), grid, block, 0, s, g);
     else if (item_rows == 128u) hipLaunchKernelGGL((pf_gemm<CB, WIDE, 8>), grid, block, 0, s, g);
     else hipLaunchKernelGGL((pf_gemm<CB, WIDE, 4>), grid, block, 0, s, g);
