@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from tests.gpu_util import MCG, MUL1, bytes_of, dev_f16_bits, dev_u16, make_x, to_f32
+from tests.gpu_util import MCG, MUL1, bytes_of, dev_f16_bits, dev_u16, host_u16, make_x, to_f32
 
 pytestmark = pytest.mark.gpu
 
@@ -136,6 +136,22 @@ def test_dense_leading_dims_and_outliers(oracle, t3):
     yref = case.ref(x_f32)
     for r in range(6):
         assert oracle.compare(got[r], yref[r], half_ulp=2.0 ** -11) <= F32_BAR
+
+
+@pytest.mark.parametrize("in_f,out_f,n", [(128, 128, 64), (128, 256, 16), (256, 128, 128), (128, 384, 34), (384, 128, 96)])
+def test_smallest_and_odd_shapes(oracle, t3, in_f, out_f, n):
+    # the smallest admitted widths (one 128-block either side), the extreme rates, a fractional one, a width that is
+    # three blocks: every path by its rows (one launch or arriving GEMV, chain, two MFMA blocks, trellis GEMM, W_hat form)
+    for codebook in (MCG, MUL1):
+        case = DenseCase(oracle, t3, 0x5A11 + in_f + out_f + n, in_f, out_f, n, codebook)
+        x_dev, x_f32 = make_x(case.rng, 520, in_f, torch.float32)
+        yref = case.ref(x_f32)
+        for rows in (1, 2, 5, 17, 32, 33, 70, 520):
+            got = to_f32(t3.linear(x_dev[:rows], case.d_trellis, case.d_suh, case.d_svh, case.dec))
+            worst = max(oracle.compare(got[r], yref[r]) for r in range(rows))
+            assert worst <= F32_BAR, f"{in_f}x{out_f} n={n} codebook {codebook} rows {rows}: {worst:.3e}"
+        assert np.array_equal(host_u16(t3.dequant(case.d_trellis, case.dec)),
+                              oracle.reconstruct_inner(case.trellis, in_f, out_f, n, codebook))
 
 
 def test_dense_refusals(t3):

@@ -150,6 +150,29 @@ def test_launch_forms_give_the_same_bytes(oracle, t3):
         assert not ws[:65536].any()
 
 
+@pytest.mark.parametrize("hidden,inter,experts,topk,n", [(128, 128, 1, 1, 64), (128, 256, 3, 2, 16), (384, 128, 5, 3, 128),
+                                                         (256, 384, 4, 4, 34)])
+def test_smallest_and_odd_banks(oracle, t3, hidden, inter, experts, topk, n):
+    # one 128-block either side, a single expert, the extreme rates, a fractional one, three-block widths: decode rows
+    # (waves past the last K part idle), the row boundary of the chains, and the prefill chain
+    rng = np.random.default_rng(0xB0B + hidden + inter + n)
+    bank = oracle.synth_bank(rng, experts, hidden, inter, n)
+    dbank = dev_bank(t3, bank)
+    for codebook in (MCG, MUL1):
+        ref = RefBank(oracle, bank, codebook, 0xFFFF)
+        dec = t3.Decode(codebook, 16)
+        x_dev, x_f32 = make_x(rng, 40, hidden, torch.float32)
+        slots, scores = routing(rng, 40, topk, experts)
+        d_slots, d_scores = torch.from_numpy(slots).cuda(), torch.from_numpy(scores).cuda()
+        for rows in (1, 3, 16, 17, 40):
+            y = t3.moe_clamped(x_dev[:rows].reshape(1, rows, hidden), dbank, d_slots[:rows].reshape(1, rows, topk),
+                               d_scores[:rows].reshape(1, rows, topk), dec, 7)
+            got = to_f32(y).reshape(rows, hidden)
+            for r in sorted({0, rows // 2, rows - 1}):
+                e = oracle.compare(got[r], ref.row(x_f32[r], slots[r], scores[r], 7.0))
+                assert e <= 5e-3, f"{hidden}/{inter} n={n} codebook {codebook} rows {rows} row {r}: {e:.3e}"
+
+
 def test_clamp_skipped_slots_and_score_dtypes(oracle, t3):
     rng = np.random.default_rng(21)
     hidden, inter, experts, topk, n = 512, 256, 6, 4, 64
