@@ -122,6 +122,39 @@ def test_config5_shape_few_rows_on_the_trellis_gemm(oracle, t3):
         t3.configure()
 
 
+def test_many_rows_dense_and_routed(oracle, t3):
+    # long prefill chunks: 20,000 dense rows on both forms above 32 rows, 6,000 routed tokens; sampled rows (the first, the
+    # last, the item boundaries' neighbours) against the oracle
+    in_f, out_f, n, rows = 1024, 512, 48, 20000
+    rng = np.random.default_rng(0xB16)
+    trellis, suh, svh = oracle.synth_linear(rng, in_f, out_f, n)
+    d_t, d_suh, d_svh = dev_u16(trellis), dev_f16_bits(suh), dev_f16_bits(svh)
+    x_dev, x_f32 = make_x(rng, rows, in_f, torch.bfloat16)
+    sample = [0, 127, 128, 9999, rows - 129, rows - 1]
+    ref = oracle.project_rows(x_f32[sample], trellis, suh, svh, in_f, out_f, n, MUL1, 0xFFFF, threads=8)
+    for gemm_rows in (512, 0):
+        t3.configure(dense_gemm_rows=gemm_rows)
+        try:
+            got = to_f32(t3.linear(x_dev, d_t, d_suh, d_svh, t3.Decode.mul1)[sample])
+        finally:
+            t3.configure()
+        for i, r in enumerate(sample):
+            e = oracle.compare(got[i], ref[i])
+            assert e <= BF16_DENSE_BAR, f"dense_gemm_rows {gemm_rows} row {r}: {e:.3e}"
+    experts, hidden, inter, topk, tokens = 16, 512, 256, 6, 6000
+    bank = oracle.synth_bank(rng, experts, hidden, inter, 64)
+    dbank = dev_bank(t3, bank)
+    rb = RefBank(oracle, bank, MCG, 0xFFFF)
+    xm_dev, xm_f32 = make_x(rng, tokens, hidden, torch.float32)
+    slots, scores = routing_softmax(rng, tokens, topk, experts)
+    y = t3.moe(xm_dev.reshape(1, tokens, hidden), dbank, torch.from_numpy(slots).cuda().reshape(1, tokens, topk),
+               torch.from_numpy(scores).cuda().reshape(1, tokens, topk), t3.Decode.mcg)
+    got = to_f32(y).reshape(tokens, hidden)
+    for r in (0, 1, 2999, tokens - 2, tokens - 1):
+        e = oracle.compare(got[r], rb.row(xm_f32[r], slots[r], scores[r]))
+        assert e <= F32_BAR, f"token {r}: {e:.3e}"
+
+
 def routing_softmax(rng, tokens, topk, experts):
     logits = rng.standard_normal((tokens, experts)).astype(np.float32)
     slots = np.argsort(-logits, axis=1)[:, :topk].astype(np.int32)
