@@ -14,8 +14,8 @@
 // ascending order, so a row's partial sum is a function of (matrix, K part, row) only.
 //
 // Cost model (measured on MI355X): per tile a lane issues 13 vector-ALU instructions (1 v_alignbit, then v_bfe,
-// v_mul_lo, v_bitop3 a weight) and one MFMA; the MFMA holds the SIMD's issue for its 16 cycles, it does not overlap
-// vector ALU work. About 80 cycles a tile a SIMD: the kernel is instruction-bound below 6 bits a weight.
+// v_mul_lo, v_bitop3 a weight), 4 cycles of a SIMD's issue each, and one MFMA, about half of whose 16 cycles overlap
+// other waves' vector-ALU work. 60-70 cycles a tile a SIMD: the kernel is instruction-bound below 6 bits a weight.
 #pragma once
 
 #include "t3_decode.hpp"
