@@ -248,6 +248,34 @@ def test_trellis_gemm_every_live_block_count(oracle, t3):
             t3.configure()
 
 
+def test_routed_prefill_an_expert_past_the_item_cut(oracle, t3):
+    """A mean share of 64 rows an expert runs the GEMM shape whose items the route cuts at 96 rows; a skewed routing then
+    gives one expert every token (two items: 96 rows and the rest) and leaves others without a row. Every row within the
+    bar, and the rows' bytes the same as under a routing of the same tokens that takes the 128-row shape (a row's sums
+    depend on its matrix and the K order alone)."""
+    rng = np.random.default_rng(0x5CE3)
+    hidden, inter, experts, topk, tokens = 512, 256, 16, 8, 128
+    bank = oracle.synth_bank(rng, experts, hidden, inter, 48)
+    dbank = dev_bank(t3, bank)
+    ref = RefBank(oracle, bank, MCG, 0xFFFF)
+    x_dev, x_f32 = make_x(rng, 2 * tokens, hidden, torch.float32)
+    assert t3.moe_plan(x_dev[:tokens].reshape(1, tokens, hidden), dbank,
+                       torch.zeros(1, tokens, topk, dtype=torch.int32, device="cuda"))["item_rows"] == 96
+    slots = np.stack([np.concatenate([[0], 1 + rng.permutation(9)[:topk - 1]]) for _ in range(2 * tokens)]).astype(np.int32)
+    scores = (0.05 + rng.random((2 * tokens, topk)) * 0.2).astype(np.float32)
+    d_slots, d_scores = torch.from_numpy(slots).cuda(), torch.from_numpy(scores).cuda()
+    call = lambda n: t3.moe(x_dev[:n].reshape(1, n, hidden), dbank, d_slots[:n].reshape(1, n, topk),
+                            d_scores[:n].reshape(1, n, topk), t3.Decode.mcg)
+    y = call(tokens)
+    got = to_f32(y).reshape(tokens, hidden)
+    for r in (0, 63, 95, 96, 97, tokens - 1):
+        e = oracle.compare(got[r], ref.row(x_f32[r], slots[r], scores[r]))
+        assert e <= F32_BAR, f"row {r}: {e:.3e}"
+    twice = call(2 * tokens)  # 128 rows an expert on average: the 128-row shape
+    assert t3.moe_plan(x_dev.reshape(1, 2 * tokens, hidden), dbank, d_slots.reshape(1, 2 * tokens, topk))["item_rows"] == 128
+    assert bytes_of(twice[0, :tokens]) == bytes_of(y[0])
+
+
 def test_routed_prefill_many_experts_and_wide_topk(oracle, t3):
     """More experts than the route's scan handles in one pass (1024), most of them without a row, and the widest
     top-k (32)."""

@@ -111,8 +111,11 @@ def test_config3_routed_partition(lib):
 def test_config4_prefill_items(lib):
     p = moe_plan(lib, 2048, 256, 7168, 2048, 8, 32, 48)
     assert p.path == 3 and p.row_slots == 16384
-    assert p.item_rows == 128                      # 64 rows an expert on average: an expert stays one item
-    assert p.max_items == 256 + 16384 // 128
+    assert p.item_rows == 96                       # 64 rows an expert on average, 64 + 3 sqrt(64) = 88 within 96
+    assert p.max_items == 256 + 16384 // 96
+    q = moe_plan(lib, 4096, 256, 7168, 2048, 8, 32, 48)
+    assert q.item_rows == 128                      # 128 rows an expert: the full shape
+    assert [moe_plan(lib, t, 256, 7168, 2048, 8, 32, 48).item_rows for t in (512, 1024, 1280, 1344)] == [32, 64, 64, 96]
     assert p.expert_code_bytes == 2 * 3670016 + 5505024
 
 

@@ -102,6 +102,20 @@ hipError_t launch_route_softmax_gate(const void* logits, int32_t* inds, void* sc
                                      uint32_t k, const uint16_t* x, const uint16_t* gate_vec, uint16_t* glogit,
                                      uint32_t hidden, hipStream_t s);
 
+// Rows a GEMM item of a routed call of `slots` row-slots over `experts` experts (the shared slots' among them). An item
+// pays its matrix's whole decode whatever its rows, so items are as tall as the experts' shares of the call: 32 rows
+// when the mean share is small, 64, then the 128-row shape once it passes 40 (most experts then stay one item). Between
+// the two, while the mean share plus three of its standard deviations (a routing's counts scatter like sqrt(mean))
+// stays within 96 rows, the route cuts items at 96 and the GEMM runs with accumulators for six row blocks instead of
+// eight: three waves a SIMD instead of two, and the rare expert past 96 rows becomes two items.
+inline uint32_t moe_item_rows(size_t slots, size_t experts) {
+    const size_t share = slots / experts;
+    if (share <= 24u) return 32u;
+    if (share <= 40u) return 64u;
+    const float mean = static_cast<float>(slots) / static_cast<float>(experts);
+    return mean + 3.0f * __builtin_sqrtf(mean) <= 96.0f ? 96u : 128u;
+}
+
 // The same call above the decode rows: route, prepare, gate|up GEMM, mid, down GEMM, combine. xg, xu, hd hold plain f16
 // here (pair-quad order), zg, zu, zd one plane each, all by sorted position.
 hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s);

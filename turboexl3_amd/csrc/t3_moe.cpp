@@ -157,10 +157,7 @@ void carve_moe_prefill(MoeCall* call, void* workspace) {
     MoeLaunch& l = call->launch;
     const size_t p = static_cast<size_t>(l.rows) * (l.topk + l.shared_slots);
     const size_t et = static_cast<size_t>(l.bank.experts) + l.shared_slots;
-    // An item pays its matrix's whole decode whatever its rows, so items are as tall as the experts' shares of the
-    // call: 128 rows once an expert's mean share passes 40 (most experts then stay one item), 32 when it is small.
-    const size_t share = p / et;
-    l.item_rows = share <= 24u ? 32u : share <= 40u ? 64u : 128u;
+    l.item_rows = moe_item_rows(p, et);
     l.max_items = static_cast<uint32_t>((p < et ? p : et) + p / l.item_rows);
     Carver c(workspace);
     c.take<uint32_t>(kCounterBytes);

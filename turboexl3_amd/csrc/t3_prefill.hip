@@ -107,9 +107,14 @@ __device__ __forceinline__ void wait_loads() {
 //                banks at row stride 64 (measured: 4.2 cycles a wave's read, 8 unswizzled).
 // Measured before this form, with loads held in registers one step ahead: the kernel waited on the weight loads 12 %
 // of its time (strided 256-byte pieces come back slower than one step takes).
-template <int CB, bool WIDE, int RB>
-__global__ void __launch_bounds__(256) pf_gemm(const PfGemm a) {
-    constexpr uint32_t D = RB == 2 ? 3u : 4u;                // steps in flight + 1
+//
+// LBMAX < RB (the 128-row shape only): the same kernel with accumulators for LBMAX live row blocks (16 LBMAX registers
+// a lane instead of 128) and rings three steps deep, which fits three waves a SIMD where the full shape fits two. It
+// serves routings whose items the route cuts at 16 LBMAX = 96 rows (src: `moe_item_rows`).
+template <int CB, bool WIDE, int RB, int LBMAX = RB>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(LBMAX < RB ? 3 : 1, 8))) pf_gemm(const PfGemm a) {
+    constexpr bool kShort = LBMAX < RB;
+    constexpr uint32_t D = (RB == 2 || kShort) ? 3u : 4u;    // steps in flight + 1
     constexpr uint32_t BM = RB * 16u;
     constexpr uint32_t kAStep = BM * 64u;                     // LDS bytes of the item's rows a step
     constexpr uint32_t kALoads = RB >= 4 ? RB / 4u : 1u;      // activation loads a wave a step (16 rows each)
@@ -278,6 +283,15 @@ __global__ void __launch_bounds__(256) pf_gemm(const PfGemm a) {
             case 2: run.template operator()<2>(); break;
             case 3: run.template operator()<3>(); break;
             default: run.template operator()<4>(); break;
+        }
+    } else if constexpr (kShort) {
+        switch (live_blocks) {
+            case 1: run.template operator()<1>(); break;
+            case 2: run.template operator()<2>(); break;
+            case 3: run.template operator()<3>(); break;
+            case 4: run.template operator()<4>(); break;
+            case 5: run.template operator()<5>(); break;
+            default: run.template operator()<6>(); break;
         }
     } else {
         switch (live_blocks) {
@@ -656,6 +670,7 @@ hipError_t launch_gemm_rb(PfGemm g, uint32_t max_items, uint32_t nproj, uint32_t
     const dim3 grid(gemm_grid_x(g.nblk, max_items), nproj, g.kparts), block(256);
     if (item_rows == 32u) hipLaunchKernelGGL((pf_gemm<CB, WIDE, 2>), grid, block, 0, s, g);
     else if (item_rows == 128u) hipLaunchKernelGGL((pf_gemm<CB, WIDE, 8>), grid, block, 0, s, g);
+    else if (item_rows == 96u) hipLaunchKernelGGL((pf_gemm<CB, WIDE, 8, 6>), grid, block, 0, s, g);
     else hipLaunchKernelGGL((pf_gemm<CB, WIDE, 4>), grid, block, 0, s, g);
     return hipGetLastError();
 }
