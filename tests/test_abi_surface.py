@@ -54,7 +54,8 @@ def test_configure_refuses_unserved_values(lib):
     from turboexl3_amd._lib import Config
     cfg = Config()
     lib.t3_config_default(C.byref(cfg))
-    assert (cfg.decode_form, cfg.dec_one, cfg.prefill, cfg.mcg_pair, cfg.mul1_defer, cfg.dense_gemm_rows) == (9, 1, 1, 1, 1, 512)
+    assert (cfg.decode_form, cfg.dec_one, cfg.prefill, cfg.mcg_pair, cfg.mul1_defer, cfg.dense_gemm_rows,
+            cfg.dense_rows_alone) == (9, 1, 1, 1, 1, 512, 0)
     cfg.decode_form = 5
     assert lib.t3_error_name(lib.t3_configure(C.byref(cfg))).decode() == "InvalidTurboexl3Config"
     cfg.decode_form, cfg.dense_gemm_rows = 9, -1

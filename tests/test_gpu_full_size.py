@@ -122,6 +122,36 @@ def test_config5_shape_few_rows_on_the_trellis_gemm(oracle, t3):
         t3.configure()
 
 
+def test_config5_shape_rows_alone_configuration(oracle, t3):
+    # The reference's own GEMM holds rows 0-16 of a 40-, 129- or 200-row call to the bytes of the 17-row call
+    # (src/hip_tests.zig:876-879). Here the launch shape above 32 rows follows the rows by default (sixteen K parts at 64
+    # rows of this shape, two at 600, the W_hat form from 512), so those bytes may differ between row counts;
+    # dense_rows_alone = 1 pins one K part on the trellis GEMM and gives the reference's invariant back.
+    in_f, out_f, n = 4096, 14336, 64
+    rng = np.random.default_rng(0xC57)
+    trellis, suh, svh = oracle.synth_linear(rng, in_f, out_f, n)
+    d_t, d_suh, d_svh = dev_u16(trellis), dev_f16_bits(suh), dev_f16_bits(svh)
+    x_dev, x_f32 = make_x(rng, 600, in_f, torch.bfloat16)
+    plans = {rows: t3.linear_plan(x_dev[:rows], d_t, t3.Decode.mcg) for rows in (64, 300, 600)}
+    assert [plans[r]["k_slices"] for r in (64, 300, 600)] == [16, 4, 1] and plans[600]["path"] == 4
+    t3.configure(dense_rows_alone=1)
+    try:
+        first = None
+        for rows in (33, 64, 300, 600):
+            plan = t3.linear_plan(x_dev[:rows], d_t, t3.Decode.mcg)
+            assert (plan["path"], plan["k_slices"]) == (3, 1)
+            y = t3.linear(x_dev[:rows], d_t, d_suh, d_svh, t3.Decode.mcg)
+            first = bytes_of(y[:33]) if first is None else first
+            assert bytes_of(y[:33]) == first, f"rows 0-32 of {rows} rows differ from the 33-row call"
+        got = to_f32(y[[0, 32, 599]])
+        for blk in (0, 57, out_f // 128 - 1):
+            ref = block_ref(oracle, trellis, suh, svh, x_f32[[0, 32, 599]], in_f, n, MCG, blk)
+            for i in range(3):
+                assert oracle.compare(got[i, 128 * blk:128 * blk + 128], ref[i]) <= BF16_DENSE_BAR
+    finally:
+        t3.configure()
+
+
 def test_many_rows_dense_and_routed(oracle, t3):
     # long prefill chunks: 20,000 dense rows on both forms above 32 rows, 6,000 routed tokens; sampled rows (the first, the
     # last, the item boundaries' neighbours) against the oracle

@@ -82,7 +82,7 @@ void carve_dense(DenseCall* call, void* workspace) {
 // Above 32 rows: xq plain f16 [rows][in], xs f32 [rows][in / 128], z f32 [K parts][rows][out].
 void carve_dense_prefill(DenseCall* call, void* workspace) {
     DenseLaunch& l = call->launch;
-    l.ks = dense_prefill_kparts(l.rows, l.in, l.out);
+    l.ks = config().dense_rows_alone ? 1u : dense_prefill_kparts(l.rows, l.in, l.out);
     Carver c(workspace);
     l.arrive = c.take<uint32_t>(kCounterBytes);
     l.xq = c.take<uint32_t>(static_cast<size_t>(l.rows) * l.in * 2u);
@@ -97,7 +97,7 @@ constexpr uint32_t kGemvRowsMax = 32;
 // (src/core/dense.zig:909-922,1290-1302): the decode is paid once a call, not once a 64-row item.
 bool takes_w_hat(const DenseLaunch& l) {
     const int32_t from = config().dense_gemm_rows;
-    return from > 0 && l.rows >= static_cast<uint32_t>(from) && blas_available();
+    return !config().dense_rows_alone && from > 0 && l.rows >= static_cast<uint32_t>(from) && blas_available();
 }
 
 struct WhatScratch {
