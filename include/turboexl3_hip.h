@@ -153,6 +153,20 @@ int32_t t3_linear_stages(t3_stream stream, const t3_array* x, const t3_array* tr
                          const t3_array* svh, t3_decode dec, t3_array* y, void* workspace, size_t workspace_bytes,
                          uint32_t stages);
 
+/* `t3_linear` at its decode rows (1..32) for callers that cannot allocate or pass scratch: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc. It has no counterpart in the reference (whose engines
+ * own their scratch, src/hip/plan.zig:137-146). The scratch `t3_linear` takes as `workspace` lives in a device array of
+ * the library itself, T3_STATIC_SCRATCH_BYTES on every GPU the library runs on, held until the process ends; the call
+ * allocates nothing, frees nothing and calls no library routine that could. Same kernels, same launches, same bytes
+ * as `t3_linear` for the same operands. Refusals before any launch: more than 32 rows: T3_Exl3EngineNotImplemented;
+ * a call whose scratch (`t3_linear_workspace_bytes`) exceeds T3_STATIC_SCRATCH_BYTES: T3_WorkspaceTooSmall; else as
+ * `t3_linear`. All calls on one GPU share that GPU's array: calls that overlap on one GPU (two streams, two threads)
+ * race on it; order them on one stream. The first call on a device looks up the array's address there
+ * (hipGetSymbolAddress) and clears its counter head on `stream`: make that call outside graph capture. */
+#define T3_STATIC_SCRATCH_BYTES (16u << 20)
+int32_t t3_linear_static(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
+                         const t3_array* svh, t3_decode dec, t3_array* y);
+
 /* `t3_linear` plus a bias [out] in x's dtype: one add in x's dtype after the projection's own output rounding, so a
  * sum rounds twice (src/root.zig:358-376 `linearBias`). */
 int32_t t3_linear_bias(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,

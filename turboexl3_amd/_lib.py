@@ -9,6 +9,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "lib", "libturboexl3_hip.so")
 
 T3_MAX_DIMS = 8
+STATIC_SCRATCH_BYTES = 16 << 20
 
 # t3_dtype
 F32, F16, BF16, U16, I16, U32, I32 = range(7)
@@ -81,6 +82,7 @@ SYMBOLS = {
     "t3_configure": (C.c_int32, [C.POINTER(Config)]),
     "t3_release_engines": (None, []),
     "t3_linear": (C.c_int32, [C.c_void_p, _AP, _AP, _AP, _AP, Decode, _AP, C.c_void_p, C.c_size_t]),
+    "t3_linear_static": (C.c_int32, [C.c_void_p, _AP, _AP, _AP, _AP, Decode, _AP]),
     "t3_linear_workspace_bytes": (C.c_int32, [_AP, _AP, Decode, C.POINTER(C.c_size_t)]),
     "t3_linear_plan_of": (C.c_int32, [_AP, _AP, Decode, C.POINTER(LinearPlan)]),
     "t3_moe_plan_of": (C.c_int32, [_AP, _BP, _AP, _BP, C.POINTER(MoePlan)]),

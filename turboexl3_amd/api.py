@@ -163,6 +163,17 @@ def linear(x, trellis, suh, svh, dec: Decode = Decode.mul1, stream=None) -> torc
     return _linear(_lib.lib().t3_linear, x, trellis, suh, svh, dec, stream)
 
 
+def linear_static(x, trellis, suh, svh, dec: Decode = Decode.mul1, stream=None, out=None) -> torch.Tensor:
+    """`linear` at decode rows through the entry point that allocates nothing: its scratch is the library's own device
+    array (16 MiB a GPU). `out`: the caller's y (this harness allocates one otherwise; the C call never does)."""
+    ax, at, asu, asv = _arr(x), _arr(trellis), _arr(suh), _arr(svh)
+    y = out if out is not None else torch.empty(*x.shape[:-1], trellis.shape[1] * 16, dtype=x.dtype, device=x.device)
+    ay = _arr(y)
+    _check(_lib.lib().t3_linear_static(_stream_ptr(stream), C.byref(ax), C.byref(at), C.byref(asu), C.byref(asv), dec.c(),
+                                       C.byref(ay)))
+    return y
+
+
 def linear_chain(x, trellis, suh, svh, dec: Decode = Decode.mul1, stream=None) -> torch.Tensor:
     """The three-launch chain `linear`'s fused launch must equal byte for byte."""
     return _linear(_lib.lib().t3_linear_chain, x, trellis, suh, svh, dec, stream)

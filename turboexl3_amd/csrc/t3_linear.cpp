@@ -1,5 +1,7 @@
 // `linear`: one dense EXL3 projection (turboexl3 src/root.zig:309-351), its chain form, and W_hat's decode.
 
+#include <atomic>
+
 #include "t3_host.hpp"
 
 namespace t3 {
@@ -442,6 +444,68 @@ int32_t t3_linear_unrot(t3_stream stream, const t3_array* x, const t3_array* w_s
                               static_cast<const unsigned char*>(w_std->data) + static_cast<size_t>(col0) * esz,
                               static_cast<uint32_t>(w_std->shape[1]), y->data, static_cast<uint32_t>(rows),
                               static_cast<uint32_t>(in), static_cast<uint32_t>(cols));
+}
+
+}  // extern "C"
+
+/* ---- the decode-row projection for callers that cannot allocate ------------------------------------------------ */
+
+namespace {
+
+// The scratch `t3_linear` takes from its caller (arrival counters, prepared rows, block sums, planes), here in the
+// library's own device memory: every GPU that runs this library holds its own copy of the array until the process
+// ends. In host code the array's name is only a handle for hipGetSymbolAddress: the address each device gave its copy
+// is looked up once a device and kept in `static_scratch_ptr`, and only that pointer ever reaches a kernel.
+static __device__ __align__(256) unsigned char scratch[T3_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+std::atomic<unsigned char*> static_scratch_ptr[kMaxDevices];
+
+// grid (ceil(words / 256)), 256 threads
+__global__ void __launch_bounds__(256) static_scratch_clear(uint32_t* p, uint32_t words) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i < words) p[i] = 0u;
+}
+
+// The current device's copy of the array. The first call on a device looks its address up and clears the counter head
+// on `s` (the loader zero-fills the array too; the clear makes the contract explicit). Two threads racing through the
+// first call store the same address and both clear before their own launches on their own streams' order.
+int32_t static_scratch_of(hipStream_t s, unsigned char** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return T3_HipFailed;
+    unsigned char* p = static_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        void* sym = nullptr;
+        if (hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)) != hipSuccess || !sym) return T3_HipFailed;
+        p = static_cast<unsigned char*>(sym);
+        const uint32_t words = static_cast<uint32_t>(t3::kCounterBytes / 4u);
+        hipLaunchKernelGGL(static_scratch_clear, dim3((words + 255u) / 256u), dim3(256), 0, s,
+                           reinterpret_cast<uint32_t*>(p), words);
+        if (hipGetLastError() != hipSuccess) return T3_HipFailed;
+        static_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return T3_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t t3_linear_static(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
+                         const t3_array* svh, t3_decode dec, t3_array* y) {
+    if (!suh || !svh || !y) return T3_BadArgs;
+    t3::DenseCall call;
+    if (const int32_t st = t3::check_dense(x, trellis, suh, svh, dec, y, 0, &call); st != T3_OK) return st;
+    // decode rows only: above them `t3_linear` may run a library GEMM, which allocates
+    if (call.launch.rows > t3::kGemvRowsMax) return T3_Exl3EngineNotImplemented;
+    t3::carve_dense(&call, nullptr);
+    if (call.workspace > static_cast<size_t>(T3_STATIC_SCRATCH_BYTES)) return T3_WorkspaceTooSmall;
+    unsigned char* base = nullptr;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (const int32_t st = static_scratch_of(s, &base); st != T3_OK) return st;
+    t3::carve_dense(&call, base);
+    return t3::run_fused(call, s);
 }
 
 }  // extern "C"
