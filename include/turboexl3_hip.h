@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define T3_ABI_VERSION 3
+#define T3_ABI_VERSION 4
 #define T3_WORKSPACE_COUNTER_BYTES 65536
 
 typedef void* t3_stream; /* hipStream_t */
@@ -312,6 +312,11 @@ typedef struct t3_moe_plan {
     uint32_t item_rows, max_items;                           /* prefill: rows a GEMM item, items at most */
     uint64_t expert_code_bytes;  /* one expert's three matrices */
     size_t workspace_bytes;
+    /* prefill: where the route's arrays sit in the workspace (byte offsets; the roles of src/hip/plan.zig:40-45), for a
+     * host that reads the routing back: order u32 [row_slots] position -> row-slot; inv u32 [row_slots] row-slot ->
+     * position (~0: skipped); items u32 [max_items][4] {expert, first position, rows, 0}; counts u32 [E + S + 2]: rows an
+     * expert, then the item count, then the positions placed. 0 on the decode paths. */
+    size_t route_order_at, route_inv_at, route_items_at, route_counts_at;
 } t3_moe_plan;
 int32_t t3_moe_plan_of(const t3_array* x, const t3_bank* bank, const t3_array* inds, const t3_bank* shared_bank,
                        t3_moe_plan* plan);

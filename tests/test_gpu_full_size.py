@@ -237,3 +237,57 @@ def test_config4_routed_prefill_widths_mixed_rates(oracle, t3):
     y17 = t3.moe_clamped(x_dev[:17].reshape(1, 17, hidden), dbank, d_slots[:17].reshape(1, 17, topk),
                          d_scores[:17].reshape(1, 17, topk), t3.Decode.mcg, limit)
     assert bytes_of(y17[0]) == bytes_of(y[0, :17]), "rows 0-16 of 512 tokens differ from the 17-row call"
+
+
+def test_config4_routed_prefill_full_size(oracle, t3):
+    # config 4 as the benchmark runs it: 2048 tokens x 256 experts, top-8, 7168 / 2048, gate|up K2, down K3, bf16, clamp 7
+    # (a 3.3 GB bank, 16,384 routed positions, 96-row items). Sampled rows against ref.moeRowClamped (the reference samples
+    # rows the same way, src/core/prefill_test.zig:177-182), the first 17 rows' bytes against the 17-row call, and the
+    # route's integer work (rows an expert, items, placement) recounted on the host from the ids, to the bit.
+    experts, hidden, inter, topk, tokens, limit = 256, 7168, 2048, 8, 2048, 7
+    rng = np.random.default_rng(0xC4F)
+    bank = oracle.synth_bank(rng, experts, hidden, inter, 32, 48)
+    dbank = dev_bank(t3, bank)
+    x_dev, x_f32 = make_x(rng, tokens, hidden, torch.bfloat16)
+    slots, scores = routing_softmax(rng, tokens, topk, experts)
+    d_slots, d_scores = torch.from_numpy(slots).cuda(), torch.from_numpy(scores).cuda()
+    args = (x_dev.reshape(1, tokens, hidden), dbank, d_slots.reshape(1, tokens, topk))
+    plan = t3.moe_plan(*args)
+    assert (plan["path"], plan["item_rows"], plan["row_slots"]) == (3, 96, tokens * topk)
+    y = t3.moe_clamped(*args, d_scores.reshape(1, tokens, topk), t3.Decode.mcg, limit)
+    torch.cuda.synchronize()
+
+    # the route, read back from the workspace the call ran in
+    ws = t3._workspace(x_dev.device, 0)
+    p = tokens * topk
+
+    def words(at, count):
+        return ws[at:at + 4 * count].view(torch.int32).cpu().numpy().view(np.uint32)
+
+    counts = words(plan["route_counts_at"], experts + 2)
+    want_counts = np.bincount(slots.ravel(), minlength=experts).astype(np.uint32)
+    assert np.array_equal(counts[:experts], want_counts), "rows an expert"
+    want_items, pos = [], 0
+    for e in range(experts):
+        c = int(want_counts[e])
+        want_items += [(e, pos + i, min(96, c - i)) for i in range(0, c, 96)]
+        pos += c
+    assert counts[experts] == len(want_items) and counts[experts + 1] == p, "item count and positions placed"
+    items = words(plan["route_items_at"], 4 * len(want_items)).reshape(-1, 4)
+    assert [tuple(int(v) for v in it[:3]) for it in items] == want_items, "items: expert, first position, rows"
+    order, inv = words(plan["route_order_at"], p), words(plan["route_inv_at"], p)
+    assert np.array_equal(np.sort(order), np.arange(p, dtype=np.uint32)), "order is a permutation of the row-slots"
+    assert np.array_equal(order[inv], np.arange(p, dtype=np.uint32)), "inv inverts order"
+    starts = np.concatenate([[0], np.cumsum(want_counts)]).astype(np.int64)
+    for e in (0, 1, 100, experts - 1):  # an expert's run of positions holds exactly its row-slots
+        run = order[starts[e]:starts[e + 1]]
+        assert (slots.ravel()[run] == e).all()
+
+    got = to_f32(y).reshape(tokens, hidden)
+    for r in (0, 1023, tokens - 1):
+        ref = RefBank(oracle, bank, MCG, 0xFFFF)  # a fresh cache a row: an expert's three W_hat are 88 MB
+        e = oracle.compare(got[r], ref.row(x_f32[r], slots[r], scores[r], float(limit)))
+        assert e <= BF16_MOE_BAR, f"row {r}: {e:.3e}"
+    y17 = t3.moe_clamped(x_dev[:17].reshape(1, 17, hidden), dbank, d_slots[:17].reshape(1, 17, topk),
+                         d_scores[:17].reshape(1, 17, topk), t3.Decode.mcg, limit)
+    assert bytes_of(y17[0]) == bytes_of(y[0, :17]), "rows 0-16 of 2048 tokens differ from the 17-row call"

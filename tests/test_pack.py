@@ -68,15 +68,20 @@ def test_pack_claims_validation_and_bill(oracle, tmp_path):
 
 @pytest.mark.gpu
 def test_pack_loads_and_runs(oracle, tmp_path):
-    from tests.gpu_util import MCG, bytes_of, dev_f16_bits, dev_u16, make_x
+    from tests.gpu_util import MCG, bytes_of, dev_f16_bits, dev_u16, make_x, to_f32
     from turboexl3_amd import api as t3
     from turboexl3_amd import pack, table
     rng = np.random.default_rng(4)
     (tr, suh, svh), bank = write_pack(str(tmp_path), oracle, rng)
     p = pack.Pack(str(tmp_path))
     w = p.linear("model.layers.0.attn.q_proj", in_dim=512)
-    x, _ = make_x(rng, 3, 512, torch.bfloat16)
-    assert bytes_of(table.matmul(w, x)) == bytes_of(t3.linear(x, dev_u16(tr), dev_f16_bits(suh), dev_f16_bits(svh), t3.Decode.mcg))
+    x, x_f32 = make_x(rng, 3, 512, torch.bfloat16)
+    y = table.matmul(w, x)
+    assert bytes_of(y) == bytes_of(t3.linear(x, dev_u16(tr), dev_f16_bits(suh), dev_f16_bits(svh), t3.Decode.mcg))
+    # what the pack's tensors came to on the device, against format.project on the arrays the pack was written from
+    ref = oracle.project_rows(x_f32, tr, suh, svh, 512, tr.shape[1] * 16, tr.shape[2], MCG, 0xFFFF)
+    for r in range(3):
+        assert oracle.compare(to_f32(y)[r], ref[r], 2.0 ** -8) <= 2.5e-2, r
     with pytest.raises(table.Refused) as e:
         p.linear("model.layers.0.attn.k_proj")
     assert (e.value.kind, e.value.why) == ("failed", "MissingWeight")
@@ -87,4 +92,8 @@ def test_pack_loads_and_runs(oracle, tmp_path):
     dev = lambda t, a, b: t3.Proj(dev_u16(t), dev_f16_bits(a), dev_f16_bits(b))
     tbank = t3.Bank(dev(bank.gate_t, bank.gate_suh, bank.gate_svh), dev(bank.up_t, bank.up_suh, bank.up_svh),
                     dev(bank.down_t, bank.down_suh, bank.down_svh))
-    assert bytes_of(table.swiglu(g, u, d, x3, inds, scores)) == bytes_of(t3.moe(x3, tbank, inds, scores, t3.Decode.mcg))
+    y3 = table.swiglu(g, u, d, x3, inds, scores)
+    assert bytes_of(y3) == bytes_of(t3.moe(x3, tbank, inds, scores, t3.Decode.mcg))
+    for r in range(3):
+        want, _ = oracle.moe_row(bank, x_f32[r], inds[0, r].cpu().numpy(), scores[0, r].cpu().numpy(), MCG, 0xFFFF, 0.0)
+        assert oracle.compare(to_f32(y3)[0, r], want, 2.0 ** -8) <= 1.5e-2, r

@@ -10,6 +10,7 @@ struct MoeCall {
     MoeLaunch launch;
     size_t workspace = 0;
     int64_t rows = 0;
+    size_t order_at = 0, inv_at = 0, items_at = 0, counts_at = 0;  // prefill: the route's arrays inside the workspace
 };
 
 // One projection's arrays against the geometry (src/root.zig:87-102).
@@ -170,9 +171,13 @@ void carve_moe_prefill(MoeCall* call, void* workspace) {
     l.zg = c.take<float>(p * l.inter * 4u);
     l.zu = c.take<float>(p * l.inter * 4u);
     l.zd = c.take<float>(p * l.hidden * 4u);
+    call->order_at = c.used;
     l.order = c.take<uint32_t>(p * 4u);
+    call->inv_at = c.used;
     l.inv = c.take<uint32_t>(p * 4u);
+    call->items_at = c.used;
     l.items = c.take<uint32_t>(static_cast<size_t>(l.max_items) * 16u);
+    call->counts_at = c.used;
     l.counts = c.take<uint32_t>((et + 4u) * 4u);
     l.cursor = c.take<uint32_t>(et * 4u);
     call->workspace = c.used;
@@ -267,6 +272,10 @@ int32_t t3_moe_plan_of(const t3_array* x, const t3_bank* bank, const t3_array* i
         p.launches = 9;
         p.item_rows = l.item_rows;
         p.max_items = l.max_items;
+        p.route_order_at = call.order_at;
+        p.route_inv_at = call.inv_at;
+        p.route_items_at = call.items_at;
+        p.route_counts_at = call.counts_at;
     } else {
         t3::carve_moe(&call, nullptr);
         const int form = t3::decode_form_of(l);
