@@ -1,25 +1,30 @@
 #!/usr/bin/env python3
 """Benchmark of the EXL3 projection path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sweep]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick] [--no-cpu]
 
 A step is one `linear` call of the dense decode-row GEMV workload the headline metric is quoted on
 (in=4096, out=12288, K=4 bits/weight, 1 row, MCG codebook, f16 activations with 1 % outliers x20; synthetic seeded
 codes). Calls rotate over enough distinct weight copies (> 512 MB in total) that every call reads its codes from
-HBM, not from the 256 MB Infinity Cache. Inputs are resident in HBM before the timed region starts.
+HBM, not from the 256 MB Infinity Cache. Inputs are resident in HBM before the timed region starts. Every timing
+captures its calls once into a HIP graph and brackets a replay with events on the launch stream.
 
-Prints ONE JSON line: the whole-call rate as GB/s of trellis code bytes (`value`), the dominant kernel's roofline
-(`roofline`: algorithmic code bytes of one launch / its average duration, timed alone with HIP events on the launch
-stream, against 8 TB/s), and the CPU oracle (`format.project` restated in C) timed on this box's host cores
-(`cpu_baseline`). The same line carries the other benchmark configurations as extra objects: `moe_decode`
-(config 3: routed decode at 1 and 8 tokens), `moe_prefill` (config 4: the routed prefill chain, TFLOP/s against the
-2.5 PFLOP/s dense f16 MFMA peak) and `dense_prefill` (config 5: 4096 rows); `--quick` leaves them out. `--sweep` adds
-K = 3, 4, 5 x rows = 1, 4, 16, 32; `--in-f/--out-f/--k/--rows` time another dense shape (lm_head: --in-f 4096
---out-f 151936 --k 6).
+Prints ONE JSON line. `value`: the whole call's rate as GB/s of trellis code bytes. `roofline`: the kernel that call
+launches (one launch at one row: the call's time is that kernel's), its algorithmic code bytes over its duration
+against 8 TB/s; `gemv_launch_alone` is the chain's GEMV launch without prepare and finish, for comparison. Beside
+them, unless --quick: `sweep` (the metric's K = 3, 4, 5 x rows = 1, 4, 16, 32), `lm_head` (4096 -> 151936 at K6, 1 and
+256 rows), `moe_decode` (config 3 at 1 and 8 tokens, each launch timed alone as well), `moe_prefill` (config 4, each
+stage timed alone; TFLOP/s against the 2.5 PFLOP/s f16 MFMA figure and against a dense f16 GEMM measured in this
+process, `measured_dense_f16_peak`), `dense_prefill` (config 5's 4096 rows and its resident-weight forms),
+`codebook_forms` (the price of exact f16 weights in the GEMV), `rates` (a fractional narrow rate and a wide one) and
+`dense_rows` (few-row dense calls with and without the rows-alone partition). `cpu_baseline`: the CPU oracle
+(`format.project` restated in C) timed on this box's host cores, and, in the same leg, one sampled output block (or row)
+of every timed cell held against the oracle by the reference's bars (`parity_checks`).
 """
 from __future__ import annotations
 
 import argparse
+import ctypes as C
 import json
 import os
 import sys
@@ -32,10 +37,14 @@ sys.path.insert(0, ROOT)
 
 IN_F, OUT_F = 4096, 12288
 HBM_PEAK = 8.0e12
+MFMA_F16_PEAK = 2.5e15
 MIN_ROTATION_BYTES = 512 << 20
-# HBM bytes one chain-GEMV launch moves, from the profiler's FETCH_SIZE and WRITE_SIZE counters scaled by a 256 MiB
-# copy (profiles/dense_gemv_in4096_out12288_k4_rows1.txt): keyed by (in, out, K, rows); other workloads report null
-MEASURED_TRAFFIC = {(4096, 12288, 4, 1): 25_762_406}
+# HBM bytes one launch of the served one-row kernel moves, from the profiler's FETCH_SIZE and WRITE_SIZE counters scaled
+# by a 256 MiB copy (profiles/dense_gemv_in4096_out12288_k4_rows1.txt): keyed by (in, out, n, rows); others report null
+MEASURED_TRAFFIC = {(4096, 12288, 64, 1): 25_762_406}
+F32_BAR, BF16_DENSE_BAR, BF16_MOE_BAR = 5e-3, 2.5e-2, 1.5e-2
+
+MCG_CB, MUL1_CB = 1, 0
 
 
 def code_bytes(in_f: int, out_f: int, n: int) -> int:
@@ -43,206 +52,239 @@ def code_bytes(in_f: int, out_f: int, n: int) -> int:
     return (in_f // 16) * (out_f // 16) * n * 2
 
 
-def make_weights(torch, n: int, copies: int, seed: int):
-    g = torch.Generator(device="cuda")
-    g.manual_seed(seed)
-    trellis = torch.randint(-32768, 32768, (copies, IN_F // 16, OUT_F // 16, n), dtype=torch.int16, device="cuda",
-                            generator=g)
-    sign = lambda k: (torch.randint(0, 2, (k,), device="cuda", generator=g) * 2 - 1).to(torch.float32)
-    suh = (sign(IN_F) * (1.0 + 0.1 * torch.randn(IN_F, device="cuda", generator=g))).to(torch.float16)
-    svh = (sign(OUT_F) * (1.0 + 0.1 * torch.randn(OUT_F, device="cuda", generator=g)) / (IN_F ** 0.5)).to(torch.float16)
-    return trellis, suh, svh
+def graph_time(torch, call, steps: int, warmup: int) -> float:
+    """Seconds a call over exactly `steps` back-to-back calls `call(i, stream)`, captured once into a HIP graph (as a
+    serving loop would hold its decode step) so the host's per-launch cost stays out of the GPU's timeline; events
+    bracket one replay on the launch stream."""
+    cur = torch.cuda.current_stream().cuda_stream
+    for i in range(max(warmup, 1)):
+        call(i, cur)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(steps):
+                call(warmup + i, side.cuda_stream)
+        torch.cuda.synchronize()
+        graph.replay()  # untimed: the graph's first replay uploads it
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(side)
+        graph.replay()
+        e1.record(side)
+        torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / steps
 
 
-def make_x(torch, rows: int, seed: int):
-    g = torch.Generator(device="cuda")
-    g.manual_seed(seed)
-    x = torch.randn(rows, IN_F, device="cuda", generator=g)
-    outl = torch.rand(rows, IN_F, device="cuda", generator=g) < 0.01
-    return torch.where(outl, x * 20.0, x).to(torch.float16)
+def host_u16(t) -> np.ndarray:
+    import torch
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
 
 
-class DenseRunner:
-    """Pre-built descriptors for back-to-back C-ABI calls: nothing is allocated inside the timed region."""
+class Dense:
+    """One dense shape at one rate: rotating weight copies, descriptors built once, nothing allocated while timing."""
 
-    def __init__(self, torch, api, trellis, suh, svh, x, dec):
-        import ctypes as C
-
+    def __init__(self, torch, api, in_f, out_f, n, codebook, max_rows, act_dtype, seed, copies=None, outliers=True):
         from turboexl3_amd import _lib
-        self.C, self.L, self.torch = C, _lib.lib(), torch
-        self.copies = trellis.shape[0]
-        self.dec = dec.c()
-        self.ax = api._arr(x)
-        self.at = [api._arr(trellis[i]) for i in range(self.copies)]
-        self.asu, self.asv = api._arr(suh), api._arr(svh)
-        self.y = torch.empty(x.shape[0], OUT_F, dtype=x.dtype, device="cuda")
+        self.torch, self.api, self.L = torch, api, _lib.lib()
+        self.in_f, self.out_f, self.n, self.codebook = in_f, out_f, n, codebook
+        self.dec = api.Decode(codebook, 16)
+        self.cb = code_bytes(in_f, out_f, n)
+        self.copies = copies or (-(-MIN_ROTATION_BYTES // self.cb) + 1)
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+        self.trellis = torch.randint(-32768, 32768, (self.copies, in_f // 16, out_f // 16, n), dtype=torch.int16,
+                                     device="cuda", generator=g)
+        sign = lambda k: (torch.randint(0, 2, (k,), device="cuda", generator=g) * 2 - 1).to(torch.float32)
+        self.suh = (sign(in_f) * (1.0 + 0.1 * torch.randn(in_f, device="cuda", generator=g))).to(torch.float16)
+        self.svh = (sign(out_f) * (1.0 + 0.1 * torch.randn(out_f, device="cuda", generator=g)) / (in_f ** 0.5)).to(torch.float16)
+        x = torch.randn(max_rows, in_f, device="cuda", generator=g)
+        if outliers:
+            x = torch.where(torch.rand(max_rows, in_f, device="cuda", generator=g) < 0.01, x * 20.0, x)
+        self.x = x.to(act_dtype)
+        self.at = [api._arr(self.trellis[i]) for i in range(self.copies)]
+        self.asu, self.asv = api._arr(self.suh), api._arr(self.svh)
+        self.ws = None
+
+    def bind(self, rows: int):
+        api = self.api
+        self.rows = rows
+        self.xr = self.x[:rows]
+        self.ax = api._arr(self.xr)
+        self.y = self.torch.empty(rows, self.out_f, dtype=self.x.dtype, device="cuda")
         self.ay = api._arr(self.y)
         need = C.c_size_t(0)
-        st = self.L.t3_linear_workspace_bytes(C.byref(self.ax), C.byref(self.at[0]), self.dec, C.byref(need))
-        assert st == 0, _lib.error_name(st)
-        self.ws = torch.zeros(need.value, dtype=torch.uint8, device="cuda")
-        self.stream = torch.cuda.current_stream().cuda_stream
+        st = self.L.t3_linear_workspace_bytes(C.byref(self.ax), C.byref(self.at[0]), self.dec.c(), C.byref(need))
+        assert st == 0, self.L.t3_error_name(st).decode()
+        if self.ws is None or self.ws.numel() < need.value:
+            self.ws = self.torch.zeros(need.value, dtype=self.torch.uint8, device="cuda")
+        self.plan = api.linear_plan(self.xr, self.trellis[0], self.dec)
 
-    def call(self, i: int, stages: int = 0):
-        C = self.C
+    def call(self, i: int, stream: int, stages: int = 0):
         t = self.at[i % self.copies]
+        dec = self.dec.c()
         if stages:
-            st = self.L.t3_linear_stages(self.stream, C.byref(self.ax), C.byref(t), C.byref(self.asu), C.byref(self.asv),
-                                         self.dec, C.byref(self.ay), self.ws.data_ptr(), self.ws.numel(), stages)
+            st = self.L.t3_linear_stages(stream, C.byref(self.ax), C.byref(t), C.byref(self.asu), C.byref(self.asv), dec,
+                                         C.byref(self.ay), self.ws.data_ptr(), self.ws.numel(), stages)
         else:
-            st = self.L.t3_linear(self.stream, C.byref(self.ax), C.byref(t), C.byref(self.asu), C.byref(self.asv),
-                                  self.dec, C.byref(self.ay), self.ws.data_ptr(), self.ws.numel())
+            st = self.L.t3_linear(stream, C.byref(self.ax), C.byref(t), C.byref(self.asu), C.byref(self.asv), dec,
+                                  C.byref(self.ay), self.ws.data_ptr(), self.ws.numel())
         if st != 0:
             raise RuntimeError(self.L.t3_error_name(st).decode())
 
-    def time(self, steps: int, warmup: int, stages: int = 0) -> float:
-        """Seconds per call over exactly `steps` back-to-back calls. The calls are captured once into a HIP graph
-        (as a serving loop would hold its decode step) so the host's per-launch cost stays out of the GPU's
-        timeline; events bracket the replay on the launch stream."""
+    def sample(self, name: str, blk: int, rows_to_check, bar: float, half_ulp: float):
+        """One eager call over copy 0, and what the CPU leg needs to hold output columns [128 blk, 128 blk + 128) of the
+        chosen rows against format.project."""
         torch = self.torch
-        for i in range(max(warmup, 1)):
-            self.call(i, stages)
+        self.call(0, torch.cuda.current_stream().cuda_stream)
         torch.cuda.synchronize()
-        side = torch.cuda.Stream()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.stream(side):
-            self.stream = side.cuda_stream
-            with torch.cuda.graph(graph, stream=side):
-                for i in range(steps):
-                    self.call(warmup + i, stages)
-            torch.cuda.synchronize()
-            graph.replay()  # untimed: the graph's first replay uploads it
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(side)
-            graph.replay()
-            e1.record(side)
-            torch.cuda.synchronize()
-        self.stream = torch.cuda.current_stream().cuda_stream
-        return e0.elapsed_time(e1) * 1e-3 / steps
+        rows_to_check = sorted(set(rows_to_check))
+        return {"kind": "dense", "cell": name, "in_f": self.in_f, "n": self.n, "codebook": self.codebook, "bar": bar,
+                "half_ulp": half_ulp, "rows": rows_to_check,
+                "trellis": host_u16(self.trellis[0][:, 8 * blk:8 * blk + 8, :]), "suh": host_u16(self.suh.view(torch.int16)),
+                "svh": host_u16(self.svh[128 * blk:128 * blk + 128].view(torch.int16)),
+                "x": self.xr[rows_to_check].to(torch.float32).cpu().numpy(),
+                "y": self.y[rows_to_check, 128 * blk:128 * blk + 128].to(torch.float32).cpu().numpy()}
+
+    def time(self, steps: int, warmup: int, stages: int = 0) -> float:
+        return graph_time(self.torch, lambda i, s: self.call(i, s, stages), steps, warmup)
 
 
-class MoeRunner:
-    """Benchmark configuration 3: 512 experts, hidden 2048, inter 512, K3, top-10, clamp 7, one shared expert (inter 512) in the
-    same launches. Every call routes to a fresh set of experts (a rotation of disjoint routings) so the codes come from
-    HBM: the bank alone is 604 MB."""
+def dense_cell(d: Dense, rows: int, steps: int, warmup: int, todo: list, name: str, gemv_alone: bool = False) -> dict:
+    import torch
+    d.bind(rows)
+    bf16 = d.x.dtype == torch.bfloat16
+    todo.append(d.sample(name, blk=(d.out_f // 128) // 3, rows_to_check=[0, rows - 1],
+                         bar=BF16_DENSE_BAR if bf16 else F32_BAR, half_ulp=2.0 ** -8 if bf16 else 2.0 ** -11))
+    t = d.time(steps, warmup)
+    out = {"n": d.n, "k": d.n / 16, "rows": rows, "code_bytes": d.cb, "copies": d.copies, "us_per_call": t * 1e6,
+           "call_gbps": d.cb / t / 1e9, "frac_of_hbm": d.cb / t / HBM_PEAK,
+           "plan": {key: d.plan[key] for key in ("path", "launches", "tiles_a_load", "k_slices", "tiles_a_wave", "workgroups")}}
+    if gemv_alone and rows <= 32:
+        tg = d.time(steps, warmup, stages=2)
+        out.update({"gemv_us": tg * 1e6, "gemv_gbps": d.cb / tg / 1e9, "gemv_frac_of_hbm": d.cb / tg / HBM_PEAK})
+    return out
 
-    E, HIDDEN, INTER, K, TOPK, LIMIT = 512, 2048, 512, 3, 10, 7
 
-    def __init__(self, torch, api, tokens: int, seed: int = 5):
-        import ctypes as C
+class Moe:
+    """A routed call over a synthetic bank: config 3 (decode rows, a shared expert in the same launches, rotating routings
+    so every call reads fresh experts from HBM) or config 4 (prefill)."""
 
+    def __init__(self, torch, api, experts, hidden, inter, k_gu, k_dn, topk, tokens, limit, shared: bool, sets: int, seed: int):
         from turboexl3_amd import _lib
-        self.C, self.L, self.torch, self.api = C, _lib.lib(), torch, api
+        self.torch, self.api, self.L = torch, api, _lib.lib()
+        self.E, self.hidden, self.inter, self.topk, self.tokens, self.limit = experts, hidden, inter, topk, tokens, limit
+        self.n_gu, self.n_dn = 16 * k_gu, 16 * k_dn
         g = torch.Generator(device="cuda")
         g.manual_seed(seed)
-        n = 16 * self.K
 
-        def proj(experts, in_f, out_f):
-            t = torch.randint(-32768, 32768, (experts, in_f // 16, out_f // 16, n), dtype=torch.int16, device="cuda",
-                              generator=g)
-            suh = (0.5 + torch.rand(experts, in_f, device="cuda", generator=g)).to(torch.float16)
-            svh = ((0.5 + torch.rand(experts, out_f, device="cuda", generator=g)) / in_f ** 0.5).to(torch.float16)
+        def proj(e, in_f, out_f, n):
+            t = torch.randint(-32768, 32768, (e, in_f // 16, out_f // 16, n), dtype=torch.int16, device="cuda", generator=g)
+            suh = (0.5 + torch.rand(e, in_f, device="cuda", generator=g)).to(torch.float16)
+            svh = ((0.5 + torch.rand(e, out_f, device="cuda", generator=g)) / in_f ** 0.5).to(torch.float16)
             return api.Proj(t, suh, svh)
 
-        def bank(experts):
-            return api.Bank(proj(experts, self.HIDDEN, self.INTER), proj(experts, self.HIDDEN, self.INTER),
-                            proj(experts, self.INTER, self.HIDDEN))
+        def bank(e):
+            return api.Bank(proj(e, hidden, inter, self.n_gu), proj(e, hidden, inter, self.n_gu), proj(e, inter, hidden, self.n_dn))
 
-        self.bank, self.shared = bank(self.E), bank(1)
-        self.tokens = tokens
-        self.x = torch.randn(1, tokens, self.HIDDEN, device="cuda", generator=g).to(torch.bfloat16)
+        self.bank = bank(experts)
+        self.shared = bank(1) if shared else None
+        self.x = torch.randn(1, tokens, hidden, device="cuda", generator=g).to(torch.bfloat16)
         # router logits ~ N(0,1) -> top-k -> softmax over the selected (harness side, as in the reference's benches)
-        self.sets = 24
-        logits = torch.randn(self.sets, tokens, self.E, device="cuda", generator=g)
-        top = torch.topk(logits, self.TOPK, dim=-1)
+        self.sets = sets
+        logits = torch.randn(sets, tokens, experts, device="cuda", generator=g)
+        top = torch.topk(logits, topk, dim=-1)
         self.inds = top.indices.to(torch.int32).contiguous()
         self.scores = torch.softmax(top.values, dim=-1).to(torch.float32).contiguous()
         self.cb, self._k1 = api._cbank(self.bank)
-        self.sb, self._k2 = api._cbank(self.shared)
+        self.sb, self._k2 = api._cbank(self.shared) if shared else (None, None)
         self.ax = api._arr(self.x)
-        self.ai = [api._arr(self.inds[i:i + 1]) for i in range(self.sets)]
-        self.asc = [api._arr(self.scores[i:i + 1]) for i in range(self.sets)]
+        self.ai = [api._arr(self.inds[i:i + 1]) for i in range(sets)]
+        self.asc = [api._arr(self.scores[i:i + 1]) for i in range(sets)]
         self.y = torch.empty_like(self.x)
         self.ay = api._arr(self.y)
         need = C.c_size_t(0)
-        st = self.L.t3_moe_workspace_bytes(C.byref(self.ax), C.byref(self.cb), C.byref(self.ai[0]), C.byref(self.sb),
-                                           C.byref(need))
-        assert st == 0, _lib.error_name(st)
+        sbp = C.byref(self.sb) if shared else None
+        st = self.L.t3_moe_workspace_bytes(C.byref(self.ax), C.byref(self.cb), C.byref(self.ai[0]), sbp, C.byref(need))
+        assert st == 0, self.L.t3_error_name(st).decode()
         self.ws = torch.zeros(need.value, dtype=torch.uint8, device="cuda")
-        self.dec = api.Decode.mcg.c()
-        self.stream = torch.cuda.current_stream().cuda_stream
-        per_expert = 3 * (self.HIDDEN // 16) * (self.INTER // 16) * n * 2
-        distinct = [len(set(self.inds[i].flatten().tolist())) for i in range(self.sets)]
-        self.code_bytes = (sum(distinct) / self.sets + 1) * per_expert  # + the shared expert
-
-    def call(self, i: int, stages: int = 0):
-        C = self.C
-        j = i % self.sets
-        st = self.L.t3_moe_shared_expert(self.stream, C.byref(self.ax), C.byref(self.cb), C.byref(self.ai[j]),
-                                         C.byref(self.asc[j]), self.dec, self.LIMIT, C.byref(self.sb), C.byref(self.ay),
-                                         self.ws.data_ptr(), self.ws.numel())
-        if st != 0:
-            raise RuntimeError(self.L.t3_error_name(st).decode())
-
-    time = DenseRunner.time
-
-
-class PrefillRunner:
-    """Benchmark configuration 4: 2048 tokens, 256 experts, top-8, hidden 7168, inter 2048, gate|up K2, down K3, bf16, clamp 7.
-    flops = tokens * topk * 3 * 2 * hidden * inter. `scale` shrinks experts and tokens together (same rows an expert)."""
-
-    def __init__(self, torch, api, tokens=2048, experts=256, topk=8, hidden=7168, inter=2048, k_gu=2, k_dn=3, seed=9):
-        import ctypes as C
-
-        from turboexl3_amd import _lib
-        self.C, self.L, self.torch, self.api = C, _lib.lib(), torch, api
-        g = torch.Generator(device="cuda")
-        g.manual_seed(seed)
-
-        def proj(in_f, out_f, k):
-            t = torch.randint(-32768, 32768, (experts, in_f // 16, out_f // 16, 16 * k), dtype=torch.int16,
-                              device="cuda", generator=g)
-            suh = (0.5 + torch.rand(experts, in_f, device="cuda", generator=g)).to(torch.float16)
-            svh = ((0.5 + torch.rand(experts, out_f, device="cuda", generator=g)) / in_f ** 0.5).to(torch.float16)
-            return api.Proj(t, suh, svh)
-
-        self.bank = api.Bank(proj(hidden, inter, k_gu), proj(hidden, inter, k_gu), proj(inter, hidden, k_dn))
-        self.x = torch.randn(1, tokens, hidden, device="cuda", generator=g).to(torch.bfloat16)
-        logits = torch.randn(tokens, experts, device="cuda", generator=g)
-        top = torch.topk(logits, topk, dim=-1)
-        self.inds = top.indices.to(torch.int32).reshape(1, tokens, topk).contiguous()
-        self.scores = torch.softmax(top.values, dim=-1).to(torch.float32).reshape(1, tokens, topk).contiguous()
-        self.cb, self._k1 = api._cbank(self.bank)
-        self.ax, self.ai, self.asc = api._arr(self.x), api._arr(self.inds), api._arr(self.scores)
-        self.y = torch.empty_like(self.x)
-        self.ay = api._arr(self.y)
-        need = C.c_size_t(0)
-        st = self.L.t3_moe_workspace_bytes(C.byref(self.ax), C.byref(self.cb), C.byref(self.ai), None, C.byref(need))
-        assert st == 0, _lib.error_name(st)
-        self.ws = torch.zeros(need.value, dtype=torch.uint8, device="cuda")
-        self.dec = api.Decode.mcg.c()
-        self.stream = torch.cuda.current_stream().cuda_stream
+        self.dec = api.Decode.mcg
+        self.per_expert = code_bytes(hidden, inter, self.n_gu) * 2 + code_bytes(inter, hidden, self.n_dn)
+        distinct = [len(set(self.inds[i].flatten().tolist())) for i in range(sets)]
+        self.distinct = sum(distinct) / sets + (1 if shared else 0)
         self.flops = tokens * topk * 3 * 2 * hidden * inter
-        self.code_bytes = experts * (2 * code_bytes_of(hidden, inter, 16 * k_gu) + code_bytes_of(inter, hidden, 16 * k_dn))
+        self.plan = api.moe_plan(self.x, self.bank, self.inds[0:1], self.shared)
 
-    def call(self, i: int, stages: int = 0):
-        C = self.C
-        st = self.L.t3_moe_clamped(self.stream, C.byref(self.ax), C.byref(self.cb), C.byref(self.ai), C.byref(self.asc),
-                                   self.dec, 7, C.byref(self.ay), self.ws.data_ptr(), self.ws.numel())
+    def call(self, i: int, stream: int, stages: int = 63):
+        j = i % self.sets
+        sbp = C.byref(self.sb) if self.sb is not None else None
+        st = self.L.t3_moe_stages(stream, C.byref(self.ax), C.byref(self.cb), C.byref(self.ai[j]), C.byref(self.asc[j]),
+                                  self.dec.c(), self.limit, sbp, C.byref(self.ay), self.ws.data_ptr(), self.ws.numel(), stages)
         if st != 0:
             raise RuntimeError(self.L.t3_error_name(st).decode())
 
-    time = DenseRunner.time
+    def time(self, steps: int, warmup: int, stages: int = 63) -> float:
+        return graph_time(self.torch, lambda i, s: self.call(i, s, stages), steps, warmup)
+
+    def sample(self, name: str, token: int, bar: float):
+        """One eager call over routing 0, and the chosen token's experts for ref.moeRowClamped on the host."""
+        torch = self.torch
+        self.call(0, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        ids = self.inds[0, token].tolist()
+        side = lambda t, sh: np.stack([host_u16(t[e].view(torch.int16)) for e in ids] +
+                                      ([host_u16(sh[0].view(torch.int16))] if self.shared else []))
+        b, s = self.bank, self.shared
+        arrays = {}
+        for nm in ("gate", "up", "down"):
+            p, q = getattr(b, nm), getattr(s, nm) if s else None
+            arrays[nm + "_t"] = np.stack([host_u16(p.trellis[e]) for e in ids] + ([host_u16(q.trellis[0])] if s else []))
+            arrays[nm + "_suh"] = side(p.suh, q.suh if s else None)
+            arrays[nm + "_svh"] = side(p.svh, q.svh if s else None)
+        scores = self.scores[0, token].tolist() + ([1.0] if s else [])
+        return {"kind": "moe", "cell": name, "hidden": self.hidden, "inter": self.inter, "n_gu": self.n_gu, "n_dn": self.n_dn,
+                "limit": float(self.limit), "bar": bar, "arrays": arrays, "scores": np.asarray(scores, dtype=np.float32),
+                "x": self.x[0, token].to(torch.float32).cpu().numpy(), "y": self.y[0, token].to(torch.float32).cpu().numpy()}
 
 
-def code_bytes_of(in_f: int, out_f: int, n: int) -> int:
-    return (in_f // 16) * (out_f // 16) * n * 2
+def measured_f16_peak(torch) -> dict:
+    """A plain dense f16 GEMM (8192^3, the library GEMM torch dispatches to) in this process: the matrix cores' practical
+    rate on this GPU at its sustained clock, beside the 2.5 PFLOP/s figure."""
+    m = 8192
+    a = torch.randn(m, m, device="cuda", dtype=torch.float16)
+    b = torch.randn(m, m, device="cuda", dtype=torch.float16)
+    for _ in range(3):
+        torch.matmul(a, b)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    reps = 10
+    for _ in range(reps):
+        torch.matmul(a, b)
+    e1.record()
+    torch.cuda.synchronize()
+    t = e0.elapsed_time(e1) * 1e-3 / reps
+    return {"tflops": 2 * m ** 3 / t / 1e12, "shape": f"{m} x {m} x {m} f16, f32 accumulate", "ms": t * 1e3,
+            "frac_of_2.5_pflops": 2 * m ** 3 / t / MFMA_F16_PEAK}
 
 
-def cpu_baseline(n: int, seed: int, budget_s: float = 20.0):
-    """format.project (the C oracle) on the host: the same shape and seeded distributions, one row, one thread,
-    re-decoding every tile as the reference does. A bounded sample: whole calls until ~budget_s is spent."""
+def eager_time(torch, fn, reps: int = 5) -> float:
+    fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / reps
+
+
+def cpu_leg(n: int, seed: int, todo: list, budget_s: float = 20.0):
+    """The only place this program touches the CPU oracle. (1) format.project (the C restatement) timed on the host: the
+    headline workload's shape and seeded distributions, one row, one thread, re-decoding every tile as the reference does;
+    a bounded sample: whole calls until ~budget_s is spent. (2) The sampled outputs of the timed cells held against it."""
     from oracle import oracle
     rng = np.random.default_rng(seed)
     trellis, suh, svh = oracle.synth_linear(rng, IN_F, OUT_F, n)
@@ -255,12 +297,11 @@ def cpu_baseline(n: int, seed: int, budget_s: float = 20.0):
         oracle.project(x, trellis, suh, svh, IN_F, OUT_F, n, oracle.MCG)
         times.append(time.perf_counter() - t0)
     med = float(np.median(times))
-    cores = os.cpu_count() or 1
-    threads = min(cores, 16)
+    threads = min(os.cpu_count() or 1, 16)
     t0 = time.perf_counter()
     oracle.project_rows(x[None, :], trellis, suh, svh, IN_F, OUT_F, n, oracle.MCG, threads=threads)
     par = time.perf_counter() - t0
-    return {
+    base = {
         "value": code_bytes(IN_F, OUT_F, n) / med / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
         "sample": f"{len(times)} whole calls of the same workload (in={IN_F}, out={OUT_F}, n={n}, 1 row), median "
                   f"{med * 1e3:.1f} ms a call; scalar single thread as the reference's format.project",
@@ -268,6 +309,21 @@ def cpu_baseline(n: int, seed: int, budget_s: float = 20.0):
         "all_cores": {"value": code_bytes(IN_F, OUT_F, n) / par / 1e9, "unit": "GB/s", "threads": threads,
                       "note": "decode-once + OpenMP over output blocks, same bits"},
     }
+    checks = []
+    for s in todo:
+        if s["kind"] == "dense":
+            ref = oracle.project_rows(s["x"], s["trellis"], s["suh"], s["svh"], s["in_f"], 128, s["n"], s["codebook"], 0xFFFF,
+                                      threads=threads)
+            err = max(oracle.compare(s["y"][i], ref[i], s["half_ulp"]) for i in range(len(s["rows"])))
+        else:
+            a = s["arrays"]
+            bank = oracle.Bank(a["gate_t"].shape[0], s["hidden"], s["inter"], s["n_gu"], s["n_dn"], a["gate_t"], a["gate_suh"],
+                               a["gate_svh"], a["up_t"], a["up_suh"], a["up_svh"], a["down_t"], a["down_suh"], a["down_svh"])
+            want, _ = oracle.moe_row(bank, s["x"], np.arange(len(s["scores"]), dtype=np.int32), s["scores"], oracle.MCG,
+                                     0xFFFF, s["limit"])
+            err = oracle.compare(s["y"], want, 2.0 ** -8)
+        checks.append({"cell": s["cell"], "err_over_rms": err, "bar": s["bar"], "ok": bool(err <= s["bar"])})
+    return base, checks
 
 
 def main() -> int:
@@ -275,32 +331,30 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--sweep", action="store_true", help="also time K = 3, 4, 5 x rows = 1, 4, 16, 32")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU leg (the oracle's timing and the parity checks)")
     ap.add_argument("--k", type=int, default=4)
     ap.add_argument("--rows", type=int, default=1)
-    ap.add_argument("--moe", action="store_true", help="(default on) time the routed-expert decode chain (config 3)")
-    ap.add_argument("--quick", action="store_true", help="the headline workload only: no routed or prefill timings")
-    ap.add_argument("--prefill", action="store_true",
-                    help="(default on) time the routed prefill chain (config 4) and the dense 4096-row projection "
-                         "(config 5)")
+    ap.add_argument("--quick", action="store_true", help="the headline workload only")
+    ap.add_argument("--only", default="", help="comma-separated sections to run beside the headline: sweep, forms, rates, "
+                                               "lm_head, moe_decode, moe_prefill, dense_prefill, dense_rows, peak")
+    ap.add_argument("--sweep", action="store_true", help="(default on) K = 3, 4, 5 x rows = 1, 4, 16, 32")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run one 256 MiB device copy, the known-size kernel that scales the profiler's "
                          "FETCH_SIZE / WRITE_SIZE readings")
-    ap.add_argument("--dense-rows", default="",
-                    help="comma-separated row counts above 32: time the dense projection --in-f x --out-f at --k on the "
-                         "trellis GEMM and on the W_hat form (dense_gemm_rows forced either way)")
     ap.add_argument("--in-f", type=int, default=4096)
     ap.add_argument("--out-f", type=int, default=12288)
     args = ap.parse_args()
     global IN_F, OUT_F
     IN_F, OUT_F = args.in_f, args.out_f
-    if not args.quick:
-        args.moe = args.prefill = True
     if args.gpus != 1:
         print(f"bench.py: this build measures one GPU (the path has no collective); --gpus {args.gpus} is not served",
               file=sys.stderr)
         return 2
+    sections = {"sweep", "forms", "rates", "lm_head", "moe_decode", "moe_prefill", "dense_prefill", "dense_rows", "peak"}
+    if args.quick:
+        sections = set()
+    elif args.only:
+        sections = set(args.only.split(","))
 
     import torch
 
@@ -309,23 +363,8 @@ def main() -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 2
     torch.cuda.set_device(0)
-    dec = api.Decode.mcg
-
-    def measure(k: int, rows: int, steps: int, warmup: int):
-        n = 16 * k
-        cb = code_bytes(IN_F, OUT_F, n)
-        copies = -(-MIN_ROTATION_BYTES // cb) + 1
-        trellis, suh, svh = make_weights(torch, n, copies, seed=1000 + k)
-        x = make_x(torch, rows, seed=7)
-        run = DenseRunner(torch, api, trellis, suh, svh, x, dec)
-        t_call = run.time(steps, warmup)
-        t_gemv = run.time(steps, warmup, stages=2)
-        plan = api.linear_plan(x, trellis[0], dec)
-        return {"k": k, "rows": rows, "code_bytes": cb, "copies": copies, "us_per_call": t_call * 1e6,
-                "plan": {key: plan[key] for key in ("path", "launches", "tiles_a_load", "k_slices", "tiles_a_wave",
-                                                    "workgroups")},
-                "call_gbps": cb / t_call / 1e9, "gemv_us": t_gemv * 1e6, "gemv_gbps": cb / t_gemv / 1e9,
-                "gemv_frac_of_hbm": cb / t_gemv / HBM_PEAK}
+    todo: list = []
+    sub_steps = max(50, args.steps // 4)
 
     if args.traffic_probe:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_()
@@ -333,7 +372,12 @@ def main() -> int:
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    head = measure(args.k, args.rows, args.steps, args.warmup)
+
+    # ---- the headline: one row of the q|k|v shape --------------------------------------------------------------
+    n_head = 16 * args.k
+    d = Dense(torch, api, IN_F, OUT_F, n_head, MCG_CB, 32, torch.float16, seed=1000 + args.k)
+    head = dense_cell(d, args.rows, args.steps, args.warmup, todo, f"headline K{args.k} rows {args.rows}", gemv_alone=True)
+    one_launch = head["plan"]["launches"] == 1
     out = {
         "metric": "EXL3 GEMV HBM GB/s (% of 8 TB/s) at decode rows; MoE prefill GEMM TFLOP/s",
         "value": head["call_gbps"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -341,123 +385,186 @@ def main() -> int:
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": f"dense decode-row GEMV in={IN_F} out={OUT_F} K={args.k} rows={args.rows} MCG w16, "
                                f"f16 activations, {head['copies']} rotating weight copies",
-                   "pct_of_8TBps": 100.0 * head["call_gbps"] * 1e9 / HBM_PEAK, "plan": head["plan"]},
-        "roofline": {"bound": "hbm", "achieved": head["gemv_gbps"], "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": head["gemv_frac_of_hbm"],
-                     "traffic": MEASURED_TRAFFIC.get((IN_F, OUT_F, args.k, args.rows)), "kernel": "t3::dense_gemv",
-                     "us_per_launch": head["gemv_us"], "algorithmic_bytes_per_launch": head["code_bytes"]},
+                   "pct_of_8TBps": 100.0 * head["frac_of_hbm"], "plan": head["plan"]},
+        # the kernel the timed step launches: at one row the call is that one launch, so its duration is the call's
+        "roofline": {"bound": "hbm", "achieved": head["call_gbps"], "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": head["frac_of_hbm"], "traffic": MEASURED_TRAFFIC.get((IN_F, OUT_F, n_head, args.rows)),
+                     "kernel": "t3::dense_gemv<kMcgPair, narrow, 1 row block, 8 tiles, one launch> (prepare, GEMV and finish "
+                               "in the launch)" if one_launch else "t3::dense_gemv (the call's GEMV launch, see gemv_launch_alone)",
+                     "us_per_launch": head["us_per_call"] if one_launch else head.get("gemv_us"),
+                     "algorithmic_bytes_per_launch": head["code_bytes"]},
+        "gemv_launch_alone": {"kernel": "t3::dense_gemv<..., chain> (t3_linear_stages, the GEMV stage only: planes out, no "
+                                        "prepare, no finish)", "us_per_launch": head.get("gemv_us"),
+                              "achieved": head.get("gemv_gbps"), "unit": "GB/s", "frac": head.get("gemv_frac_of_hbm")},
     }
-    if args.moe:
+
+    if "sweep" in sections:
+        out["sweep"] = []
+        for k in (3, 4, 5):
+            dk = d if 16 * k == n_head else Dense(torch, api, IN_F, OUT_F, 16 * k, MCG_CB, 32, torch.float16, seed=1000 + k)
+            for rows in (1, 4, 16, 32):
+                out["sweep"].append(dense_cell(dk, rows, sub_steps, 10, todo, f"sweep K{k} rows {rows}", gemv_alone=True))
+            if dk is not d:
+                del dk
+                torch.cuda.empty_cache()
+
+    if "forms" in sections:
+        # what bit-exact f16 weights cost in the GEMV: MCG's pair form against the rounded weight, MUL1's deferred map
+        # against the weight decoded one by one (t3_configure's mcg_pair, mul1_defer)
+        out["codebook_forms"] = []
+        d.bind(1)
+        dm = Dense(torch, api, IN_F, OUT_F, n_head, MUL1_CB, 1, torch.float16, seed=77)
+        dm.bind(1)
+        for label, obj, cfg in (("MCG, the hashed pair unrounded (served)", d, {}), ("MCG, the f16 weight", d, {"mcg_pair": 0}),
+                                ("MUL1, the deferred map (served)", dm, {}), ("MUL1, the f16 weight", dm, {"mul1_defer": 0})):
+            api.configure(**cfg)
+            try:
+                t = obj.time(sub_steps, 10)
+            finally:
+                api.configure()
+            out["codebook_forms"].append({"form": label, "us_per_call": t * 1e6, "gbps": obj.cb / t / 1e9,
+                                          "frac_of_hbm": obj.cb / t / HBM_PEAK})
+        del dm
+        torch.cuda.empty_cache()
+
+    if "rates" in sections:
+        # a fractional narrow rate (2.5 bits a weight) and a wide one (5.375: the two-register reader)
+        out["rates"] = []
+        for n in (40, 86):
+            dn = Dense(torch, api, IN_F, OUT_F, n, MCG_CB, 1, torch.float16, seed=500 + n)
+            out["rates"].append(dense_cell(dn, 1, sub_steps, 10, todo, f"rate n {n} rows 1", gemv_alone=True))
+            del dn
+            torch.cuda.empty_cache()
+    del d
+    torch.cuda.empty_cache()
+
+    if "peak" in sections or "moe_prefill" in sections or "dense_prefill" in sections or "lm_head" in sections:
+        out["measured_dense_f16_peak"] = measured_f16_peak(torch)
+    peak_meas = out.get("measured_dense_f16_peak", {}).get("tflops")
+    both = lambda flops, t: {"tflops": flops / t / 1e12, "frac_of_f16_mfma_peak": flops / t / MFMA_F16_PEAK,
+                             "frac_of_measured_f16_peak": (flops / t / 1e12 / peak_meas) if peak_meas else None}
+
+    if "lm_head" in sections:
+        in_f, out_f, n = 4096, 151936, 96
+        dl = Dense(torch, api, in_f, out_f, n, MCG_CB, 256, torch.bfloat16, seed=6, copies=2, outliers=False)
+        one = dense_cell(dl, 1, 40, 4, todo, "lm_head K6 rows 1", gemv_alone=True)
+        one["roofline"] = {"bound": "hbm", "kernel": "t3::dense_gemv<kMcgPair, wide, 1, 4 tiles>", "us_per_launch": one.get("gemv_us"),
+                           "algorithmic_bytes_per_launch": dl.cb, "achieved": one.get("gemv_gbps"), "peak": HBM_PEAK / 1e9,
+                           "unit": "GB/s", "frac": one.get("gemv_frac_of_hbm")}
+        many = dense_cell(dl, 256, 10, 2, todo, "lm_head K6 rows 256")
+        flops = 2 * 256 * in_f * out_f
+        t = many["us_per_call"] * 1e-6
+        many.update(both(flops, t))
+        many["roofline"] = {"bound": "mfma", "kernel": "t3::pf_gemm (the trellis GEMM; whole call)", "us_per_call": many["us_per_call"],
+                            "flops": flops, "achieved": flops / t / 1e12, "peak": MFMA_F16_PEAK / 1e12, "unit": "TFLOP/s",
+                            "frac": flops / t / MFMA_F16_PEAK, "frac_of_hbm_on_code_bytes": dl.cb / t / HBM_PEAK}
+        out["lm_head"] = [one, many]
+        del dl
+        torch.cuda.empty_cache()
+
+    if "moe_decode" in sections:
         out["moe_decode"] = []
         for tokens in (1, 8):
-            run = MoeRunner(torch, api, tokens)
-            t = run.time(max(50, args.steps // 2), 10)
-            out["moe_decode"].append({"tokens": tokens, "us_per_call": t * 1e6, "code_bytes": run.code_bytes,
-                                      "gbps": run.code_bytes / t / 1e9, "frac_of_hbm": run.code_bytes / t / HBM_PEAK})
-            del run
-    if args.prefill:
-        run = PrefillRunner(torch, api)
-        t = run.time(5, 2)
-        out["moe_prefill"] = {"workload": "2048 tokens, E256 top-8, 7168/2048, gate|up K2, down K3, bf16, clamp 7",
-                              "ms_per_call": t * 1e3, "tflops": run.flops / t / 1e12,
-                              "frac_of_f16_mfma_peak": run.flops / t / 2.5e15, "code_gbps": run.code_bytes / t / 1e9}
-        del run
+            m = Moe(torch, api, 512, 2048, 512, 3, 3, 10, tokens, 7, shared=True, sets=24, seed=5)
+            todo.append(m.sample(f"moe_decode {tokens} token(s), token 0", 0, BF16_MOE_BAR))
+            steps = max(50, args.steps // 2)
+            t = m.time(steps, 10)
+            t_gu, t_dn = m.time(steps, 10, stages=1), m.time(steps, 10, stages=2)
+            bytes_call = m.distinct * m.per_expert
+            gu_bytes = bytes_call * (2 * code_bytes(2048, 512, 48)) / m.per_expert
+            out["moe_decode"].append({
+                "tokens": tokens, "us_per_call": t * 1e6, "code_bytes": bytes_call, "distinct_experts": m.distinct,
+                "gbps": bytes_call / t / 1e9, "frac_of_hbm": bytes_call / t / HBM_PEAK,
+                "plan": {key: m.plan[key] for key in ("path", "launches", "row_slots", "k_slices_gu", "k_slices_dn")},
+                "roofline": {"bound": "hbm", "kernel": "t3::moe_gemv<gate|up, prepare in LDS, arriving mid> (the longer of "
+                                                       "the call's two launches)",
+                             "us_per_launch": t_gu * 1e6, "algorithmic_bytes_per_launch": gu_bytes,
+                             "achieved": gu_bytes / t_gu / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                             "frac": gu_bytes / t_gu / HBM_PEAK},
+                "launches": {"gate_up_mid_us": t_gu * 1e6, "down_combine_us": t_dn * 1e6}})
+            del m
+            torch.cuda.empty_cache()
+
+    if "moe_prefill" in sections:
+        m = Moe(torch, api, 256, 7168, 2048, 2, 3, 8, 2048, 7, shared=False, sets=1, seed=9)
+        todo.append(m.sample("moe_prefill token 0", 0, BF16_MOE_BAR))
+        t = m.time(5, 2)
+        names = ("route", "prepare", "gemm_gate_up", "mid", "gemm_down", "combine")
+        stage_t = {nm: m.time(5, 1, stages=1 << i) for i, nm in enumerate(names)}
+        gu_flops = m.flops * 2 / 3
+        t_gu = stage_t["gemm_gate_up"]
+        code = 256 * m.per_expert
+        out["moe_prefill"] = {
+            "workload": "2048 tokens, E256 top-8, 7168/2048, gate|up K2, down K3, bf16, clamp 7", "ms_per_call": t * 1e3,
+            "flops": m.flops, **both(m.flops, t), "code_gbps": code / t / 1e9, "frac_of_hbm_on_code_bytes": code / t / HBM_PEAK,
+            "plan": {key: m.plan[key] for key in ("path", "launches", "row_slots", "item_rows", "max_items")},
+            "roofline": {"bound": "mfma", "kernel": "t3::pf_gemm<kMcg, narrow, 8 row blocks, 6 live> (gate|up, the call's longest "
+                                                    "launch)",
+                         "us_per_launch": t_gu * 1e6, "flops_per_launch": gu_flops, "achieved": gu_flops / t_gu / 1e12,
+                         "peak": MFMA_F16_PEAK / 1e12, "unit": "TFLOP/s", "frac": gu_flops / t_gu / MFMA_F16_PEAK,
+                         "frac_of_measured_f16_peak": (gu_flops / t_gu / 1e12 / peak_meas) if peak_meas else None},
+            "stages_us": {nm: v * 1e6 for nm, v in stage_t.items()}}
+        del m
         torch.cuda.empty_cache()
-        rows, in_f, out_f, k = 4096, 4096, 14336, 4
-        g = torch.Generator(device="cuda")
-        g.manual_seed(3)
-        tr = torch.randint(-32768, 32768, (in_f // 16, out_f // 16, 16 * k), dtype=torch.int16, device="cuda", generator=g)
-        suh = (0.5 + torch.rand(in_f, device="cuda", generator=g)).to(torch.float16)
-        svh = ((0.5 + torch.rand(out_f, device="cuda", generator=g)) / in_f ** 0.5).to(torch.float16)
-        x = torch.randn(rows, in_f, device="cuda", generator=g).to(torch.bfloat16)
-        api.linear(x, tr, suh, svh, dec)
-        torch.cuda.synchronize()
+
+    if "dense_prefill" in sections:
+        rows, in_f, out_f, n = 4096, 4096, 14336, 64
+        dp = Dense(torch, api, in_f, out_f, n, MCG_CB, rows, torch.bfloat16, seed=3, copies=1, outliers=False)
+        cell = dense_cell(dp, rows, 5, 2, todo, "dense_prefill 4096 rows")
+        flops = 2 * rows * in_f * out_f
+        t = cell["us_per_call"] * 1e-6
+        tr, suh, svh, x = dp.trellis[0], dp.suh, dp.svh, dp.xr
+        out["dense_prefill"] = {"workload": "4096 rows x (4096 -> 14336) K4 bf16", "ms_per_call": t * 1e3, "flops": flops,
+                                **both(flops, t), "plan": cell["plan"],
+                                "roofline": {"bound": "mfma", "kernel": "the call (W_hat decode, prepare, f16 GEMM, finish)",
+                                             "us_per_call": t * 1e6, "flops": flops, "achieved": flops / t / 1e12,
+                                             "peak": MFMA_F16_PEAK / 1e12, "unit": "TFLOP/s", "frac": flops / t / MFMA_F16_PEAK,
+                                             "frac_of_measured_f16_peak": (flops / t / 1e12 / peak_meas) if peak_meas else None}}
+        # the same projection with its un-rotated weight resident (made once a weight): one plain GEMM a call
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        for _ in range(5):
-            api.linear(x, tr, suh, svh, dec)
-        e1.record()
-        torch.cuda.synchronize()
-        t = e0.elapsed_time(e1) * 1e-3 / 5
-        out["dense_prefill"] = {"workload": "4096 rows x (4096 -> 14336) K4 bf16", "ms_per_call": t * 1e3,
-                                "tflops": 2 * rows * in_f * out_f / t / 1e12,
-                                "frac_of_f16_mfma_peak": 2 * rows * in_f * out_f / t / 2.5e15}
-        # the same projection with its un-rotated weight resident (made once a weight): one plain GEMM a call
-        e0.record()
-        w_std, bad = api.unrot_weight(tr, suh, svh, dec, torch.bfloat16)
+        w_std, bad = api.unrot_weight(tr, suh, svh, dp.dec, torch.bfloat16)
         e1.record()
         torch.cuda.synchronize()
         once = e0.elapsed_time(e1)
-        api.linear_unrot(x, w_std)
-        torch.cuda.synchronize()
-        e0.record()
-        for _ in range(5):
-            api.linear_unrot(x, w_std)
-        e1.record()
-        torch.cuda.synchronize()
-        t = e0.elapsed_time(e1) * 1e-3 / 5
+        t = eager_time(torch, lambda: api.linear_unrot(x, w_std))
         out["dense_prefill_unrot"] = {"workload": "the same, W_std bf16 resident (117 MB)", "ms_per_call": t * 1e3,
-                                      "tflops": 2 * rows * in_f * out_f / t / 1e12,
-                                      "frac_of_f16_mfma_peak": 2 * rows * in_f * out_f / t / 2.5e15,
-                                      "ms_to_make_w_std_once": once, "nonfinite": bad}
+                                      **both(flops, t), "ms_to_make_w_std_once": once, "nonfinite": bad}
         # and with the W_hat of the trellis kept (decoded once a weight): the call above without its decode
-        w_hat = api.dequant(tr, dec)
-        api.linear_resident(x, w_hat, suh, svh)
-        torch.cuda.synchronize()
-        e0.record()
-        for _ in range(5):
-            api.linear_resident(x, w_hat, suh, svh)
-        e1.record()
-        torch.cuda.synchronize()
-        t = e0.elapsed_time(e1) * 1e-3 / 5
+        w_hat = api.dequant(tr, dp.dec)
+        t = eager_time(torch, lambda: api.linear_resident(x, w_hat, suh, svh))
         out["dense_prefill_resident"] = {"workload": "the same, W_hat f16 resident (117 MB)", "ms_per_call": t * 1e3,
-                                         "tflops": 2 * rows * in_f * out_f / t / 1e12,
-                                         "frac_of_f16_mfma_peak": 2 * rows * in_f * out_f / t / 2.5e15}
+                                         **both(flops, t)}
         del w_hat, w_std
-    if args.dense_rows:
-        g = torch.Generator(device="cuda")
-        g.manual_seed(5)
-        tr = torch.randint(-32768, 32768, (IN_F // 16, OUT_F // 16, 16 * args.k), dtype=torch.int16, device="cuda",
-                           generator=g)
-        suh = (0.5 + torch.rand(IN_F, device="cuda", generator=g)).to(torch.float16)
-        svh = ((0.5 + torch.rand(OUT_F, device="cuda", generator=g)) / IN_F ** 0.5).to(torch.float16)
 
-        def dense_us(rows, gemm_rows):
-            api.configure(dense_gemm_rows=gemm_rows)
-            x = torch.randn(rows, IN_F, device="cuda", generator=g).to(torch.bfloat16)
-            api.linear(x, tr, suh, svh, dec)
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(5):
-                api.linear(x, tr, suh, svh, dec)
-            e1.record()
-            torch.cuda.synchronize()
-            return e0.elapsed_time(e1) * 1e3 / 5
+        if "dense_rows" in sections:
+            # few-row dense calls of the same shape: the served partition (K parts follow the rows) against the rows-alone
+            # configuration (one K part whatever the rows: a row's bytes then ignore the call's other rows)
+            out["dense_rows"] = []
+            for r in (64, 256, 1024):
+                xr = dp.x[:r]
+                served = eager_time(torch, lambda: api.linear(xr, tr, suh, svh, dp.dec))
+                api.configure(dense_rows_alone=1)
+                try:
+                    alone = eager_time(torch, lambda: api.linear(xr, tr, suh, svh, dp.dec))
+                finally:
+                    api.configure()
+                out["dense_rows"].append({"rows": r, "served_us": served * 1e6, "rows_alone_us": alone * 1e6,
+                                          "served_plan": {k: v for k, v in api.linear_plan(xr, tr, dp.dec).items()
+                                                          if k in ("path", "k_slices", "workgroups")}})
+        del dp
+        torch.cuda.empty_cache()
 
-        w_hat = api.dequant(tr, dec)
-
-        def resident_us(rows):
-            x = torch.randn(rows, IN_F, device="cuda", generator=g).to(torch.bfloat16)
-            api.linear_resident(x, w_hat, suh, svh)
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(5):
-                api.linear_resident(x, w_hat, suh, svh)
-            e1.record()
-            torch.cuda.synchronize()
-            return e0.elapsed_time(e1) * 1e3 / 5
-
-        out["dense_rows"] = [{"rows": r, "trellis_gemm_us": dense_us(r, 1 << 30), "w_hat_form_us": dense_us(r, 33),
-                              "resident_w_hat_us": resident_us(r)}
-                             for r in (int(v) for v in args.dense_rows.split(","))]
-        api.configure()
-    if args.sweep:
-        out["sweep"] = [measure(k, r, max(50, args.steps // 4), 10) for k in (3, 4, 5) for r in (1, 4, 16, 32)]
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(16 * args.k, seed=11)
+        out["cpu_baseline"], checks = cpu_leg(n_head, seed=11, todo=todo)
+        out["parity_checks"] = {"ok": all(c["ok"] for c in checks), "cells": len(checks),
+                                "worst": max(checks, key=lambda c: c["err_over_rms"] / c["bar"]) if checks else None,
+                                "failed": [c for c in checks if not c["ok"]]}
     print(json.dumps(out))
+    if not args.no_cpu and not out["parity_checks"]["ok"]:
+        print("bench.py: a sampled output missed the reference's bar: " + json.dumps(out["parity_checks"]["failed"]),
+              file=sys.stderr)
+        return 1
     return 0
 
 

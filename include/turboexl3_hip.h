@@ -263,6 +263,22 @@ int32_t t3_moe_with_shared(t3_stream stream, const t3_array* x, const t3_bank* b
 int32_t t3_moe_shared_expert(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
                              const t3_array* scores, t3_decode dec, int32_t limit, const t3_bank* shared_bank,
                              t3_array* y, void* workspace, size_t workspace_bytes);
+/* `t3_moe_shared_expert` (shared_bank NULL: `t3_moe_swiglu` at gate_in; limit 0: no clamp) with a choice of its
+ * launches, for profilers and benchmarks that time one stage at a time (the role `t3_linear_stages` has for the dense
+ * chain; src/hip/plan.zig:294-364,436-476 publishes the same launches one by one). The workspace carries the stages'
+ * results between calls. Up to 16 rows in the two-launch form: bit 0 gate|up + mid, bit 1 down + combine (the four- and
+ * five-launch forms run whole). Above: bit 0 the route, 1 prepare, 2 gate|up GEMM, 3 mid, 4 down GEMM, 5 combine. */
+#define T3_MOE_STAGE_GATE_UP 1u
+#define T3_MOE_STAGE_DOWN 2u
+#define T3_PREFILL_STAGE_ROUTE 1u
+#define T3_PREFILL_STAGE_PREPARE 2u
+#define T3_PREFILL_STAGE_GEMM_GATE_UP 4u
+#define T3_PREFILL_STAGE_MID 8u
+#define T3_PREFILL_STAGE_GEMM_DOWN 16u
+#define T3_PREFILL_STAGE_COMBINE 32u
+int32_t t3_moe_stages(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
+                      const t3_array* scores, t3_decode dec, int32_t limit, const t3_bank* shared_bank, t3_array* y,
+                      void* workspace, size_t workspace_bytes, uint32_t stages);
 /* Decode / verify rows (up to T3_SHARED_ROWS_MAX) of a MoE with a GATED shared expert inside the routed launches
  * (src/models/qwen38/api.zig:305-312 `moeFusedShared`): y = routed + sigmoid(logit) * shared(x), with the roundings of
  * the host's chain it stands for: the routed sum rounds to x's dtype; the shared expert's SwiGLU is the table form in

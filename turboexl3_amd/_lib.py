@@ -105,6 +105,8 @@ SYMBOLS = {
                                         C.c_size_t]),
     "t3_moe_shared_expert": (C.c_int32, [C.c_void_p, _AP, _BP, _AP, _AP, Decode, C.c_int32, _BP, _AP, C.c_void_p,
                                           C.c_size_t]),
+    "t3_moe_stages": (C.c_int32, [C.c_void_p, _AP, _BP, _AP, _AP, Decode, C.c_int32, _BP, _AP, C.c_void_p, C.c_size_t,
+                                  C.c_uint32]),
     "t3_moe_fused_shared": (C.c_int32, [C.c_void_p, _AP, _BP, _AP, _AP, Decode, _BP, _AP, _AP, _AP, C.c_void_p,
                                         C.c_size_t]),
     "t3_moe_fused_shared_routed_workspace_bytes": (C.c_int32, [_AP, _BP, _AP, C.c_int64, _BP, C.POINTER(C.c_size_t)]),

@@ -88,6 +88,11 @@ struct MoeLaunch {
     uint32_t* counts = nullptr;
     uint32_t* cursor = nullptr;
     uint32_t max_items = 0, item_rows = 64;
+    // which launches of the chain a call makes (t3_moe_stages: a profiler's or a benchmark's view of one stage at a
+    // time; the workspace carries the stages' results between calls). Decode, two launches: bit 0 gate|up + mid, bit 1
+    // down + combine. Prefill: bit 0 the route (clear, histogram, scan, place), 1 prepare, 2 gate|up GEMM, 3 mid, 4 down
+    // GEMM, 5 combine. The other decode forms run whole.
+    uint32_t stages = 0xFFFFFFFFu;
 };
 
 // Five launches (prepare, gate|up, mid, down, combine); four (each gate|up wave prepares its own 128-block in LDS);

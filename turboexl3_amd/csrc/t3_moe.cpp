@@ -206,12 +206,14 @@ int decode_form_of(const MoeLaunch& l) {
 
 int32_t run_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
                 const t3_array* scores, const t3_bank* shared_bank, const t3_array* shared_add, t3_decode dec,
-                int32_t limit, t3_array* y, void* workspace, size_t workspace_bytes, int32_t clamp_at = 0) {
+                int32_t limit, t3_array* y, void* workspace, size_t workspace_bytes, int32_t clamp_at = 0,
+                uint32_t stages = 0xFFFFFFFFu) {
     if (!scores || !y) return T3_BadArgs;
     MoeCall call;
     if (const int32_t st = check_moe(x, bank, inds, scores, shared_bank, shared_add, dec, limit, y, &call, clamp_at);
         st != T3_OK)
         return st;
+    call.launch.stages = stages;
     if (!workspace_ok(workspace)) return T3_BadArgs;
     // rows above the decode chain's take the prefill GEMM chain (src/root.zig:850-853)
     if (call.rows > T3_DECODE_ROWS_MAX) {
@@ -328,6 +330,15 @@ int32_t t3_moe_shared_expert(t3_stream stream, const t3_array* x, const t3_bank*
                              t3_array* y, void* workspace, size_t workspace_bytes) {
     if (!shared_bank) return T3_BadArgs;
     return t3::run_moe(stream, x, bank, inds, scores, shared_bank, nullptr, dec, limit, y, workspace, workspace_bytes);
+}
+
+int32_t t3_moe_stages(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
+                      const t3_array* scores, t3_decode dec, int32_t limit, const t3_bank* shared_bank, t3_array* y,
+                      void* workspace, size_t workspace_bytes, uint32_t stages) {
+    if (limit < 0 || limit > 128) return T3_InvalidExl3Clamp;
+    if (stages == 0u || stages > 63u) return T3_BadArgs;
+    return t3::run_moe(stream, x, bank, inds, scores, shared_bank, nullptr, dec, limit, y, workspace, workspace_bytes, 0,
+                       stages);
 }
 
 /* GLM's rounding profile of the routed experts (src/hip/plan.zig:219-247 `Profile.glm`): x bf16, each routed slot's own

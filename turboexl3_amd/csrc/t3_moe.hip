@@ -272,8 +272,10 @@ hipError_t launch_moe_decode(const MoeLaunch& a, int form, hipStream_t s) {
     const uint32_t rkt = a.rows * (a.topk + a.shared_slots);
     hipError_t e;
     if (form == kMoeTwoLaunches && !a.glm) {
-        if ((e = launch_gemv_cb<2, true, true>(a, s)) != hipSuccess) return e;
-        return launch_gemv_cb<1, false, true>(a, s);
+        if (a.stages & 1u)
+            if ((e = launch_gemv_cb<2, true, true>(a, s)) != hipSuccess) return e;
+        if (a.stages & 2u) return launch_gemv_cb<1, false, true>(a, s);
+        return hipSuccess;
     }
     if (a.glm) {
         // GLM's profile runs the five launches with its own roundings in the stages between the GEMVs

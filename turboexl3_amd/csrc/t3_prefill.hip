@@ -697,19 +697,23 @@ hipError_t launch_gemm(const PfGemm& g, int codebook, uint32_t max_items, uint32
 hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s) {
     const uint32_t kt = a.topk + a.shared_slots, p = a.rows * kt, et = a.bank.experts + a.shared_slots;
     hipError_t e;
-    hipLaunchKernelGGL(pf_clear, dim3((et + 2u + 255u) / 256u), dim3(256), 0, s, a.counts, et + 2u);
-    if ((e = hipGetLastError()) != hipSuccess) return e;
-    hipLaunchKernelGGL(pf_hist, dim3((p + 255u) / 256u), dim3(256), 0, s, a);
-    if ((e = hipGetLastError()) != hipSuccess) return e;
-    hipLaunchKernelGGL(pf_scan, dim3(1), dim3(1024), 0, s, a);
-    if ((e = hipGetLastError()) != hipSuccess) return e;
-    hipLaunchKernelGGL(pf_place, dim3((p + 255u) / 256u), dim3(256), 0, s, a);
-    if ((e = hipGetLastError()) != hipSuccess) return e;
-    if (a.glm) hipLaunchKernelGGL((pf_prep<kBf16, 1>), unit_grid(p, a.hidden), dim3(256), 0, s, a);
-    else if (a.dtype == kF32) hipLaunchKernelGGL((pf_prep<kF32, 0>), unit_grid(p, a.hidden), dim3(256), 0, s, a);
-    else if (a.dtype == kF16) hipLaunchKernelGGL((pf_prep<kF16, 0>), unit_grid(p, a.hidden), dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((pf_prep<kBf16, 0>), unit_grid(p, a.hidden), dim3(256), 0, s, a);
-    if ((e = hipGetLastError()) != hipSuccess) return e;
+    if (a.stages & 1u) {
+        hipLaunchKernelGGL(pf_clear, dim3((et + 2u + 255u) / 256u), dim3(256), 0, s, a.counts, et + 2u);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        hipLaunchKernelGGL(pf_hist, dim3((p + 255u) / 256u), dim3(256), 0, s, a);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        hipLaunchKernelGGL(pf_scan, dim3(1), dim3(1024), 0, s, a);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        hipLaunchKernelGGL(pf_place, dim3((p + 255u) / 256u), dim3(256), 0, s, a);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+    }
+    if (a.stages & 2u) {
+        if (a.glm) hipLaunchKernelGGL((pf_prep<kBf16, 1>), unit_grid(p, a.hidden), dim3(256), 0, s, a);
+        else if (a.dtype == kF32) hipLaunchKernelGGL((pf_prep<kF32, 0>), unit_grid(p, a.hidden), dim3(256), 0, s, a);
+        else if (a.dtype == kF16) hipLaunchKernelGGL((pf_prep<kF16, 0>), unit_grid(p, a.hidden), dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((pf_prep<kBf16, 0>), unit_grid(p, a.hidden), dim3(256), 0, s, a);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+    }
 
     PfGemm g{};
     g.w[0] = a.bank.gate_t;
@@ -728,11 +732,14 @@ hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s) {
     g.wbits = a.wbits;
     g.positions = p;
     g.experts = a.bank.experts;
-    if ((e = launch_gemm(g, a.codebook, a.max_items, 2u, a.item_rows, s)) != hipSuccess) return e;
+    if (a.stages & 4u)
+        if ((e = launch_gemm(g, a.codebook, a.max_items, 2u, a.item_rows, s)) != hipSuccess) return e;
 
-    if (a.glm) hipLaunchKernelGGL(pf_mid<1>, unit_grid(p, a.inter), dim3(256), 0, s, a);
-    else hipLaunchKernelGGL(pf_mid<0>, unit_grid(p, a.inter), dim3(256), 0, s, a);
-    if ((e = hipGetLastError()) != hipSuccess) return e;
+    if (a.stages & 8u) {
+        if (a.glm) hipLaunchKernelGGL(pf_mid<1>, unit_grid(p, a.inter), dim3(256), 0, s, a);
+        else hipLaunchKernelGGL(pf_mid<0>, unit_grid(p, a.inter), dim3(256), 0, s, a);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+    }
 
     g.w[0] = a.bank.down_t;
     g.ws[0] = a.shared.down_t;
@@ -744,8 +751,10 @@ hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s) {
     g.in = a.inter;
     g.out = a.hidden;
     g.n = a.n_dn;
-    if ((e = launch_gemm(g, a.codebook, a.max_items, 1u, a.item_rows, s)) != hipSuccess) return e;
+    if (a.stages & 16u)
+        if ((e = launch_gemm(g, a.codebook, a.max_items, 1u, a.item_rows, s)) != hipSuccess) return e;
 
+    if (!(a.stages & 32u)) return hipSuccess;
     if (a.glm) hipLaunchKernelGGL(pf_slots, unit_grid(p, a.hidden), dim3(256), 0, s, a);
     else hipLaunchKernelGGL(pf_combine, unit_grid(a.rows, a.hidden), dim3(256), 0, s, a);
     return hipGetLastError();
