@@ -17,8 +17,8 @@ LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(LIBDIR, "obj")
 LIB = os.path.join(LIBDIR, "libturboexl3_hip.so")
 
-HIP_SOURCES = ["t3_dense.hip", "t3_dequant.hip", "t3_moe.hip", "t3_prefill.hip", "t3_unrot.hip"]
-HOST_SOURCES = ["t3_api.cpp", "t3_blas.cpp", "t3_linear.cpp", "t3_moe.cpp", "t3_table.cpp"]
+HIP_SOURCES = ["t3_dense.hip", "t3_dequant.hip", "t3_gemm.hip", "t3_moe.hip", "t3_prefill.hip", "t3_unrot.hip"]
+HOST_SOURCES = ["t3_api.cpp", "t3_linear.cpp", "t3_moe.cpp", "t3_table.cpp"]
 
 ARCH = "gfx950"
 COMMON = ["-O3", "-std=c++20", "-fPIC", "-ffp-contract=off", "-Wall", "-Wno-unused-function"]

@@ -49,13 +49,6 @@ inline int32_t resolve_decode(t3_decode dec, Dec* out) {
     return T3_OK;
 }
 
-// rocBLAS, opened at run time (t3_blas.cpp)
-bool blas_available();
-int32_t blas_gemm_f16(hipStream_t s, const uint16_t* xp, const uint16_t* w_hat, uint16_t* z, uint32_t rows, uint32_t in,
-                      uint32_t out);
-int32_t blas_gemm_half(hipStream_t s, bool bf16, const void* x, const void* w, uint32_t ldw, void* y, uint32_t rows,
-                       uint32_t in, uint32_t cols);
-
 // Scratch carved from the caller's workspace in 256-byte steps.
 struct Carver {
     unsigned char* base;

@@ -95,11 +95,11 @@ void carve_dense_prefill(DenseCall* call, void* workspace) {
 
 constexpr uint32_t kGemvRowsMax = 32;
 
-// From dense_gemm_rows rows up (and with rocBLAS present) a dense call decodes W_hat once and multiplies plainly
-// (src/core/dense.zig:909-922,1290-1302): the decode is paid once a call, not once a 64-row item.
+// From dense_gemm_rows rows up a dense call decodes W_hat once and multiplies plainly (src/core/dense.zig:909-922,
+// 1290-1302): the decode is paid once a call, not once a 64-row item.
 bool takes_w_hat(const DenseLaunch& l) {
     const int32_t from = config().dense_gemm_rows;
-    return !config().dense_rows_alone && from > 0 && l.rows >= static_cast<uint32_t>(from) && blas_available();
+    return !config().dense_rows_alone && from > 0 && l.rows >= static_cast<uint32_t>(from) && gemm_half_ok(l.in, l.out);
 }
 
 struct WhatScratch {
@@ -123,7 +123,8 @@ WhatScratch carve_dense_w_hat(DenseCall* call, void* workspace) {
 // prepare (natural order) -> z = f16(xp W_hat) -> finish, over a W_hat that is already there
 int32_t run_over_w_hat(const DenseLaunch& l, const uint16_t* w_hat, uint16_t* xp, uint16_t* z, hipStream_t s) {
     if (const int32_t st = hip_status(launch_dense_prep_natural(l, xp, s)); st != T3_OK) return st;
-    if (const int32_t st = blas_gemm_f16(s, xp, w_hat, z, l.rows, l.in, l.out); st != T3_OK) return st;
+    if (const int32_t st = hip_status(launch_gemm_half(xp, w_hat, z, l.rows, l.in, l.out, l.out, false, s)); st != T3_OK)
+        return st;
     return hip_status(launch_dense_finish_half(l, z, s));
 }
 
@@ -163,8 +164,8 @@ int32_t check_resident(const t3_array* x, const t3_array* w_hat, const t3_array*
             if (y->shape[i] != x->shape[i]) return T3_BadExl3Shape;
         if (y->dtype != x->dtype) return T3_BadExl3Dtype;
     }
-    // decode and verify rows never read a W_hat (src/core/dense.zig:1309 `prefillOperands`), and the GEMM is rocBLAS's
-    if (rows <= kGemvRowsMax || !blas_available()) return T3_Exl3EngineNotImplemented;
+    // decode and verify rows never read a W_hat (src/core/dense.zig:1309 `prefillOperands`)
+    if (rows <= kGemvRowsMax || !gemm_half_ok(in, out)) return T3_Exl3EngineNotImplemented;
     if (rows * in * 4 >= (1ll << 31)) return T3_Exl3EngineNotImplemented;
     DenseLaunch& l = call->launch;
     l.x = x->data;
@@ -438,12 +439,14 @@ int32_t t3_linear_unrot(t3_stream stream, const t3_array* x, const t3_array* w_s
         return T3_BadExl3Shape;
     if ((w_std->dtype != T3_F16 && w_std->dtype != T3_BF16) || x->dtype != w_std->dtype || y->dtype != w_std->dtype)
         return T3_BadExl3Dtype;
-    if (rows <= 32 || !t3::blas_available()) return T3_Exl3EngineNotImplemented;
+    if (!t3::aligned16(x) || !t3::aligned16(w_std) || !t3::aligned16(y) || col0 % 8 != 0) return T3_BadArgs;
+    if (rows <= 32 || !t3::gemm_half_ok(static_cast<uint64_t>(in), static_cast<uint64_t>(w_std->shape[1])))
+        return T3_Exl3EngineNotImplemented;
     const size_t esz = 2u;
-    return t3::blas_gemm_half(static_cast<hipStream_t>(stream), w_std->dtype == T3_BF16, x->data,
-                              static_cast<const unsigned char*>(w_std->data) + static_cast<size_t>(col0) * esz,
-                              static_cast<uint32_t>(w_std->shape[1]), y->data, static_cast<uint32_t>(rows),
-                              static_cast<uint32_t>(in), static_cast<uint32_t>(cols));
+    return t3::hip_status(t3::launch_gemm_half(
+        x->data, static_cast<const unsigned char*>(w_std->data) + static_cast<size_t>(col0) * esz, y->data,
+        static_cast<uint32_t>(rows), static_cast<uint32_t>(in), static_cast<uint32_t>(cols),
+        static_cast<uint32_t>(w_std->shape[1]), w_std->dtype == T3_BF16, static_cast<hipStream_t>(stream)));
 }
 
 }  // extern "C"
