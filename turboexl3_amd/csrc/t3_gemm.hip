@@ -20,11 +20,20 @@
 //                (ds_read_b64_tr_b16: inside every 16 lanes, the 4 x 16 halfwords the lanes address are transposed, lane
 //                i receiving column i) delivers them, two reads a fragment, and f(k) spreads one such read's sixteen
 //                rows over the banks.
+// The end. The accumulators go to LDS as one 256 x 256 tile of halfwords (528-byte rows, so the matrix-core layout's
+// 16 rows a store spread over the banks), and leave it 16 bytes a lane, 256 contiguous bytes a row segment. FINISH: the
+// tile is z = f16(xp W_hat), format.innerGemv's rounding point (src/core/format.zig:366), and the launch ends with
+// format.finishOutput (:370-380) on it: four 128-blocks a wave, 16 lanes a block, the statements of the prefill chains'
+// finish kernel, then y in the call's dtype. z never sees memory.
 // Workgroup ids: consecutive ids go round the eight dies; a die takes column blocks nt = 8 j + die and walks every row
-// block of one column block before the next, so a die's L2 holds the weight strip its workgroups share.
+// block of one column block before the next, so a die's L2 holds the weight strip its workgroups share. A workgroup
+// holds a compute unit alone (135 KB of LDS), so the launch runs in rounds of 256 workgroups; where the last round would
+// fill at most half the GPU, its column blocks are cut to 128 columns (the same kernel with two column blocks a wave):
+// 4096 rows x 14336 columns is 896 tiles = 3.5 rounds, and runs as 768 full tiles + 256 half ones.
 
 #include "t3_common.hpp"
 #include "t3_kernels.hpp"
+#include "t3_stages.hpp"
 
 namespace t3 {
 namespace {
@@ -32,6 +41,8 @@ namespace {
 constexpr uint32_t kGM = 256, kGN = 256, kGK = 32, kGD = 4;     // tile rows, columns, K a step, steps in the ring
 constexpr uint32_t kGXBytes = kGM * kGK * 2u, kGWBytes = kGK * kGN * 2u, kGStep = kGXBytes + kGWBytes;
 constexpr int kGLoadsAStep = 4;                                  // loads a wave a step: two of x, two of w
+constexpr uint32_t kGZRow = kGN * 2u + 16u;                      // bytes a row of the output tile in LDS
+constexpr uint32_t kGLds = kGD * kGStep > kGM * kGZRow ? kGD * kGStep : kGM * kGZRow;
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef short short4v __attribute__((ext_vector_type(4)));
@@ -41,7 +52,10 @@ struct GemmArgs {
     const void* x;
     const void* w;
     void* y;
-    uint32_t rows, in, cols, ldw, mt, nt;
+    const uint16_t* svh;  // FINISH: the output scale vector f16 [cols]
+    int dt;               // FINISH: y's dtype (t3::Dtype); else y is in the operands' dtype
+    uint32_t rows, in, cols, ldw, mt;
+    uint32_t ntf, nth;    // column blocks of 256, then of 128
 };
 
 __device__ __forceinline__ uint4v gemm_rsrc(const void* p, uint64_t bytes) {
@@ -68,15 +82,20 @@ __device__ __forceinline__ float4v gemm_mfma(uint4v a, uint4v b, float4v c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c, 0, 0, 0);
 }
 
-// Grid (8 mt, ceil(nt / 8)), 512 threads.
-template <bool BF16>
+// Grid (8 mt, ceil(ntf / 8) + ceil(nth / 8)), 512 threads: ntf column blocks of 256 first, then nth of 128 (launched
+// last, so they fill the launch's tail: a workgroup holds a compute unit alone, and a last round of full tiles on half
+// the compute units would take as long as a full one).
+template <bool BF16, bool FINISH>
 __global__ void __launch_bounds__(512) gemm_half(const GemmArgs a) {
-    __shared__ __attribute__((aligned(16))) unsigned char smem[kGD * kGStep];
-    const uint32_t die = blockIdx.x & 7u, mi = blockIdx.x >> 3, ni = blockIdx.y * 8u + die;
-    if (ni >= a.nt) return;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[kGLds];
+    const uint32_t die = blockIdx.x & 7u, mi = blockIdx.x >> 3;
+    const uint32_t yf = (a.ntf + 7u) >> 3;
+    const bool half = blockIdx.y >= yf;   // uniform over the workgroup
+    const uint32_t ni = (half ? blockIdx.y - yf : blockIdx.y) * 8u + die;
+    if (ni >= (half ? a.nth : a.ntf)) return;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
     const uint32_t wm = wave & 1u, wn = wave >> 1;
-    const uint32_t row0 = mi * kGM, col0 = ni * kGN;
+    const uint32_t row0 = mi * kGM, col0 = half ? a.ntf * kGN + ni * (kGN / 2u) : ni * kGN;
 
     // the tile's windows of x and w: rows past the last one, and the bytes past w's end, read as zeros
     const uint32_t rows_here = a.rows - row0 < kGM ? a.rows - row0 : kGM;
@@ -84,7 +103,8 @@ __global__ void __launch_bounds__(512) gemm_half(const GemmArgs a) {
                                    static_cast<uint64_t>(rows_here) * a.in * 2u);
     const uint4v wdesc = gemm_rsrc(static_cast<const unsigned char*>(a.w) + static_cast<size_t>(col0) * 2u,
                                    (static_cast<uint64_t>(a.in) * a.ldw - col0) * 2u);
-    // this wave's loads a step: x rows 32 wave .. + 31 (two loads of 16 rows), w rows k = 4 wave .. + 3 (two of 2 rows)
+    // this wave's loads a step: x rows 32 wave .. + 31 (two loads of 16 rows), w rows k = 4 wave .. + 3 (two of 2 rows;
+    // a 128-column tile loads 256 columns all the same and leaves the second half alone)
     uint32_t x_voff[2], w_voff[2];
 #pragma unroll
     for (uint32_t i = 0; i < 2u; ++i) {
@@ -108,87 +128,121 @@ __global__ void __launch_bounds__(512) gemm_half(const GemmArgs a) {
     // where a lane's fragments sit inside a step's 32 KB
     // activations, row block rb: row 128 wm + 16 rb + lane % 16, piece lane / 16, swizzled
     const uint32_t xf_at = (128u * wm + (lane & 15u)) * 64u + (((lane >> 4) ^ ((lane >> 1) & 3u)) * 16u);
-    // weights, column block cb, half h: row k = 8 g + 4 h + j / 4, columns 16 (4 wn + cb) + 4 (j % 4) .. + 3
     const uint32_t g = lane >> 4, j = lane & 15u;
-    const uint32_t fk = 2u * ((j >> 2) + 4u * (g & 1u));
-    uint32_t wf_at[4];
-#pragma unroll
-    for (uint32_t cb = 0; cb < 4u; ++cb) {
-        const uint32_t piece = (8u * wn + 2u * cb + ((j >> 1) & 1u)) ^ fk;
-        wf_at[cb] = kGXBytes + (8u * g + (j >> 2)) * 512u + piece * 16u + (j & 1u) * 8u;
-    }
 
-    float4v acc[4][8];
+    // The K loop and the end for a wave that owns CBN column blocks: 4 (a 256-column tile) or 2 (a 128-column one).
+    auto run = [&]<int CBN>() {
+        constexpr uint32_t kCols = 64u * CBN;   // the tile's columns
+        // weights, column block cb, half h: row k = 8 g + 4 h + j / 4, columns 16 (CBN wn + cb) + 4 (j % 4) .. + 3
+        const uint32_t fk = 2u * ((j >> 2) + 4u * (g & 1u));
+        uint32_t wf_at[CBN];
 #pragma unroll
-    for (int cb = 0; cb < 4; ++cb)
-#pragma unroll
-        for (int rb = 0; rb < 8; ++rb) acc[cb][rb] = float4v{0.f, 0.f, 0.f, 0.f};
-
-    const uint32_t steps = a.in / kGK;
-#pragma unroll
-    for (uint32_t t = 0; t + 1u < kGD; ++t) issue(t, t);   // loads past the last step fall outside the buffers: zeros
-    gemm_wait_loads<static_cast<int>(kGD - 2u) * kGLoadsAStep>();
-    __syncthreads();
-    uint32_t slot = 0;
-    for (uint32_t s = 0; s < steps; ++s) {
-        // the slot step s - 1 used is free: every wave passed the barrier that ended it
-        issue(s + kGD - 1u, slot == 0u ? kGD - 1u : slot - 1u);
-        const unsigned char* st = smem + slot * kGStep;
-        uint4v wf[4], xf[8];
-#pragma unroll
-        for (uint32_t cb = 0; cb < 4u; ++cb) {
-            const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v*)(st + wf_at[cb]));
-            const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v*)(st + wf_at[cb] + 4u * 512u));
-            const uint2 l2 = __builtin_bit_cast(uint2, lo), h2 = __builtin_bit_cast(uint2, hi);
-            wf[cb] = uint4v{l2.x, l2.y, h2.x, h2.y};
+        for (uint32_t cb = 0; cb < static_cast<uint32_t>(CBN); ++cb) {
+            const uint32_t piece = (2u * CBN * wn + 2u * cb + ((j >> 1) & 1u)) ^ fk;
+            wf_at[cb] = kGXBytes + (8u * g + (j >> 2)) * 512u + piece * 16u + (j & 1u) * 8u;
         }
+        float4v acc[CBN][8];
 #pragma unroll
-        for (uint32_t rb = 0; rb < 8u; ++rb) xf[rb] = *reinterpret_cast<const uint4v*>(st + xf_at + rb * 1024u);
+        for (int cb = 0; cb < CBN; ++cb)
 #pragma unroll
-        for (int cb = 0; cb < 4; ++cb)
+            for (int rb = 0; rb < 8; ++rb) acc[cb][rb] = float4v{0.f, 0.f, 0.f, 0.f};
+
+        const uint32_t steps = a.in / kGK;
 #pragma unroll
-            for (int rb = 0; rb < 8; ++rb) acc[cb][rb] = gemm_mfma<BF16>(wf[cb], xf[rb], acc[cb][rb]);
-        // step s + 1's loads of this wave have landed once at most kGD - 2 steps' are in flight; the barrier then
-        // publishes every wave's part of it
+        for (uint32_t t = 0; t + 1u < kGD; ++t) issue(t, t);   // loads past the last step bring zeros or unused bytes
         gemm_wait_loads<static_cast<int>(kGD - 2u) * kGLoadsAStep>();
         __syncthreads();
-        slot = slot + 1u == kGD ? 0u : slot + 1u;
-    }
-    gemm_wait_loads<0>();
-
-    // lane: row 16 rb + lane % 16, columns 16 cb + 4 (lane / 16) .. + 3 of the wave's 128 x 64
-    const bool vec = (a.cols & 3u) == 0u;
+        uint32_t slot = 0;
+        for (uint32_t s = 0; s < steps; ++s) {
+            // the slot step s - 1 used is free: every wave passed the barrier that ended it
+            issue(s + kGD - 1u, slot == 0u ? kGD - 1u : slot - 1u);
+            const unsigned char* st = smem + slot * kGStep;
+            uint4v wf[CBN], xf[8];
 #pragma unroll
-    for (int rb = 0; rb < 8; ++rb) {
-        const uint32_t row = row0 + 128u * wm + static_cast<uint32_t>(rb) * 16u + (lane & 15u);
-        if (row >= a.rows) continue;
+            for (uint32_t cb = 0; cb < static_cast<uint32_t>(CBN); ++cb) {
+                const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v*)(st + wf_at[cb]));
+                const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4v*)(st + wf_at[cb] + 4u * 512u));
+                const uint2 l2 = __builtin_bit_cast(uint2, lo), h2 = __builtin_bit_cast(uint2, hi);
+                wf[cb] = uint4v{l2.x, l2.y, h2.x, h2.y};
+            }
 #pragma unroll
-        for (int cb = 0; cb < 4; ++cb) {
-            const uint32_t col = col0 + 64u * wn + static_cast<uint32_t>(cb) * 16u + 4u * (lane >> 4);
-            if (col >= a.cols) continue;
-            uint16_t h[4];
+            for (uint32_t rb = 0; rb < 8u; ++rb) xf[rb] = *reinterpret_cast<const uint4v*>(st + xf_at + rb * 1024u);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) h[c] = BF16 ? bf16_bits(acc[cb][rb][c]) : half_bits(acc[cb][rb][c]);
-            uint16_t* dst = static_cast<uint16_t*>(a.y) + static_cast<size_t>(row) * a.cols + col;
-            if (vec) {
-                *reinterpret_cast<uint2*>(dst) = uint2{h[0] | (static_cast<uint32_t>(h[1]) << 16),
-                                                       h[2] | (static_cast<uint32_t>(h[3]) << 16)};
-            } else {
+            for (int cb = 0; cb < CBN; ++cb)
 #pragma unroll
-                for (uint32_t c = 0; c < 4u; ++c)
-                    if (col + c < a.cols) dst[c] = h[c];
+                for (int rb = 0; rb < 8; ++rb) acc[cb][rb] = gemm_mfma<BF16>(wf[cb], xf[rb], acc[cb][rb]);
+            // step s + 1's loads of this wave have landed once at most kGD - 2 steps' are in flight; the barrier then
+            // publishes every wave's part of it
+            gemm_wait_loads<static_cast<int>(kGD - 2u) * kGLoadsAStep>();
+            __syncthreads();
+            slot = slot + 1u == kGD ? 0u : slot + 1u;
+        }
+        gemm_wait_loads<0>();
+        // every wave is past its last fragment reads (the loop's last barrier) and no load is in flight: the ring's
+        // memory takes the output tile. lane: row 16 rb + lane % 16, columns 16 cb + 4 (lane / 16) .. + 3 of the wave's part
+        __syncthreads();
+#pragma unroll
+        for (int rb = 0; rb < 8; ++rb)
+#pragma unroll
+            for (int cb = 0; cb < CBN; ++cb) {
+                const uint32_t row = 128u * wm + static_cast<uint32_t>(rb) * 16u + (lane & 15u);
+                const uint32_t col = 16u * CBN * wn + static_cast<uint32_t>(cb) * 16u + 4u * (lane >> 4);
+                uint32_t h[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) h[c] = (BF16 && !FINISH) ? bf16_bits(acc[cb][rb][c]) : half_bits(acc[cb][rb][c]);
+                *reinterpret_cast<uint2*>(smem + row * kGZRow + col * 2u) = uint2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+            }
+        __syncthreads();
+        if constexpr (FINISH) {
+            // units = 256 rows x the tile's 128-blocks; a wave takes four a pass
+            constexpr uint32_t kBlocks = kCols / 128u, kPasses = 256u * kBlocks / 32u;
+            // (unit u = 32 it + 4 wave + lane / 16 is row u / kBlocks, block u % kBlocks: a lane keeps its block, so its
+            // eight svh values are loaded once and no pass waits on memory: LDS read, butterflies, store)
+            const Row16 g16 = row16(lane);
+            const uint32_t q = lane & 15u, blk = (lane >> 4) % kBlocks;
+            const uint32_t col = col0 + 128u * blk + 8u * q;
+            const bool col_live = col < a.cols;
+            float sv[8];
+            load8_half(a.svh, col_live ? col : 0u, sv);
+#pragma unroll 4
+            for (uint32_t it = 0; it < kPasses; ++it) {
+                const uint32_t row = (it * 32u + wave * 4u + (lane >> 4)) / kBlocks;
+                float v[8];
+                load8_half(reinterpret_cast<const uint16_t*>(smem + row * kGZRow), 128u * blk + 8u * q, v);
+                finish_row16(v, sv, g16);
+                if (col_live && row0 + row < a.rows) store8_act_rt(a.dt, a.y, static_cast<size_t>(row0 + row) * a.cols + col, v);
+            }
+        } else {
+            // 16-byte pieces: a wave stores whole row segments an instruction
+            constexpr uint32_t kPieces = kCols / 8u, kPasses = 256u * kPieces / 512u;
+            const bool vec = (a.cols & 7u) == 0u;
+            for (uint32_t it = 0; it < kPasses; ++it) {
+                const uint32_t p = it * 512u + threadIdx.x, row = p / kPieces, piece = p % kPieces;
+                const uint32_t col = col0 + piece * 8u;
+                if (row0 + row >= a.rows || col >= a.cols) continue;
+                const uint4v w = *reinterpret_cast<const uint4v*>(smem + row * kGZRow + piece * 16u);
+                uint16_t* dst = static_cast<uint16_t*>(a.y) + static_cast<size_t>(row0 + row) * a.cols + col;
+                if (vec) {
+                    *reinterpret_cast<uint4v*>(dst) = w;
+                } else {
+#pragma unroll
+                    for (uint32_t c = 0; c < 8u; ++c)
+                        if (col + c < a.cols) dst[c] = static_cast<uint16_t>(w[c >> 1] >> (16u * (c & 1u)));
+                }
             }
         }
-    }
+    };
+    if (half) run.template operator()<2>();
+    else run.template operator()<4>();
 }
 
 }  // namespace
 
-// y [rows][cols] = x [rows][in] w[:, 0:cols] for w [in][ldw] (all f16 or all bf16; y row-contiguous). The host has
-// checked: in a multiple of 32, ldw a multiple of 8, w and x 16-byte aligned, in ldw 2 bytes under 4 GiB.
-hipError_t launch_gemm_half(const void* x, const void* w, void* y, uint32_t rows, uint32_t in, uint32_t cols, uint32_t ldw,
-                            bool bf16, hipStream_t s) {
-    GemmArgs a;
+namespace {
+// The launch's column blocks. Every block 256 wide, except that a launch whose last round of workgroups (one a compute
+// unit) would fill at most half the GPU cuts that round's column blocks in two: twice the workgroups, half as long.
+GemmArgs gemm_args(const void* x, const void* w, void* y, uint32_t rows, uint32_t in, uint32_t cols, uint32_t ldw) {
+    GemmArgs a{};
     a.x = x;
     a.w = w;
     a.y = y;
@@ -197,10 +251,42 @@ hipError_t launch_gemm_half(const void* x, const void* w, void* y, uint32_t rows
     a.cols = cols;
     a.ldw = ldw;
     a.mt = (rows + kGM - 1u) / kGM;
-    a.nt = (cols + kGN - 1u) / kGN;
-    const dim3 grid(8u * a.mt, (a.nt + 7u) / 8u), block(512);
-    if (bf16) hipLaunchKernelGGL(gemm_half<true>, grid, block, 0, s, a);
-    else hipLaunchKernelGGL(gemm_half<false>, grid, block, 0, s, a);
+    const uint32_t nt = (cols + kGN - 1u) / kGN, cus = 256u;
+    const uint32_t last = (a.mt * nt) % cus;          // workgroups of the last round
+    uint32_t cut = last != 0u && last <= cus / 2u ? last / a.mt : 0u;   // whole column blocks among them
+    if (a.mt * nt < cus) cut = 0u;                    // a launch that never fills the GPU has no tail to balance
+    if (cut > nt) cut = nt;
+    a.ntf = nt - cut;
+    a.nth = 0u;
+    if (cut != 0u) {
+        const uint32_t first = a.ntf * kGN;           // the cut blocks' first column
+        a.nth = (cols - first + kGN / 2u - 1u) / (kGN / 2u);
+    }
+    return a;
+}
+dim3 gemm_grid(const GemmArgs& a) { return dim3(8u * a.mt, (a.ntf + 7u) / 8u + (a.nth + 7u) / 8u); }
+}  // namespace
+
+// y [rows][cols] = x [rows][in] w[:, 0:cols] for w [in][ldw] (all f16 or all bf16; y row-contiguous). The host has
+// checked: in a multiple of 32, ldw a multiple of 8, w and x 16-byte aligned, in ldw 2 bytes under 4 GiB.
+hipError_t launch_gemm_half(const void* x, const void* w, void* y, uint32_t rows, uint32_t in, uint32_t cols, uint32_t ldw,
+                            bool bf16, hipStream_t s) {
+    const GemmArgs a = gemm_args(x, w, y, rows, in, cols, ldw);
+    const dim3 grid = gemm_grid(a), block(512);
+    if (bf16) hipLaunchKernelGGL((gemm_half<true, false>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((gemm_half<false, false>), grid, block, 0, s, a);
+    return hipGetLastError();
+}
+
+// y [rows][out] = finish(f16(xp [rows][in] w_hat [in][out])) in `dtype`: the W_hat form's product and finish in one
+// launch (xp: the prepared rows, f16 in natural order; out a multiple of 128)
+hipError_t launch_gemm_finish(const uint16_t* xp, const uint16_t* w_hat, const uint16_t* svh, void* y, uint32_t rows,
+                              uint32_t in, uint32_t out, int dtype, hipStream_t s) {
+    GemmArgs a = gemm_args(xp, w_hat, y, rows, in, out, out);
+    a.svh = svh;
+    a.dt = dtype;
+    const dim3 grid = gemm_grid(a), block(512);
+    hipLaunchKernelGGL((gemm_half<false, true>), grid, block, 0, s, a);
     return hipGetLastError();
 }
 

@@ -153,16 +153,17 @@ inline uint32_t gemm_grid_x(uint32_t nblk, uint32_t max_items) {
 // workgroups a K part of the dense trellis GEMM launches
 inline uint32_t dense_prefill_workgroups(uint32_t out, uint32_t items) { return gemm_grid_x((out + 255u) / 256u, items); }
 
-// The W_hat form's own stages: the prepare in natural order (plain f16 [rows][in], what a plain GEMM multiplies), and the
-// finish of an f16 z [rows][out].
+// The W_hat form's own prepare: natural order (plain f16 [rows][in], what a plain GEMM multiplies).
 hipError_t launch_dense_prep_natural(const DenseLaunch& d, uint16_t* xp, hipStream_t s);
-hipError_t launch_dense_finish_half(const DenseLaunch& d, const uint16_t* z, hipStream_t s);
 
 // The plain half-precision GEMM on the matrix cores (t3_gemm.hip): y [rows][cols] = x [rows][in] w[:, 0:cols] for
 // w [in][ldw], all f16 or all bf16, f32 accumulation, y row-contiguous. in a multiple of 32, ldw of 8, x and w 16-byte
 // aligned, in * ldw * 2 under 4 GiB (gemm_half_ok).
 hipError_t launch_gemm_half(const void* x, const void* w, void* y, uint32_t rows, uint32_t in, uint32_t cols, uint32_t ldw,
                             bool bf16, hipStream_t s);
+// the same product over a W_hat with format.finishOutput at its end: y [rows][out] in `dtype` from the prepared rows
+hipError_t launch_gemm_finish(const uint16_t* xp, const uint16_t* w_hat, const uint16_t* svh, void* y, uint32_t rows,
+                              uint32_t in, uint32_t out, int dtype, hipStream_t s);
 inline bool gemm_half_ok(uint64_t in, uint64_t ldw) {
     return in % 32u == 0u && ldw % 8u == 0u && in * ldw * 2u < (1ull << 32);
 }

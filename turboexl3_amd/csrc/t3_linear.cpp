@@ -105,7 +105,6 @@ bool takes_w_hat(const DenseLaunch& l) {
 struct WhatScratch {
     uint16_t* w_hat;  // f16 [in][out]
     uint16_t* xp;     // f16 [rows][in], natural order
-    uint16_t* z;      // f16 [rows][out]
 };
 
 WhatScratch carve_dense_w_hat(DenseCall* call, void* workspace) {
@@ -115,17 +114,14 @@ WhatScratch carve_dense_w_hat(DenseCall* call, void* workspace) {
     WhatScratch w;
     w.w_hat = c.take<uint16_t>(static_cast<size_t>(l.in) * l.out * 2u);
     w.xp = c.take<uint16_t>(static_cast<size_t>(l.rows) * l.in * 2u);
-    w.z = c.take<uint16_t>(static_cast<size_t>(l.rows) * l.out * 2u);
     call->workspace = c.used;
     return w;
 }
 
-// prepare (natural order) -> z = f16(xp W_hat) -> finish, over a W_hat that is already there
-int32_t run_over_w_hat(const DenseLaunch& l, const uint16_t* w_hat, uint16_t* xp, uint16_t* z, hipStream_t s) {
+// prepare (natural order) -> finish(z = f16(xp W_hat)): the product and the finish are one launch, z stays in LDS
+int32_t run_over_w_hat(const DenseLaunch& l, const uint16_t* w_hat, uint16_t* xp, hipStream_t s) {
     if (const int32_t st = hip_status(launch_dense_prep_natural(l, xp, s)); st != T3_OK) return st;
-    if (const int32_t st = hip_status(launch_gemm_half(xp, w_hat, z, l.rows, l.in, l.out, l.out, false, s)); st != T3_OK)
-        return st;
-    return hip_status(launch_dense_finish_half(l, z, s));
+    return hip_status(launch_gemm_finish(xp, w_hat, l.svh, l.y, l.rows, l.in, l.out, l.dtype, s));
 }
 
 int32_t run_w_hat(const DenseCall& call, const WhatScratch& w, int codebook, hipStream_t s) {
@@ -133,7 +129,7 @@ int32_t run_w_hat(const DenseCall& call, const WhatScratch& w, int codebook, hip
     if (const int32_t st = hip_status(launch_dequant(l.trellis, w.w_hat, l.in, l.out, l.n, l.wbits, codebook, s));
         st != T3_OK)
         return st;
-    return run_over_w_hat(l, w.w_hat, w.xp, w.z, s);
+    return run_over_w_hat(l, w.w_hat, w.xp, s);
 }
 
 // The operand checks of a call over a kept W_hat f16 [in, out]: `check_dense`'s, with the W_hat in the trellis's place.
@@ -182,13 +178,12 @@ int32_t check_resident(const t3_array* x, const t3_array* w_hat, const t3_array*
 }
 
 // arrival counters (untouched here: a workspace's head stays zero whoever is called with it), xp f16 [rows][in]
-// (natural order), z f16 [rows][out]
-void carve_resident(DenseCall* call, void* workspace, uint16_t** xp, uint16_t** z) {
+// (natural order)
+void carve_resident(DenseCall* call, void* workspace, uint16_t** xp) {
     DenseLaunch& l = call->launch;
     Carver c(workspace);
     l.arrive = c.take<uint32_t>(kCounterBytes);
     *xp = c.take<uint16_t>(static_cast<size_t>(l.rows) * l.in * 2u);
-    *z = c.take<uint16_t>(static_cast<size_t>(l.rows) * l.out * 2u);
     call->workspace = c.used;
 }
 
@@ -270,7 +265,7 @@ int32_t t3_linear_plan_of(const t3_array* x, const t3_array* trellis, t3_decode 
         const uint32_t item_rows = l.rows <= 64u ? 64u : 128u, items = (l.rows + item_rows - 1u) / item_rows;
         p.workgroups = t3::dense_prefill_workgroups(l.out, items) * l.ks;
     } else {
-        p.launches = 4;
+        p.launches = 3;  // W_hat decode, prepare, the GEMM that finishes
         p.k_slices = 1;
     }
     *plan = p;
@@ -355,8 +350,8 @@ int32_t t3_linear_resident_workspace_bytes(const t3_array* x, const t3_array* w_
     if (!bytes) return T3_BadArgs;
     t3::DenseCall call;
     if (const int32_t st = t3::check_resident(x, w_hat, nullptr, nullptr, nullptr, &call); st != T3_OK) return st;
-    uint16_t *xp, *z;
-    t3::carve_resident(&call, nullptr, &xp, &z);
+    uint16_t* xp;
+    t3::carve_resident(&call, nullptr, &xp);
     *bytes = call.workspace;
     return T3_OK;
 }
@@ -367,11 +362,10 @@ int32_t t3_linear_resident(t3_stream stream, const t3_array* x, const t3_array* 
     t3::DenseCall call;
     if (const int32_t st = t3::check_resident(x, w_hat, suh, svh, y, &call); st != T3_OK) return st;
     if (!t3::workspace_ok(workspace)) return T3_BadArgs;
-    uint16_t *xp, *z;
-    t3::carve_resident(&call, workspace, &xp, &z);
+    uint16_t* xp;
+    t3::carve_resident(&call, workspace, &xp);
     if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
-    return t3::run_over_w_hat(call.launch, static_cast<const uint16_t*>(w_hat->data), xp, z,
-                              static_cast<hipStream_t>(stream));
+    return t3::run_over_w_hat(call.launch, static_cast<const uint16_t*>(w_hat->data), xp, static_cast<hipStream_t>(stream));
 }
 
 int32_t t3_unrot_workspace_bytes(const t3_array* trellis, size_t* bytes) {

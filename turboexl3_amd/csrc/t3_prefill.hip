@@ -593,9 +593,9 @@ __global__ void __launch_bounds__(256) pf_dense_prep(const void* x, const uint16
 }
 
 // the dense finish: z f32 [ks][rows][out], the planes summed in part order, with xs [rows][in / 128] for MUL1's deferred
-// map; or (HALF) one plane already rounded to f16 (format.innerGemv's rounding point) by a plain GEMM
-template <int DT, bool HALF>
-__global__ void __launch_bounds__(256) pf_dense_finish(const void* z, const float* xs, const uint16_t* svh, void* y,
+// map
+template <int DT>
+__global__ void __launch_bounds__(256) pf_dense_finish(const float* z, const float* xs, const uint16_t* svh, void* y,
                                                        uint32_t out, uint32_t rows, uint32_t inblk, int defer,
                                                        uint32_t ks) {
     const uint32_t nb = out / 128u, groups = (nb + kPfUnit - 1u) / kPfUnit;
@@ -607,20 +607,16 @@ __global__ void __launch_bounds__(256) pf_dense_finish(const void* z, const floa
     const Row16 g16 = row16(lane);
     const size_t at = static_cast<size_t>(row) * out + i;
     float v[8], sv[8];
-    if constexpr (HALF) {
-        load8_half(static_cast<const uint16_t*>(z), at, v);
-    } else {
-        load8_f32(static_cast<const float*>(z), at, v);
-        const size_t plane = static_cast<size_t>(rows) * out;
-        for (uint32_t k = 1; k < ks; ++k) {
-            float part[8];
-            load8_f32(static_cast<const float*>(z) + k * plane, at, part);
+    load8_f32(z, at, v);
+    const size_t plane = static_cast<size_t>(rows) * out;
+    for (uint32_t k = 1; k < ks; ++k) {
+        float part[8];
+        load8_f32(z + k * plane, at, part);
 #pragma unroll
-            for (uint32_t r = 0; r < 8u; ++r) v[r] += part[r];
-        }
+        for (uint32_t r = 0; r < 8u; ++r) v[r] += part[r];
     }
     load8_half(svh, i, sv);
-    if (!HALF && defer) {
+    if (defer) {
         float xsum = 0.0f;
         for (uint32_t t = 0; t < inblk; ++t) xsum += xs[static_cast<size_t>(row) * inblk + t];
 #pragma unroll
@@ -644,15 +640,13 @@ hipError_t launch_pf_dense_prep(const DenseLaunch& d, uint16_t* xq, float* xs, h
     return hipGetLastError();
 }
 
-template <bool HALF>
-hipError_t launch_pf_dense_finish(const DenseLaunch& d, const void* z, hipStream_t s) {
+hipError_t launch_pf_dense_finish(const DenseLaunch& d, const float* z, hipStream_t s) {
     const dim3 grid = unit_grid(d.rows, d.out), block(256);
     const uint32_t inblk = d.in / 128u;
     const int defer = d.codebook == kMul1Defer ? 1 : 0;
-    const uint32_t ks = HALF ? 1u : d.ks;
-    if (d.dtype == kF32) hipLaunchKernelGGL((pf_dense_finish<kF32, HALF>), grid, block, 0, s, z, d.xs, d.svh, d.y, d.out, d.rows, inblk, defer, ks);
-    else if (d.dtype == kF16) hipLaunchKernelGGL((pf_dense_finish<kF16, HALF>), grid, block, 0, s, z, d.xs, d.svh, d.y, d.out, d.rows, inblk, defer, ks);
-    else hipLaunchKernelGGL((pf_dense_finish<kBf16, HALF>), grid, block, 0, s, z, d.xs, d.svh, d.y, d.out, d.rows, inblk, defer, ks);
+    if (d.dtype == kF32) hipLaunchKernelGGL(pf_dense_finish<kF32>, grid, block, 0, s, z, d.xs, d.svh, d.y, d.out, d.rows, inblk, defer, d.ks);
+    else if (d.dtype == kF16) hipLaunchKernelGGL(pf_dense_finish<kF16>, grid, block, 0, s, z, d.xs, d.svh, d.y, d.out, d.rows, inblk, defer, d.ks);
+    else hipLaunchKernelGGL(pf_dense_finish<kBf16>, grid, block, 0, s, z, d.xs, d.svh, d.y, d.out, d.rows, inblk, defer, d.ks);
     return hipGetLastError();
 }
 
@@ -764,10 +758,6 @@ hipError_t launch_dense_prep_natural(const DenseLaunch& d, uint16_t* xp, hipStre
     return launch_pf_dense_prep<true>(d, xp, nullptr, s);
 }
 
-hipError_t launch_dense_finish_half(const DenseLaunch& d, const uint16_t* z, hipStream_t s) {
-    return launch_pf_dense_finish<true>(d, z, s);
-}
-
 hipError_t launch_dense_prefill(const DenseLaunch& d, hipStream_t s) {
     hipError_t e;
     // the block sums feed MUL1's deferred map only
@@ -787,7 +777,7 @@ hipError_t launch_dense_prefill(const DenseLaunch& d, hipStream_t s) {
     g.plane = d.rows * d.out;
     const uint32_t item_rows = d.rows <= 64u ? 64u : 128u;
     if ((e = launch_gemm(g, d.codebook, (d.rows + item_rows - 1u) / item_rows, 1u, item_rows, s)) != hipSuccess) return e;
-    return launch_pf_dense_finish<false>(d, d.z, s);
+    return launch_pf_dense_finish(d, d.z, s);
 }
 
 }  // namespace t3
