@@ -110,11 +110,12 @@ typedef struct t3_config {
     int32_t mul1_defer;    /* 1 (default): MUL1's affine map applied once an output (src/core/dense.zig deferFor); 0: per weight */
     int32_t dense_gemm_rows; /* dense calls of this many rows or more decode W_hat once into the workspace and run a plain
                               * f16 GEMM (rocBLAS, opened at run time; absent: the trellis GEMM serves). Default 512; 0: never */
-    int32_t dense_rows_alone; /* 0 (default): above 32 rows a dense call's launch shape follows its rows (K parts at few rows,
-                               * the W_hat form at many), so a row's bytes can differ between calls of different row counts
-                               * (each within the bars). 1: every such call takes the trellis GEMM with one K part, and a
-                               * row's bytes ignore the call's other rows, as the reference's own GEMM holds them
-                               * (src/hip_tests.zig:876-879); few-row calls then run up to three times as long */
+    int32_t dense_rows_alone; /* 0 (default): rows 17..32 run the GEMV and above 32 rows a dense call's launch shape follows
+                               * its rows (K parts at few rows, the W_hat form at many), so a row's bytes can differ between
+                               * calls of different row counts (each within the bars). 1: every call above 16 rows takes the
+                               * trellis GEMM with one K part, and a row's bytes ignore the call's other rows, as the
+                               * reference's own GEMM holds them for 17, 40, 129 and 200 rows (src/hip_tests.zig:866-880);
+                               * few-row calls then run up to twice as long */
 } t3_config;
 
 /* The served configuration. */

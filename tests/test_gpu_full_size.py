@@ -124,30 +124,34 @@ def test_config5_shape_few_rows_on_the_trellis_gemm(oracle, t3):
 
 def test_config5_shape_rows_alone_configuration(oracle, t3):
     # The reference's own GEMM holds rows 0-16 of a 40-, 129- or 200-row call to the bytes of the 17-row call
-    # (src/hip_tests.zig:876-879). Here the launch shape above 32 rows follows the rows by default (sixteen K parts at 64
-    # rows of this shape, two at 600, the W_hat form from 512), so those bytes may differ between row counts;
-    # dense_rows_alone = 1 pins one K part on the trellis GEMM and gives the reference's invariant back.
+    # (src/hip_tests.zig:866-880). Here the served launch shape follows the rows (the GEMV up to 32, then sixteen K parts at
+    # 64 rows of this shape, two at 600, the W_hat form from 512), so those bytes may differ between row counts;
+    # dense_rows_alone = 1 sends every call above 16 rows to the trellis GEMM with one K part and gives the reference's
+    # invariant back, at its own row counts and beyond.
     in_f, out_f, n = 4096, 14336, 64
     rng = np.random.default_rng(0xC57)
     trellis, suh, svh = oracle.synth_linear(rng, in_f, out_f, n)
     d_t, d_suh, d_svh = dev_u16(trellis), dev_f16_bits(suh), dev_f16_bits(svh)
     x_dev, x_f32 = make_x(rng, 600, in_f, torch.bfloat16)
-    plans = {rows: t3.linear_plan(x_dev[:rows], d_t, t3.Decode.mcg) for rows in (64, 300, 600)}
+    plans = {rows: t3.linear_plan(x_dev[:rows], d_t, t3.Decode.mcg) for rows in (17, 64, 300, 600)}
     assert [plans[r]["k_slices"] for r in (64, 300, 600)] == [16, 4, 1] and plans[600]["path"] == 4
+    assert plans[17]["path"] == 2  # the GEMV's chain
     t3.configure(dense_rows_alone=1)
     try:
         first = None
-        for rows in (33, 64, 300, 600):
+        for rows in (17, 40, 129, 200, 33, 64, 300, 600):
             plan = t3.linear_plan(x_dev[:rows], d_t, t3.Decode.mcg)
-            assert (plan["path"], plan["k_slices"]) == (3, 1)
+            assert (plan["path"], plan["k_slices"]) == (3, 1), rows
             y = t3.linear(x_dev[:rows], d_t, d_suh, d_svh, t3.Decode.mcg)
-            first = bytes_of(y[:33]) if first is None else first
-            assert bytes_of(y[:33]) == first, f"rows 0-32 of {rows} rows differ from the 33-row call"
+            first = bytes_of(y[:17]) if first is None else first
+            assert bytes_of(y[:17]) == first, f"rows 0-16 of {rows} rows differ from the 17-row call"
         got = to_f32(y[[0, 32, 599]])
         for blk in (0, 57, out_f // 128 - 1):
             ref = block_ref(oracle, trellis, suh, svh, x_f32[[0, 32, 599]], in_f, n, MCG, blk)
             for i in range(3):
                 assert oracle.compare(got[i, 128 * blk:128 * blk + 128], ref[i]) <= BF16_DENSE_BAR
+        # decode rows keep the GEMV under the switch
+        assert t3.linear_plan(x_dev[:16], d_t, t3.Decode.mcg)["path"] == 2
     finally:
         t3.configure()
 

@@ -94,6 +94,10 @@ void carve_dense_prefill(DenseCall* call, void* workspace) {
 }
 
 constexpr uint32_t kGemvRowsMax = 32;
+// The rows the GEMV serves in the configuration at hand. dense_rows_alone = 1 hands rows 17..32 to the trellis GEMM too:
+// every row count above 16 then runs one kernel with one K order, and rows 0..16 of a 17-, 40-, 129- or 200-row call
+// share their bytes as the reference's own GEMM holds them (src/hip_tests.zig:866-880).
+uint32_t gemv_rows_max() { return config().dense_rows_alone ? 16u : kGemvRowsMax; }
 
 // From dense_gemm_rows rows up a dense call decodes W_hat once and multiplies plainly (src/core/dense.zig:909-922,
 // 1290-1302): the decode is paid once a call, not once a 64-row item.
@@ -204,7 +208,7 @@ int32_t run_chain(const DenseCall& call, hipStream_t s, uint32_t stages) {
 // 32 rows the planes' coherent traffic costs the arriving form more than the finish launch it saves. The forms give the
 // same bytes.
 int dense_path(const DenseLaunch& l) {
-    if (l.rows > kGemvRowsMax) return takes_w_hat(l) ? T3_DENSE_W_HAT_GEMM : T3_DENSE_TRELLIS_GEMM;
+    if (l.rows > gemv_rows_max()) return takes_w_hat(l) ? T3_DENSE_W_HAT_GEMM : T3_DENSE_TRELLIS_GEMM;
     const uint32_t per = (l.in / 16u) / (4u * l.ks);
     if (!config().dec_one || l.rows > (l.bt == 8u ? 2u : 1u)) return T3_DENSE_CHAIN;
     return per % 8u == 0u && per <= 16u ? T3_DENSE_ONE_LAUNCH : T3_DENSE_ARRIVE;
@@ -228,8 +232,8 @@ int32_t t3_linear_workspace_bytes(const t3_array* x, const t3_array* trellis, t3
     if (!bytes) return T3_BadArgs;
     t3::DenseCall call;
     if (const int32_t st = t3::check_dense(x, trellis, nullptr, nullptr, dec, nullptr, 0, &call); st != T3_OK) return st;
-    if (call.launch.rows > t3::kGemvRowsMax && t3::takes_w_hat(call.launch)) t3::carve_dense_w_hat(&call, nullptr);
-    else if (call.launch.rows > t3::kGemvRowsMax) t3::carve_dense_prefill(&call, nullptr);
+    if (call.launch.rows > t3::gemv_rows_max() && t3::takes_w_hat(call.launch)) t3::carve_dense_w_hat(&call, nullptr);
+    else if (call.launch.rows > t3::gemv_rows_max()) t3::carve_dense_prefill(&call, nullptr);
     else t3::carve_dense(&call, nullptr);
     *bytes = call.workspace;
     return T3_OK;
@@ -240,7 +244,7 @@ int32_t t3_linear_plan_of(const t3_array* x, const t3_array* trellis, t3_decode 
     t3::DenseCall call;
     if (const int32_t st = t3::check_dense(x, trellis, nullptr, nullptr, dec, nullptr, 0, &call); st != T3_OK) return st;
     t3::DenseLaunch& l = call.launch;
-    if (l.rows > t3::kGemvRowsMax && !t3::config().prefill) return T3_Exl3EngineNotImplemented;
+    if (l.rows > t3::gemv_rows_max() && !t3::config().prefill) return T3_Exl3EngineNotImplemented;
     const int path = t3::dense_path(l);
     if (path == T3_DENSE_W_HAT_GEMM) t3::carve_dense_w_hat(&call, nullptr);
     else if (path == T3_DENSE_TRELLIS_GEMM) t3::carve_dense_prefill(&call, nullptr);
@@ -297,7 +301,7 @@ int32_t t3_linear(t3_stream stream, const t3_array* x, const t3_array* trellis, 
     t3::DenseCall call;
     if (const int32_t st = t3::check_dense(x, trellis, suh, svh, dec, y, 0, &call); st != T3_OK) return st;
     if (!t3::workspace_ok(workspace)) return T3_BadArgs;
-    if (call.launch.rows > t3::kGemvRowsMax) {
+    if (call.launch.rows > t3::gemv_rows_max()) {
         if (!t3::config().prefill) return T3_Exl3EngineNotImplemented;
         if (t3::takes_w_hat(call.launch)) {
             const t3::WhatScratch w = t3::carve_dense_w_hat(&call, workspace);
@@ -495,7 +499,7 @@ int32_t t3_linear_static(t3_stream stream, const t3_array* x, const t3_array* tr
     t3::DenseCall call;
     if (const int32_t st = t3::check_dense(x, trellis, suh, svh, dec, y, 0, &call); st != T3_OK) return st;
     // decode rows only: above them `t3_linear` may run a library GEMM, which allocates
-    if (call.launch.rows > t3::kGemvRowsMax) return T3_Exl3EngineNotImplemented;
+    if (call.launch.rows > t3::gemv_rows_max()) return T3_Exl3EngineNotImplemented;
     t3::carve_dense(&call, nullptr);
     if (call.workspace > static_cast<size_t>(T3_STATIC_SCRATCH_BYTES)) return T3_WorkspaceTooSmall;
     unsigned char* base = nullptr;
