@@ -429,6 +429,9 @@ int32_t t3_test_codebooks(t3_stream stream, uint16_t* mcg, uint16_t* mul1, uint1
 /* trellis: device u16 [tiles, n]; cw, mcg, mul1: device u16 [tiles, 256] by code position. */
 int32_t t3_test_lane(t3_stream stream, const uint16_t* trellis, int64_t n, int32_t window_bits, int64_t tiles,
                      uint16_t* cw, uint16_t* mcg, uint16_t* mul1);
+/* in: device f32 [count]; bf16, f16: device u16 [count]: each value narrowed as the kernels narrow an output (nearest even;
+ * a NaN stays a quiet NaN: src/test_support.zig:14-19); back: device f32 [count]: the bf16 widened again. */
+int32_t t3_test_convert(t3_stream stream, const float* in, uint16_t* bf16, uint16_t* f16, float* back, int64_t count);
 /* a f16 [16, 32], b f16 [32, 16] (bits), d f32 [16, 16] = a b through the kernels' MFMA fragments. */
 int32_t t3_test_mfma(t3_stream stream, const uint16_t* a, const uint16_t* b, float* d);
 

@@ -85,3 +85,32 @@ def test_dequant_refusals(t3):
     with pytest.raises(t3.T3Error) as e:
         t3.dequant(tr.to(torch.int32), t3.Decode.mcg)
     assert e.value.name == "BadExl3Dtype"
+
+
+def test_narrowing_to_bf16_and_f16_against_the_oracle(t3, oracle):
+    # the kernels narrow an output with the hardware's f32 -> bf16 / f16 conversions; held to the oracle's rule
+    # (nearest even, a NaN stays a quiet NaN with its sign and top payload bits: src/test_support.zig:14-19) on exact ties
+    # either way, the neighbours of every tie, overflow to infinity, subnormals, signed zeros, infinities and NaNs, and
+    # on a million random bit patterns
+    rng = np.random.default_rng(0xBF16)
+    base = rng.integers(0, 1 << 16, 4096, dtype=np.uint32) << 16            # exact bf16 values
+    ties = np.concatenate([base | 0x8000, (base | 0x8000) + 1, (base | 0x8000) - 1])
+    special = np.array([0x00000000, 0x80000000, 0x7F800000, 0xFF800000, 0x7FC00000, 0xFFC00001, 0x7F800001, 0xFF80FFFF,
+                        0x7FFFFFFF, 0x7F7FFFFF, 0xFF7FFFFF, 0x7F7F8000, 0x7F7F7FFF, 0x00000001, 0x00008000, 0x00018000,
+                        0x007FFFFF, 0x80008000, 0x3F808000, 0x3F818000, 0x477FE000, 0x477FF000, 0x33000000, 0x33800000],
+                       dtype=np.uint32)
+    bits = np.concatenate([ties.astype(np.uint32), special, rng.integers(0, 1 << 32, 1 << 20, dtype=np.uint64).astype(np.uint32)])
+    vals = torch.from_numpy(bits.view(np.int32)).cuda().view(torch.float32)
+    bf, hf, back = t3.test_convert(vals)
+    L = oracle.lib()
+    want_bf = np.fromiter((L.t3o_f32_to_bf16(float(v)) if v == v else 0 for v in bits.view(np.float32)), dtype=np.uint16,
+                          count=bits.size)
+    nan = np.isnan(bits.view(np.float32))
+    want_bf[nan] = ((bits[nan] >> 16) | 0x40).astype(np.uint16)              # ctypes would canonicalise a NaN argument
+    assert np.array_equal(host_u16(bf), want_bf)
+    got_hf = host_u16(hf)
+    with np.errstate(over="ignore"):
+        want_hf = bits.view(np.float32).astype(np.float16).view(np.uint16)
+    assert np.array_equal(got_hf[~nan], want_hf[~nan])
+    assert np.isnan(got_hf[nan].view(np.float16)).all()
+    assert np.array_equal(back.cpu().numpy().view(np.uint32), host_u16(bf).astype(np.uint32) << 16)

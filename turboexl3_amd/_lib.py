@@ -132,6 +132,7 @@ SYMBOLS = {
     "t3_test_codebooks": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "t3_test_lane": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int64, C.c_void_p, C.c_void_p,
                                  C.c_void_p]),
+    "t3_test_convert": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64]),
     "t3_test_mfma": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
 }
 

@@ -422,6 +422,16 @@ def test_lane(trellis: torch.Tensor, n: int, window_bits: int):
     return cw, mcg, mul1
 
 
+def test_convert(values: torch.Tensor):
+    """f32 values through the kernels' narrowing: (bf16 bits, f16 bits, the bf16 widened back to f32)."""
+    n = values.numel()
+    bf = torch.empty(n, dtype=torch.int16, device=values.device)
+    hf = torch.empty_like(bf)
+    back = torch.empty(n, dtype=torch.float32, device=values.device)
+    _check(_lib.lib().t3_test_convert(_stream_ptr(None), values.data_ptr(), bf.data_ptr(), hf.data_ptr(), back.data_ptr(), n))
+    return bf, hf, back
+
+
 def test_mfma(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     d = torch.empty(16, 16, dtype=torch.float32, device=a.device)
     _check(_lib.lib().t3_test_mfma(_stream_ptr(None), a.data_ptr(), b.data_ptr(), d.data_ptr()))

@@ -98,6 +98,13 @@ int32_t t3_test_lane(t3_stream stream, const uint16_t* trellis, int64_t n, int32
                                                mul1, static_cast<hipStream_t>(stream)));
 }
 
+int32_t t3_test_convert(t3_stream stream, const float* in, uint16_t* bf16, uint16_t* f16, float* back, int64_t count) {
+    if (!in || !bf16 || !f16 || !back) return T3_BadArgs;
+    if (count <= 0 || count > (1 << 28)) return T3_BadExl3Shape;
+    return t3::hip_status(t3::launch_test_convert(in, bf16, f16, back, static_cast<uint32_t>(count),
+                                                  static_cast<hipStream_t>(stream)));
+}
+
 int32_t t3_test_mfma(t3_stream stream, const uint16_t* a, const uint16_t* b, float* d) {
     if (!a || !b || !d) return T3_BadArgs;
     return t3::hip_status(t3::launch_test_mfma(a, b, d, static_cast<hipStream_t>(stream)));

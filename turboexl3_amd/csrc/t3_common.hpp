@@ -53,15 +53,18 @@ __device__ __forceinline__ uint16_t half_bits(float v) {
 }
 __device__ __forceinline__ float round_half(float v) { return half_value(half_bits(v)); }
 
+// bf16 is the top half of an f32. Narrowing is the hardware's (gfx950 converts f32 -> bf16 to nearest even in one
+// instruction, v_cvt_pk_bf16_f32, which is what the cast below compiles to); a NaN is kept apart so that it leaves with
+// its own sign and top payload bits and the quiet bit set, the host-side rule the outputs are checked against
+// (turboexl3 src/test_support.zig:14-19).
+typedef __bf16 bf16_t;
 __device__ __forceinline__ float bf16_value(uint16_t b) {
-    return __builtin_bit_cast(float, static_cast<uint32_t>(b) << 16);
+    return static_cast<float>(__builtin_bit_cast(bf16_t, b));
 }
-// f32 -> bf16, nearest even; a NaN stays a (quiet) NaN
 __device__ __forceinline__ uint16_t bf16_bits(float v) {
-    uint32_t u = __builtin_bit_cast(uint32_t, v);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return static_cast<uint16_t>(u >> 16);
+    const uint16_t nearest = __builtin_bit_cast(uint16_t, static_cast<bf16_t>(v));
+    const uint16_t quiet = static_cast<uint16_t>(__builtin_bit_cast(uint32_t, v) >> 16) | 0x40u;
+    return v != v ? quiet : nearest;
 }
 
 template <int DT>

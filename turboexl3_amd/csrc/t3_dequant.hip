@@ -98,6 +98,23 @@ hipError_t launch_test_lane(const uint32_t* trellis, uint32_t n, uint32_t wbits,
     return hipGetLastError();
 }
 
+namespace {
+// Grid (ceil(count / 256)), 256 threads: every value through the kernels' own narrowing and widening
+__global__ void __launch_bounds__(256) test_convert_kernel(const float* in, uint16_t* bf16, uint16_t* f16, float* back,
+                                                           uint32_t count) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= count) return;
+    bf16[i] = bf16_bits(in[i]);
+    f16[i] = half_bits(in[i]);
+    back[i] = bf16_value(bf16[i]);
+}
+}  // namespace
+
+hipError_t launch_test_convert(const float* in, uint16_t* bf16, uint16_t* f16, float* back, uint32_t count, hipStream_t s) {
+    hipLaunchKernelGGL(test_convert_kernel, dim3((count + 255u) / 256u), dim3(256), 0, s, in, bf16, f16, back, count);
+    return hipGetLastError();
+}
+
 hipError_t launch_test_mfma(const uint16_t* a, const uint16_t* b, float* d, hipStream_t s) {
     hipLaunchKernelGGL(test_mfma_kernel, dim3(1), dim3(64), 0, s, a, b, d);
     return hipGetLastError();

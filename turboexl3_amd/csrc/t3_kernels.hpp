@@ -184,6 +184,8 @@ hipError_t launch_unrot(const uint16_t* w_hat, float* r, const uint16_t* suh, co
 hipError_t launch_test_codebooks(uint16_t* mcg, uint16_t* mul1, uint16_t* t, hipStream_t s);
 hipError_t launch_test_lane(const uint32_t* trellis, uint32_t n, uint32_t wbits, uint32_t tiles, uint16_t* cw,
                             uint16_t* mcg, uint16_t* mul1, hipStream_t s);
+// test kernel: the kernels' f32 -> bf16 and f32 -> f16 narrowing and bf16 -> f32 widening of `count` values
+hipError_t launch_test_convert(const float* in, uint16_t* bf16, uint16_t* f16, float* back, uint32_t count, hipStream_t s);
 // test kernel: D = A B through the GEMV's MFMA with the fragments the kernels assume
 hipError_t launch_test_mfma(const uint16_t* a, const uint16_t* b, float* d, hipStream_t s);
 
