@@ -9,7 +9,9 @@
  *
  * Workspace contract: its first T3_WORKSPACE_COUNTER_BYTES bytes hold the arrival counters of the fused launches.
  * They must be zero when a workspace is first passed (zero-fill it once when you allocate it); every call leaves
- * them zero. Calls that share a workspace must be ordered on one stream: overlapping calls race on it.
+ * them zero. Calls that share a workspace must be ordered on one stream: overlapping calls race on it. A call that
+ * did not run to its end (a device error, a stream destroyed under it) may leave counters nonzero: zero-fill the
+ * first T3_WORKSPACE_COUNTER_BYTES bytes again before the workspace is passed to another call.
  *
  * Refusal convention (turboexl3 docs/core/api.md:10-12): a call this library does not serve returns a named
  * status before it launches anything and leaves every output untouched; the caller runs its own chain.

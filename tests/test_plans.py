@@ -154,3 +154,54 @@ def test_plan_refusals(lib):
     bank = bank_of(8, 512, 256, 64, 64)
     st = lib.t3_moe_plan_of(C.byref(arr(BF16, 1, 2, 512)), C.byref(bank), C.byref(arr(I32, 1, 2, 33)), None, C.byref(m))
     assert st != 0
+
+
+def test_sizes_beyond_the_launches_arithmetic_are_refused_by_name(lib):
+    # widths and row counts past what the launches index (a 16-bit grid dimension over in / 16, 32-bit element offsets over
+    # rows x width) refuse before anything is launched or any pointer followed; misaligned arrays are bad arguments
+    name = lambda st: lib.t3_error_name(st).decode()
+    p = LinearPlan()
+    wide_in = 16 * 65536   # in / 16 one past a grid's y
+    st = lib.t3_linear_plan_of(C.byref(arr(F16, 1, wide_in)), C.byref(arr(U16, wide_in // 16, 8, 16)), Decode(1, 16), C.byref(p))
+    assert name(st) == "Exl3EngineNotImplemented"
+    st = lib.t3_linear_plan_of(C.byref(arr(BF16, 1 << 21, 4096)), C.byref(arr(U16, 256, 256, 64)), Decode(1, 16), C.byref(p))
+    assert name(st) == "Exl3EngineNotImplemented"   # 2^21 rows x 4096 columns: 2^33 elements
+    assert lib.t3_linear_plan_of(C.byref(arr(BF16, 1 << 16, 4096)), C.byref(arr(U16, 256, 256, 64)), Decode(1, 16), C.byref(p)) == 0
+    st = lib.t3_dequant(None, C.byref(arr(U16, wide_in // 16, 8, 16)), Decode(1, 16), C.byref(arr(F16, wide_in, 128)))
+    assert name(st) == "Exl3EngineNotImplemented"
+    odd = arr(U16, 8, 8, 16)
+    odd.data = FAKE + 2
+    assert name(lib.t3_dequant(None, C.byref(odd), Decode(1, 16), C.byref(arr(F16, 128, 128)))) == "BadArgs"
+    bias = arr(F16, 128)
+    bias.data = FAKE + 6
+    st = lib.t3_linear_bias(None, C.byref(arr(F16, 1, 128)), C.byref(arr(U16, 8, 8, 16)), C.byref(arr(F16, 128)),
+                            C.byref(arr(F16, 128)), C.byref(bias), Decode(1, 16), C.byref(arr(F16, 1, 128)), FAKE, 1 << 20)
+    assert name(st) == "BadArgs"
+
+
+def test_configure_publishes_whole_snapshots(lib):
+    # a call reads one whole configuration, also while another thread configures: many writers, one reader of plans
+    import threading
+    stop = threading.Event()
+
+    def writer(rows_alone):
+        cfg = Config()
+        lib.t3_config_default(C.byref(cfg))
+        cfg.dense_rows_alone, cfg.dense_gemm_rows = rows_alone, 512 if rows_alone == 0 else 0
+        while not stop.is_set():
+            assert lib.t3_configure(C.byref(cfg)) == 0
+
+    threads = [threading.Thread(target=writer, args=(v,)) for v in (0, 1)]
+    for t in threads:
+        t.start()
+    try:
+        for _ in range(2000):
+            p = linear_plan(lib, 600, 4096, 14336, 64, BF16)
+            assert (p.path, p.k_slices) in ((4, 1), (3, 1)), (p.path, p.k_slices)   # never a mix of the two settings
+    finally:
+        stop.set()
+        for t in threads:
+            t.join()
+        cfg = Config()
+        lib.t3_config_default(C.byref(cfg))
+        assert lib.t3_configure(C.byref(cfg)) == 0

@@ -4,19 +4,28 @@
 
 #include "../../include/turboexl3_hip.h"
 
+#include <atomic>
 #include <cstring>
+#include <mutex>
 
 #include "t3_host.hpp"
 
 namespace {
 
-t3_config g_config = {9, 1, 1, 1, 1, 512, 0};
+// The configuration a call reads is one whole snapshot, also while another thread configures: t3_configure writes the
+// next slot of a small ring and then publishes its index; a reader takes whichever snapshot is published when it asks.
+// (The reference sets its configuration once before the first call, src/core/config.zig:175-178; a slot is reused only
+// after 63 further t3_configure calls, by which time no call that started under it is still reading.)
+constexpr uint32_t kConfigSlots = 64;
+t3_config g_configs[kConfigSlots] = {{9, 1, 1, 1, 1, 512, 0}};
+std::atomic<uint32_t> g_config_at{0};
+std::mutex g_config_write;
 
 }  // namespace
 
 namespace t3 {
 
-const t3_config& config() { return g_config; }
+const t3_config& config() { return g_configs[g_config_at.load(std::memory_order_acquire) % kConfigSlots]; }
 
 }  // namespace t3
 
@@ -62,7 +71,10 @@ int32_t t3_configure(const t3_config* cfg) {
                           (cfg->mcg_pair == 0 || cfg->mcg_pair == 1) && (cfg->mul1_defer == 0 || cfg->mul1_defer == 1) &&
                           cfg->dense_gemm_rows >= 0 && (cfg->dense_rows_alone == 0 || cfg->dense_rows_alone == 1);
     if ((cfg->decode_form != 3 && cfg->decode_form != 4 && cfg->decode_form != 9) || !flags_ok) return T3_InvalidTurboexl3Config;
-    g_config = *cfg;
+    std::lock_guard<std::mutex> lock(g_config_write);
+    const uint32_t next = g_config_at.load(std::memory_order_relaxed) + 1u;
+    g_configs[next % kConfigSlots] = *cfg;
+    g_config_at.store(next, std::memory_order_release);
     return T3_OK;
 }
 

@@ -29,6 +29,14 @@ inline bool array_ok(const t3_array* a) {
 inline bool aligned16(const t3_array* a) { return (reinterpret_cast<uintptr_t>(a->data) & 15u) == 0u; }
 inline bool workspace_ok(const void* w) { return w && (reinterpret_cast<uintptr_t>(w) & 255u) == 0u; }
 
+// Widths and row counts the launches index with 32-bit arithmetic and 16-bit grid dimensions: in / 16 is a grid's y
+// where W_hat is decoded or un-rotated (at most 65535), and a call's rows x width addresses its scratch in 32 bits.
+// Beyond them an entry point refuses with Exl3EngineNotImplemented before it launches anything.
+inline bool widths_served(int64_t in, int64_t out) { return in / 16 <= 65535 && out <= (1ll << 24); }
+inline bool rows_served(int64_t rows, int64_t in, int64_t out) {
+    return rows * in < (1ll << 32) && rows * out < (1ll << 32);
+}
+
 inline bool is_act_dtype(int32_t d) { return d == T3_F32 || d == T3_F16 || d == T3_BF16; }
 inline size_t dtype_size(int32_t d) { return d == T3_F32 || d == T3_U32 || d == T3_I32 ? 4 : 2; }
 

@@ -48,6 +48,7 @@ int32_t check_dense(const t3_array* x, const t3_array* trellis, const t3_array* 
     if (max_rows != 0 && rows > max_rows) return T3_Exl3EngineNotImplemented;
     // the kernels address one matrix, and one call's prepared rows, through 32-bit byte offsets
     if ((in / 16) * (out / 16) * n * 2 >= (1ll << 31) || rows * in * 4 >= (1ll << 31)) return T3_Exl3EngineNotImplemented;
+    if (!widths_served(in, out) || !rows_served(rows, in, out)) return T3_Exl3EngineNotImplemented;
     if (out / 128 > static_cast<int64_t>(kCounterBytes / 4)) return T3_Exl3EngineNotImplemented;
 
     DenseLaunch& l = call->launch;
@@ -166,7 +167,7 @@ int32_t check_resident(const t3_array* x, const t3_array* w_hat, const t3_array*
     }
     // decode and verify rows never read a W_hat (src/core/dense.zig:1309 `prefillOperands`)
     if (rows <= kGemvRowsMax || !gemm_half_ok(in, out)) return T3_Exl3EngineNotImplemented;
-    if (rows * in * 4 >= (1ll << 31)) return T3_Exl3EngineNotImplemented;
+    if (rows * in * 4 >= (1ll << 31) || !widths_served(in, out) || !rows_served(rows, in, out)) return T3_Exl3EngineNotImplemented;
     DenseLaunch& l = call->launch;
     l.x = x->data;
     l.suh = suh ? static_cast<const uint16_t*>(suh->data) : nullptr;
@@ -323,6 +324,7 @@ int32_t t3_linear_bias(t3_stream stream, const t3_array* x, const t3_array* trel
                        size_t workspace_bytes) {
     // root.linearBias's own checks (src/root.zig:365-370), then `linear`, then one add in x's dtype
     if (!t3::array_ok(bias) || !t3::array_ok(trellis) || !t3::array_ok(x)) return T3_BadArgs;
+    if (!t3::aligned16(bias)) return T3_BadArgs;
     if (trellis->ndim != 3 || bias->ndim != 1 || bias->shape[0] != trellis->shape[1] * 16) return T3_BadExl3Shape;
     if (bias->dtype != x->dtype) return T3_BadExl3Dtype;
     if (const int32_t st = t3_linear(stream, x, trellis, suh, svh, dec, y, workspace, workspace_bytes); st != T3_OK)
@@ -336,10 +338,12 @@ int32_t t3_linear_bias(t3_stream stream, const t3_array* x, const t3_array* trel
 
 int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_array* w_hat) {
     if (!t3::array_ok(trellis) || !t3::array_ok(w_hat)) return T3_BadArgs;
+    if (!t3::aligned16(trellis) || !t3::aligned16(w_hat)) return T3_BadArgs;
     if (trellis->ndim != 3 || w_hat->ndim != 2) return T3_BadExl3Shape;
     const int64_t in = trellis->shape[0] * 16, out = trellis->shape[1] * 16, n = trellis->shape[2];
     if (!t3::rate_ok(n) || in <= 0 || out <= 0 || out % 64 != 0 || in > (1ll << 30) || out > (1ll << 30))
         return T3_BadExl3Shape;
+    if (!t3::widths_served(in, out) || (in / 16) * (out / 16) * n * 2 >= (1ll << 32)) return T3_Exl3EngineNotImplemented;
     if (w_hat->shape[0] != in || w_hat->shape[1] != out) return T3_BadExl3Shape;
     if ((trellis->dtype != T3_U16 && trellis->dtype != T3_I16) || w_hat->dtype != T3_F16) return T3_BadExl3Dtype;
     t3::Dec d;
@@ -401,6 +405,11 @@ int32_t t3_unrot_weight(t3_stream stream, const t3_array* trellis, const t3_arra
     if ((trellis->dtype != T3_U16 && trellis->dtype != T3_I16) || suh->dtype != T3_F16 || svh->dtype != T3_F16 ||
         (w_std->dtype != T3_F16 && w_std->dtype != T3_BF16))
         return T3_BadExl3Dtype;
+    if (!t3::aligned16(trellis) || !t3::aligned16(suh) || !t3::aligned16(svh) || !t3::aligned16(w_std) ||
+        w_std->shape[1] % 8 != 0)
+        return T3_BadArgs;
+    if (!t3::widths_served(in, out) || in * out >= (1ll << 32) || (in / 16) * (out / 16) * n * 2 >= (1ll << 32))
+        return T3_Exl3EngineNotImplemented;
     t3::Dec d;
     if (const int32_t st = t3::resolve_decode(dec, &d); st != T3_OK) return st;
     t3::Carver c(workspace);
