@@ -68,6 +68,33 @@ def test_config2_qkv_shape_rows_1_4_16_32(oracle, t3, k):
         assert bytes_of(y[0]) == bytes_of(alone[0]), "row 0 differs from the row alone"
 
 
+def test_config2_qkv_shape_exact_weight_forms(oracle, t3):
+    # The served GEMV feeds MCG's hashed pair unrounded (mcg_pair) and MUL1's affine map once an output (mul1_defer): both
+    # differ from format.project's f16-rounded weight in the last bits of a product, the second as the reference's own
+    # kernels do (src/kernels/hip/common.hpp:95-104), the first this library's own form. With both switched off every
+    # weight is the format's f16 value: the q|k|v shape at K4, rows 1 and 32, both codebooks, held to the same bar, and the
+    # one launch still equal to its chain.
+    in_f, out_f, n = 4096, 12288, 64
+    rng = np.random.default_rng(0xC2E)
+    trellis, suh, svh = oracle.synth_linear(rng, in_f, out_f, n)
+    d_t, d_suh, d_svh = dev_u16(trellis), dev_f16_bits(suh), dev_f16_bits(svh)
+    x_dev, x_f32 = make_x(rng, 32, in_f, torch.float16, outliers=True)
+    t3.configure(mcg_pair=0, mul1_defer=0)
+    try:
+        for codebook, dec in ((MCG, t3.Decode.mcg), (MUL1, t3.Decode.mul1)):
+            w_hat = oracle.reconstruct_inner(trellis, in_f, out_f, n, codebook)
+            ref = oracle.project_rows(x_f32, trellis, suh, svh, in_f, out_f, n, codebook, 0xFFFF, threads=8, w_hat=w_hat)
+            for rows in (1, 32):
+                y = t3.linear(x_dev[:rows], d_t, d_suh, d_svh, dec)
+                got = to_f32(y)
+                worst = max(oracle.compare(got[r], ref[r], 2.0 ** -11) for r in range(rows))
+                assert worst <= F32_BAR, f"codebook {codebook} rows {rows}: {worst:.3e}"
+                if rows == 1:
+                    assert bytes_of(y) == bytes_of(t3.linear_chain(x_dev[:1], d_t, d_suh, d_svh, dec))
+    finally:
+        t3.configure()
+
+
 def test_config5_lm_head_k6_rows_1_and_256(oracle, t3):
     in_f, out_f, n = 4096, 151936, 96
     rng = np.random.default_rng(0xC5)
