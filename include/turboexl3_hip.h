@@ -110,8 +110,8 @@ typedef struct t3_config {
     int32_t prefill;       /* 1 (default); 0: routed calls above 16 rows refuse Exl3EngineNotImplemented */
     int32_t mcg_pair;      /* 1 (default): MCG's GEMV feeds the hashed pair to the matrix core unrounded; 0: the f16 weight */
     int32_t mul1_defer;    /* 1 (default): MUL1's affine map applied once an output (src/core/dense.zig deferFor); 0: per weight */
-    int32_t dense_gemm_rows; /* dense calls of this many rows or more decode W_hat once into the workspace and run a plain
-                              * f16 GEMM (rocBLAS, opened at run time; absent: the trellis GEMM serves). Default 512; 0: never */
+    int32_t dense_gemm_rows; /* dense calls of this many rows or more decode W_hat once into the workspace and run this
+                              * library's plain f16 GEMM, which ends with the finish. Default 512; 0: never */
     int32_t dense_rows_alone; /* 0 (default): rows 17..32 run the GEMV and above 32 rows a dense call's launch shape follows
                                * its rows (K parts at few rows, the W_hat form at many), so a row's bytes can differ between
                                * calls of different row counts (each within the bars). 1: every call above 16 rows takes the
@@ -205,9 +205,9 @@ int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_
 
 /* The resident W_hat (src/core/dense.zig:1323-1345, a host's opt-in: memory for compute): `t3_linear` above
  * t3_config.dense_gemm_rows rows decodes the whole trellis to W_hat on every call; a host that keeps the W_hat of
- * `t3_dequant` calls this instead: prepare, one plain f16 GEMM (rocBLAS, opened at run time), finish, the same launches
- * on the same operands, so y is `t3_linear`'s W_hat form byte for byte. w_hat F16 [in, out]. Up to 32 rows, and without
- * rocBLAS, it refuses with T3_Exl3EngineNotImplemented: decode and verify rows never read a W_hat (dense.zig:1309). */
+ * `t3_dequant` calls this instead: prepare, then one plain f16 GEMM that ends with the finish, the same launches on the
+ * same operands, so y is `t3_linear`'s W_hat form byte for byte. w_hat F16 [in, out]. Up to 32 rows it refuses with
+ * T3_Exl3EngineNotImplemented: decode and verify rows never read a W_hat (dense.zig:1309). */
 int32_t t3_linear_resident_workspace_bytes(const t3_array* x, const t3_array* w_hat, size_t* bytes);
 int32_t t3_linear_resident(t3_stream stream, const t3_array* x, const t3_array* w_hat, const t3_array* suh,
                            const t3_array* svh, t3_array* y, void* workspace, size_t workspace_bytes);
@@ -224,7 +224,7 @@ int32_t t3_unrot_weight(t3_stream stream, const t3_array* trellis, const t3_arra
                         t3_decode dec, t3_array* w_std, int64_t col0, uint32_t* nonfinite, void* workspace,
                         size_t workspace_bytes);
 /* y [rows, cols] = x [rows, in] W_std[:, col0 : col0 + cols], x, w_std and y in one dtype (F16 or BF16), f32
- * accumulation: one plain GEMM (rocBLAS, opened at run time; without it T3_Exl3EngineNotImplemented). Up to 32 rows
+ * accumulation: one plain GEMM on the matrix cores (w_std's row length a multiple of 8, col0 of 8). Up to 32 rows
  * (src/core/dense.zig:1611 `unrot_min_rows`) it refuses with T3_Exl3EngineNotImplemented: decode and verify rows keep
  * the trellis paths byte for byte. */
 int32_t t3_linear_unrot(t3_stream stream, const t3_array* x, const t3_array* w_std, int64_t col0, int64_t cols,

@@ -28,7 +28,9 @@ def test_captured_calls_replay_to_the_eager_bytes(oracle, t3):
     dec = t3.Decode(MCG, 16)
 
     # static inputs, as a captured step keeps them; the rows of each call are views of one buffer a kind
-    x_dense = torch.zeros(40, in_f, dtype=torch.float16, device="cuda")
+    x_dense = torch.zeros(530, in_f, dtype=torch.float16, device="cuda")
+    w_hat = t3.dequant(d_t, dec)
+    w_std, _ = t3.unrot_weight(d_t, d_suh, d_svh, dec, torch.float16)
     x_moe = torch.zeros(1, 20, hidden, dtype=torch.bfloat16, device="cuda")
     slots = torch.zeros(1, 20, topk, dtype=torch.int32, device="cuda")
     scores = torch.zeros(1, 20, topk, dtype=torch.float32, device="cuda")
@@ -37,7 +39,11 @@ def test_captured_calls_replay_to_the_eager_bytes(oracle, t3):
         return [
             t3.linear(x_dense[:1], d_t, d_suh, d_svh, dec),          # one launch, its finish by the last arriver
             t3.linear(x_dense[:8], d_t, d_suh, d_svh, dec),          # the three-launch chain
-            t3.linear(x_dense, d_t, d_suh, d_svh, dec),              # 40 rows: the trellis GEMM
+            t3.linear(x_dense[:40], d_t, d_suh, d_svh, dec),         # 40 rows: the trellis GEMM
+            t3.linear(x_dense, d_t, d_suh, d_svh, dec),              # 530 rows: W_hat decoded, the f16 GEMM with its finish
+            t3.linear_resident(x_dense[:100], w_hat, d_suh, d_svh),  # the same GEMM over a kept W_hat
+            t3.linear_unrot(x_dense[:100], w_std),                   # the plain product over the un-rotated weight
+            t3.linear_static(x_dense[:3], d_t, d_suh, d_svh, dec),   # scratch in the library's own device array
             t3.moe_clamped(x_moe[:, :2], bank, slots[:, :2], scores[:, :2], dec, 7),   # two arriving launches
             t3.moe_clamped(x_moe, bank, slots, scores, dec, 7),      # 20 rows: route, GEMMs, combine
             t3.linear(x_dense[:1], d_t, d_suh, d_svh, t3.Decode(MUL1, 16)),
@@ -45,7 +51,7 @@ def test_captured_calls_replay_to_the_eager_bytes(oracle, t3):
 
     def new_inputs(seed):
         r = np.random.default_rng(seed)
-        xd, _ = make_x(r, 40, in_f, torch.float16, outliers=True)
+        xd, _ = make_x(r, 530, in_f, torch.float16, outliers=True)
         xm, _ = make_x(r, 20, hidden, torch.bfloat16)
         s, w = routing(r, 20, topk, experts)
         x_dense.copy_(xd)

@@ -171,7 +171,7 @@ def test_routed_prefill_clamp_skips_mixed_rates_shared(oracle, t3):
 def test_dense_w_hat_form_from_512_rows(oracle, t3, in_f, out_f, n, codebook, dtype):
     """From t3_config.dense_gemm_rows rows a dense call decodes W_hat once and multiplies with the library's f16 GEMM
     (the reference's dequant + matmul + finish, src/core/dense.zig:909-922,1290-1302; held to the same bars, as its
-    Metal form is in src/core/gpu_test.zig:394-438). Without rocBLAS the call stays on the trellis GEMM: same bars."""
+    Metal form is in src/core/gpu_test.zig:394-438)."""
     case = DenseCase(oracle, t3, 0xA11 + in_f + n, in_f, out_f, n, codebook)
     rows = 530
     x_dev, x_f32 = make_x(case.rng, rows, in_f, dtype, outliers=True)

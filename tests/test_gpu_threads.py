@@ -1,5 +1,5 @@
 """Host threads: the library keeps no per-call state of its own (partitions are functions of the shapes, scratch and
-streams are the caller's, the one rocBLAS handle sits behind a lock), so threads that bring their own stream and
+streams are the caller's), so threads that bring their own stream and
 workspace may call it at the same time (turboexl3 src/root.zig:155-160 keeps its caches behind spinlocks to the same
 end). Four threads issue mixed calls on their own streams; every result must equal the single-threaded one."""
 import threading
@@ -41,7 +41,7 @@ def test_threads_with_their_own_streams_and_workspaces(oracle, t3):
     def calls(w, stream):
         xd, xm, s, sc = inputs[w]
         out = []
-        for rows in (1, 7, 40, 600):  # one launch, chain, trellis GEMM, W_hat + the shared rocBLAS handle
+        for rows in (1, 7, 40, 600):  # one launch, chain, trellis GEMM, W_hat + the plain f16 GEMM
             out.append(t3.linear(xd[:rows], d_t, d_suh, d_svh, dec, stream=stream))
         out.append(t3.linear_resident(xd[:90], w_hat, d_suh, d_svh, stream=stream))
         out.append(t3.moe_clamped(xm[:, :3], bank, s[:, :3], sc[:, :3], dec, 7, stream=stream))
