@@ -8,11 +8,14 @@
 
 namespace t3 {
 
-// activation numbering shared with the C ABI (turboexl3 src/hip/plan.zig:72-73)
-enum Dtype : int { kF32 = 0, kF16 = 1, kBf16 = 2 };
+// Activation dtypes by the C ABI's t3_dtype numbers (T3_F32, T3_F16, T3_BF16), which are the reference plan's
+// (turboexl3 src/hip/plan.zig:72-73): a launch descriptor carries the caller's number straight through.
+enum Dtype : int { kF32, kF16, kBf16 };
+static_assert(kF32 == 0 && kF16 == 1 && kBf16 == 2, "the ABI's dtype numbers");
 
-constexpr float kHadScale = 0.08838834764831845f;  // 1 / sqrt(128)
 constexpr int kWave = 64;
+// a Hadamard-128 is orthonormal with this factor: 2^-3.5
+constexpr float kHadScale = 0.088388347648318440550105545263106f;
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
@@ -45,13 +48,16 @@ __device__ __forceinline__ float load_coherent(const float* p) {
 // every store this lane has issued is acknowledged at its coherence level (with store_coherent: device-wide)
 __device__ __forceinline__ void wait_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
+// ---- activation elements ----------------------------------------------------------------------------------------
+// f16 values travel as their 16-bit patterns where they are packed by hand (two to a register for the matrix core).
 __device__ __forceinline__ float half_value(uint32_t bits) {
     return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(bits)));
 }
 __device__ __forceinline__ uint16_t half_bits(float v) {
     return __builtin_bit_cast(uint16_t, static_cast<_Float16>(v));
 }
-__device__ __forceinline__ float round_half(float v) { return half_value(half_bits(v)); }
+// v rounded to the nearest f16 and back: format.project's rounding points (turboexl3 src/core/format.zig:144-146)
+__device__ __forceinline__ float round_half(float v) { return static_cast<float>(static_cast<_Float16>(v)); }
 
 // bf16 is the top half of an f32. Narrowing is the hardware's (gfx950 converts f32 -> bf16 to nearest even in one
 // instruction, v_cvt_pk_bf16_f32, which is what the cast below compiles to); a NaN is kept apart so that it leaves with
@@ -67,17 +73,35 @@ __device__ __forceinline__ uint16_t bf16_bits(float v) {
     return v != v ? quiet : nearest;
 }
 
+// How an activation dtype sits in memory and crosses to f32: one description a dtype, used by every typed load and
+// store of the kernels (a store rounds once, to nearest even).
 template <int DT>
-__device__ __forceinline__ float load_act(const void* p, size_t i) {
-    if constexpr (DT == kF32) return static_cast<const float*>(p)[i];
-    else if constexpr (DT == kF16) return half_value(static_cast<const uint16_t*>(p)[i]);
-    else return bf16_value(static_cast<const uint16_t*>(p)[i]);
+struct ActElem;
+template <>
+struct ActElem<kF32> {
+    typedef float Stored;
+    static __device__ __forceinline__ float widen(Stored s) { return s; }
+    static __device__ __forceinline__ Stored narrow(float v) { return v; }
+};
+template <>
+struct ActElem<kF16> {
+    typedef _Float16 Stored;
+    static __device__ __forceinline__ float widen(Stored s) { return static_cast<float>(s); }
+    static __device__ __forceinline__ Stored narrow(float v) { return static_cast<Stored>(v); }
+};
+template <>
+struct ActElem<kBf16> {
+    typedef uint16_t Stored;
+    static __device__ __forceinline__ float widen(Stored s) { return bf16_value(s); }
+    static __device__ __forceinline__ Stored narrow(float v) { return bf16_bits(v); }
+};
+template <int DT>
+__device__ __forceinline__ float load_act(const void* base, size_t index) {
+    return ActElem<DT>::widen(static_cast<const typename ActElem<DT>::Stored*>(base)[index]);
 }
 template <int DT>
-__device__ __forceinline__ void store_act(void* p, size_t i, float v) {
-    if constexpr (DT == kF32) static_cast<float*>(p)[i] = v;
-    else if constexpr (DT == kF16) static_cast<uint16_t*>(p)[i] = half_bits(v);
-    else static_cast<uint16_t*>(p)[i] = bf16_bits(v);
+__device__ __forceinline__ void store_act(void* base, size_t index, float v) {
+    static_cast<typename ActElem<DT>::Stored*>(base)[index] = ActElem<DT>::narrow(v);
 }
 
 // The unscaled Hadamard of a 128-block held by one wave64: lane L owns elements L and L + 64 (v[0], v[1]).
