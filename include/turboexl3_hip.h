@@ -269,8 +269,8 @@ int32_t t3_moe_shared_expert(t3_stream stream, const t3_array* x, const t3_bank*
 /* `t3_moe_shared_expert` (shared_bank NULL: `t3_moe_swiglu` at gate_in; limit 0: no clamp) with a choice of its
  * launches, for profilers and benchmarks that time one stage at a time (the role `t3_linear_stages` has for the dense
  * chain; src/hip/plan.zig:294-364,436-476 publishes the same launches one by one). The workspace carries the stages'
- * results between calls. Up to 16 rows in the two-launch form: bit 0 gate|up + mid, bit 1 down + combine (the four- and
- * five-launch forms run whole). Above: bit 0 the route, 1 prepare, 2 gate|up GEMM, 3 mid, 4 down GEMM, 5 combine. */
+ * results between calls. Up to 16 rows in the two-launch form: bit 0 gate|up + mid, bit 1 down + combine (one and two
+ * rows: the mid stage runs inside the down launch; the four- and five-launch forms run whole). Above: bit 0 the route, 1 prepare, 2 gate|up GEMM, 3 mid, 4 down GEMM, 5 combine. */
 #define T3_MOE_STAGE_GATE_UP 1u
 #define T3_MOE_STAGE_DOWN 2u
 #define T3_PREFILL_STAGE_ROUTE 1u

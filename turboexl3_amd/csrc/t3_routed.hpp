@@ -164,10 +164,10 @@ __device__ __forceinline__ void routed_prep_block(const MoeLaunch& a, uint32_t r
 
 // gate and up finishes, the (clamped) SwiGLU in f32 on their f16 values, and the down's prepare: hd [.][inter],
 // hs f32 [.][inter / 128]
+// the values of it: hh[j], the prepared f16 of element lane + 64 j of the block, and the block's sum of them
 template <bool PF, bool COH = false, int PROF = 0>
-__device__ __forceinline__ void routed_mid_block(const MoeLaunch& a, const SlotRef& s, uint32_t q, uint32_t b,
-                                                 uint32_t lane) {
-    if (!s.live) return;
+__device__ __forceinline__ void routed_mid_values(const MoeLaunch& a, const SlotRef& s, uint32_t q, uint32_t b,
+                                                  uint32_t lane, uint32_t (&hh)[2], float& sum) {
     const RoutedBank& bank = s.shared ? a.shared : a.bank;
     const uint32_t rkt = a.rows * (a.topk + a.shared_slots), nb = a.hidden / 128u;
     const uint32_t ks = PF ? 1u : a.ks_gu;
@@ -210,15 +210,26 @@ __device__ __forceinline__ void routed_mid_block(const MoeLaunch& a, const SlotR
         for (uint32_t j = 0; j < 2u; ++j) d[j] = swiglu_glm(g[j], u[j], a.limit) * sdn[j];
     }
     h128_wave(d, lane);
-    float sum = 0.0f;
+    sum = 0.0f;
 #pragma unroll
     for (uint32_t j = 0; j < 2u; ++j) {
-        const uint32_t hh = half_bits(d[j] * kHadScale);
-        store_prepared<PF>(a.hd, static_cast<size_t>(q) * a.inter, b * 128u + lane + 64u * j, hh);
-        sum += half_value(hh);
+        hh[j] = half_bits(d[j] * kHadScale);
+        sum += half_value(hh[j]);
     }
 #pragma unroll
     for (int m = 32; m > 0; m >>= 1) sum += __shfl_xor(sum, m, 64);
+}
+
+template <bool PF, bool COH = false, int PROF = 0>
+__device__ __forceinline__ void routed_mid_block(const MoeLaunch& a, const SlotRef& s, uint32_t q, uint32_t b,
+                                                 uint32_t lane) {
+    if (!s.live) return;
+    uint32_t hh[2];
+    float sum;
+    routed_mid_values<PF, COH, PROF>(a, s, q, b, lane, hh, sum);
+#pragma unroll
+    for (uint32_t j = 0; j < 2u; ++j)
+        store_prepared<PF>(a.hd, static_cast<size_t>(q) * a.inter, b * 128u + lane + 64u * j, hh[j]);
     if (lane == 0u) a.hs[static_cast<size_t>(q) * (a.inter / 128u) + b] = sum;
 }
 
