@@ -20,6 +20,8 @@
 // The role of each launch follows the reference's HIP plan (src/hip/plan.zig:161-204); the launch shapes, the lane
 // plan and the use of MFMA are this library's own.
 
+#include <type_traits>
+
 #include "t3_gemv_core.hpp"
 #include "t3_kernels.hpp"
 #include "t3_stages.hpp"
@@ -167,12 +169,36 @@ __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
         // dense_prep, into its LDS x stage [per + 1][4][64 bytes] (the last tile row zeros). The block sums go to the
         // column block's own copy of xs (deferred MUL1 map only; the block's second workgroup column, if any, would
         // store the same values again).
-        const uint32_t blocks = per >> 3;
-        for (uint32_t r = 0; r < rows; ++r)
-            for (uint32_t b = 0; b < blocks; ++b) {
+        // Every row's loads go out together (rows and blocks past the call's alias the last real one, so there is no
+        // branch among the loads): a further row then costs its butterfly, not another round trip.
+        const uint32_t blocks = per >> 3;  // 1 or 2
+        float raw[kXldsRows][2][2], sc[2][2];
+        auto load_rows = [&](auto tag) {
+            constexpr int DT = decltype(tag)::value;
+#pragma unroll
+            for (uint32_t b = 0; b < 2u; ++b)
+#pragma unroll
+                for (uint32_t j = 0; j < 2u; ++j) {
+                    const uint32_t i = ((tk0 >> 3) + (b < blocks ? b : blocks - 1u)) * 128u + lane + 64u * j;
+                    sc[b][j] = half_value(a.suh[i]);
+#pragma unroll
+                    for (uint32_t r = 0; r < kXldsRows; ++r)
+                        raw[r][b][j] = load_act<DT>(a.x, static_cast<size_t>(r < rows ? r : rows - 1u) * a.in + i);
+                }
+        };
+        if (a.dt == kF32) load_rows(std::integral_constant<int, kF32>{});
+        else if (a.dt == kF16) load_rows(std::integral_constant<int, kF16>{});
+        else load_rows(std::integral_constant<int, kBf16>{});
+#pragma unroll
+        for (uint32_t r = 0; r < kXldsRows; ++r) {
+            if (r >= rows) break;
+#pragma unroll
+            for (uint32_t b = 0; b < 2u; ++b) {
+                if (b >= blocks) break;
+                float v[2] = {round_half(raw[r][b][0]) * sc[b][0], round_half(raw[r][b][1]) * sc[b][1]};
                 uint32_t hv[2];
                 float sum;
-                prep_values(a.dt, a.x, a.suh, a.in, r, (tk0 >> 3) + b, lane, hv, sum);
+                prep_core(v, lane, hv, sum, a.defer != 0);
 #pragma unroll
                 for (uint32_t j = 0; j < 2u; ++j) {
                     const uint32_t i = lane + 64u * j;  // element of the block: tile row b 8 + i / 16
@@ -182,6 +208,7 @@ __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
                 if (a.defer && lane == 0u && blk % kShare == 0u)
                     store_coherent(a.xs + (static_cast<size_t>(b128) * rows + r) * inblk + (tk0 >> 3) + b, sum);
             }
+        }
         for (uint32_t i = lane; i < kXldsRows * 16u; i += 64u)
             *reinterpret_cast<uint32_t*>(xst + per * (kXldsRows * 64u) + i * 4u) = 0u;
         stream.run(acc);

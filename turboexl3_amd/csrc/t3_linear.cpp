@@ -201,17 +201,18 @@ int32_t run_chain(const DenseCall& call, hipStream_t s, uint32_t stages) {
     return T3_OK;
 }
 
-// The served form (src/core/dense.zig:1229-1242 takes DEC-ONE at its fewest rows the same way). One row (two at up to
-// four bits a weight, where a wave takes eight tiles a step): one launch where a wave's K part is whole 128-blocks and small enough to prepare
-// in LDS, else the prepare launch and the arriving GEMV. More rows: the chain. Measured at 4096 x 12288: the one launch
-// takes 14.8-17.1 us at one row against the chain's 16.7-18.0, but every further row adds 1-2 us to it (each workgroup
-// prepares every row and the last arriver finishes them one after the other) and nothing to the chain, and with 16 and
-// 32 rows the planes' coherent traffic costs the arriving form more than the finish launch it saves. The forms give the
-// same bytes.
+// The served form (src/core/dense.zig:1229-1242 takes DEC-ONE at its fewest rows the same way). Up to three rows where a
+// wave takes eight tiles a step (up to four bits a weight), up to two otherwise: one launch where a wave's K part is whole
+// 128-blocks and small enough to prepare in LDS, else the prepare launch and the arriving GEMV. More rows: the chain.
+// Measured at 4096 x 12288 (us a call, one launch against the chain): K4 14.4 / 13.9 / 14.4 / 15.2 against 15.8 / 15.0 /
+// 15.1 / 15.2 at 1 / 2 / 3 / 4 rows, K5 14.8 / 15.7 / 16.7 / 17.7 against 16.7 / 16.7 / 16.9 / 16.8: every workgroup
+// prepares every row of its K part (all rows' loads in flight together, then a butterfly a row) and the last arriver
+// finishes a row a wave, which the chain's two small launches do once; with 16 and 32 rows the planes' coherent traffic
+// costs the arriving form more than the finish launch it saves. The forms give the same bytes.
 int dense_path(const DenseLaunch& l) {
     if (l.rows > gemv_rows_max()) return takes_w_hat(l) ? T3_DENSE_W_HAT_GEMM : T3_DENSE_TRELLIS_GEMM;
     const uint32_t per = (l.in / 16u) / (4u * l.ks);
-    if (!config().dec_one || l.rows > (l.bt == 8u ? 2u : 1u)) return T3_DENSE_CHAIN;
+    if (!config().dec_one || l.rows > (l.bt == 8u ? 3u : 2u)) return T3_DENSE_CHAIN;
     return per % 8u == 0u && per <= 16u ? T3_DENSE_ONE_LAUNCH : T3_DENSE_ARRIVE;
 }
 
