@@ -11,9 +11,12 @@
 // (M = column c = l % 16, K slots 8g..8g+7), so decoded registers feed the matrix core with no shuffle.
 //
 // A quad's four windows span at most 3n/16 + 17 bits. Up to n = 84 they fit one 32-bit register R (the 32 stream bits
-// ending at the last window's end): two word loads, one v_alignbit, one v_bfe a weight. Wider rates read the first two
-// windows from a second register ending at window 1's end.
+// ending at the last window's end): two word loads, one v_alignbit, one v_bfe a weight (kNarrow). Wider rates read the
+// first two windows from a second register ending at window 1's end: cut from the same two words where every quad's
+// span lies inside them (kWidePair: n = 86..90, 96, 128), from two more words otherwise (kWide).
 #pragma once
+
+#include <type_traits>
 
 #include "t3_common.hpp"
 
@@ -84,6 +87,9 @@ __device__ __forceinline__ uint32_t quad_first_position(uint32_t lane) {
     return 8u * (4u * (c & 7u) + g) + 4u * (c >> 3);
 }
 
+// How a lane reads its quad at rate n.
+enum Reader : int { kNarrow = 0, kWide = 1, kWidePair = 2 };
+
 // Whether some quad's four windows overflow one 32-bit register at rate n (host and device agree on this rule).
 __host__ __device__ inline bool quad_needs_wide(uint32_t n) {
     for (uint32_t q = 0; q < 64u; ++q) {
@@ -92,15 +98,38 @@ __host__ __device__ inline bool quad_needs_wide(uint32_t n) {
     }
     return false;
 }
+// Whether every quad's four windows lie inside the two words that hold the 32 stream bits ending at window 3's end.
+__host__ __device__ inline bool quad_in_two_words(uint32_t n) {
+    for (uint32_t q = 0; q < 64u; ++q) {
+        const uint32_t e0 = ((4u * q + 1u) * n) >> 4, e3 = ((4u * q + 4u) * n) >> 4;
+        const uint32_t w = (e3 + 16u * n - 1u) >> 5;  // one period added, as the plan does
+        if (e0 + 16u * n - 16u < 32u * (w - 1u)) return false;
+    }
+    return true;
+}
+__host__ __device__ inline int quad_reader(uint32_t n) {
+    return !quad_needs_wide(n) ? kNarrow : quad_in_two_words(n) ? kWidePair : kWide;
+}
 
-template <bool WIDE>
+// Host side: call f with the rate's reader as a compile-time constant.
+template <typename F>
+inline auto with_reader(uint32_t n, F&& f) {
+    switch (quad_reader(n)) {
+        case kWide: return f(std::integral_constant<int, kWide>{});
+        case kWidePair: return f(std::integral_constant<int, kWidePair>{});
+        default: return f(std::integral_constant<int, kNarrow>{});
+    }
+}
+
+template <int WIDE>
 struct QuadPlan {
     uint32_t ib_prev, ib_last, shb;  // register B: the 32 stream bits ending at window 3's end
-    uint32_t ia_prev, ia_last, sha;  // register A (WIDE only): ... ending at window 1's end
+    uint32_t ia_prev, ia_last, sha;  // register A (wide readers): ... ending at window 1's end
+    uint32_t a_low;                  // kWidePair: register A's low word is B's previous word (else B's last)
     uint32_t o[4];                   // window m's right shift inside its register
 };
 
-template <bool WIDE>
+template <int WIDE>
 __device__ __forceinline__ QuadPlan<WIDE> quad_plan(uint32_t n, uint32_t lane) {
     const uint32_t p = quad_first_position(lane);
     const uint32_t nw = n >> 1, total = 16u * n;
@@ -116,7 +145,19 @@ __device__ __forceinline__ QuadPlan<WIDE> quad_plan(uint32_t n, uint32_t lane) {
         q.ib_last = w - nw;
         q.ib_prev = w - 1u >= nw ? w - 1u - nw : w - 1u;
     }
-    if constexpr (WIDE) {
+    q.a_low = 0u;
+    if constexpr (WIDE == kWidePair) {
+        // the 64 bits {previous, last} shifted right until window 1's end is bit 0: by less than 32, one v_alignbit of
+        // the pair; by 32 or more, the previous word alone (its own bits fill the top, above the two windows)
+        const uint32_t sa = q.shb + (e[3] - e[1]);
+        q.a_low = sa >= 32u ? 1u : 0u;
+        q.sha = sa & 31u;
+        q.ia_last = q.ia_prev = 0u;
+        q.o[0] = e[1] - e[0];
+        q.o[1] = 0u;
+        q.o[2] = e[3] - e[2];
+        q.o[3] = 0u;
+    } else if constexpr (WIDE == kWide) {
         const uint32_t end = e[1] + total;
         const uint32_t w = (end - 1u) >> 5;
         q.sha = 32u * (w + 1u) - end;
@@ -135,17 +176,17 @@ __device__ __forceinline__ QuadPlan<WIDE> quad_plan(uint32_t n, uint32_t lane) {
 }
 
 // The words a lane holds of one tile, loaded ahead of their use.
-template <bool WIDE>
+template <int WIDE>
 struct QuadWords {
-    uint32_t b_prev, b_last, a_prev, a_last;
+    uint32_t b_prev, b_last, a_prev, a_last;  // the a words: kWide only
 };
 
-template <bool WIDE>
+template <int WIDE>
 __device__ __forceinline__ QuadWords<WIDE> quad_load(const uint32_t* tile, const QuadPlan<WIDE>& q) {
     QuadWords<WIDE> w;
     w.b_prev = tile[q.ib_prev];
     w.b_last = tile[q.ib_last];
-    if constexpr (WIDE) {
+    if constexpr (WIDE == kWide) {
         w.a_prev = tile[q.ia_prev];
         w.a_last = tile[q.ia_last];
     } else {
@@ -155,12 +196,13 @@ __device__ __forceinline__ QuadWords<WIDE> quad_load(const uint32_t* tile, const
 }
 
 // The quad's four codewords, masked to the pack's window width `wbits` (8..16).
-template <bool WIDE>
+template <int WIDE>
 __device__ __forceinline__ void quad_codewords(const QuadWords<WIDE>& w, const QuadPlan<WIDE>& q, uint32_t wbits,
                                                uint32_t (&cw)[4]) {
     const uint32_t rb = __builtin_amdgcn_alignbit(w.b_prev, w.b_last, q.shb);
     uint32_t ra = rb;
-    if constexpr (WIDE) ra = __builtin_amdgcn_alignbit(w.a_prev, w.a_last, q.sha);
+    if constexpr (WIDE == kWide) ra = __builtin_amdgcn_alignbit(w.a_prev, w.a_last, q.sha);
+    if constexpr (WIDE == kWidePair) ra = __builtin_amdgcn_alignbit(w.b_prev, q.a_low ? w.b_prev : w.b_last, q.sha);
     cw[0] = __builtin_amdgcn_ubfe(ra, q.o[0], wbits);
     cw[1] = __builtin_amdgcn_ubfe(ra, q.o[1], wbits);
     cw[2] = __builtin_amdgcn_ubfe(rb, q.o[2], wbits);

@@ -125,7 +125,7 @@ struct GemvArgs {
 // Grid (out / 16 / BT, KS), 256 threads (4 waves). A workgroup owns BT adjacent output tiles and K slice blockIdx.y;
 // wave sg takes part sg of the slice, `per` = in_tiles / (4 KS) input tiles (the host divides: the GPU has no scalar
 // divide). RB = 16-row blocks of x (1 or 2). z f32 [KS][rows][out]: the four waves' sums, wave 0 first.
-template <int CB, bool WIDE, int RB, int BT, int FUSE>
+template <int CB, int WIDE, int RB, int BT, int FUSE>
 __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
     constexpr int ST = 2;  // tile rows in flight a wave: occupancy hides more latency here than a deeper ring does
     constexpr uint32_t kStage = gemv_stage_bytes<BT>();
@@ -273,7 +273,7 @@ __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
     }
 }
 
-template <int CB, bool WIDE, int RB, int BT>
+template <int CB, int WIDE, int RB, int BT>
 hipError_t launch_gemv_fuse(const DenseLaunch& d, int fuse, hipStream_t s) {
     GemvArgs a;
     a.w = d.trellis;
@@ -312,15 +312,16 @@ hipError_t launch_gemv_fuse(const DenseLaunch& d, int fuse, hipStream_t s) {
 
 template <int CB>
 hipError_t launch_gemv_cb(const DenseLaunch& d, int fuse, hipStream_t s) {
-    const bool wide = quad_needs_wide(d.n);
     const bool two = d.rows > 16u;
-    const bool bt8 = d.bt == 8u;
-    if (wide) {
-        if (two) return bt8 ? launch_gemv_fuse<CB, true, 2, 8>(d, fuse, s) : launch_gemv_fuse<CB, true, 2, 4>(d, fuse, s);
-        return bt8 ? launch_gemv_fuse<CB, true, 1, 8>(d, fuse, s) : launch_gemv_fuse<CB, true, 1, 4>(d, fuse, s);
-    }
-    if (two) return bt8 ? launch_gemv_fuse<CB, false, 2, 8>(d, fuse, s) : launch_gemv_fuse<CB, false, 2, 4>(d, fuse, s);
-    return bt8 ? launch_gemv_fuse<CB, false, 1, 8>(d, fuse, s) : launch_gemv_fuse<CB, false, 1, 4>(d, fuse, s);
+    return with_reader(d.n, [&](auto reader) {
+        constexpr int R = decltype(reader)::value;
+        if constexpr (R == kNarrow) {
+            if (d.bt == 8u) return two ? launch_gemv_fuse<CB, R, 2, 8>(d, fuse, s) : launch_gemv_fuse<CB, R, 1, 8>(d, fuse, s);
+        }
+        // a wide rate's tile is over 128 bytes: eight of them never fit a load, the host gives them four
+        if (d.bt != 4u && R != kNarrow) return hipErrorInvalidValue;
+        return two ? launch_gemv_fuse<CB, R, 2, 4>(d, fuse, s) : launch_gemv_fuse<CB, R, 1, 4>(d, fuse, s);
+    });
 }
 
 }  // namespace

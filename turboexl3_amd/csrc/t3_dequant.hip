@@ -10,7 +10,7 @@ namespace {
 
 // Grid (out / 64, in / 16), 256 threads: wave sg decodes tile (tk, 4 blockIdx.x + sg); the four tiles' rows leave
 // through LDS as 128-byte row segments.
-template <int CB, bool WIDE>
+template <int CB, int WIDE>
 __global__ void __launch_bounds__(256) dequant_kernel(const uint32_t* __restrict__ w, uint16_t* __restrict__ w_hat,
                                                       uint32_t out, uint32_t n, uint32_t wbits) {
     __shared__ __attribute__((aligned(16))) uint16_t stage[16][64 + 8];
@@ -37,7 +37,7 @@ __global__ void __launch_bounds__(256) test_codebooks_kernel(uint16_t* mcg, uint
 }
 
 // Grid (tiles), 64 threads: the quad reader's codewords by code position and both codebooks' values of them.
-template <bool WIDE>
+template <int WIDE>
 __global__ void __launch_bounds__(64) test_lane_kernel(const uint32_t* trellis, uint32_t n, uint32_t wbits,
                                                        uint16_t* cw_out, uint16_t* mcg, uint16_t* mul1) {
     const uint32_t lane = threadIdx.x, tile = blockIdx.x;
@@ -76,12 +76,12 @@ __global__ void __launch_bounds__(64) test_mfma_kernel(const uint16_t* a, const 
 hipError_t launch_dequant(const uint32_t* trellis, uint16_t* w_hat, uint32_t in, uint32_t out, uint32_t n,
                           uint32_t wbits, int codebook, hipStream_t s) {
     const dim3 grid(out / 64u, in / 16u), block(256);
-    const bool wide = quad_needs_wide(n);
     const bool mcg = codebook == kMcg || codebook == kMcgPair;
-    if (mcg && wide) hipLaunchKernelGGL((dequant_kernel<kMcg, true>), grid, block, 0, s, trellis, w_hat, out, n, wbits);
-    else if (mcg) hipLaunchKernelGGL((dequant_kernel<kMcg, false>), grid, block, 0, s, trellis, w_hat, out, n, wbits);
-    else if (wide) hipLaunchKernelGGL((dequant_kernel<kMul1, true>), grid, block, 0, s, trellis, w_hat, out, n, wbits);
-    else hipLaunchKernelGGL((dequant_kernel<kMul1, false>), grid, block, 0, s, trellis, w_hat, out, n, wbits);
+    with_reader(n, [&](auto reader) {
+        constexpr int R = decltype(reader)::value;
+        if (mcg) hipLaunchKernelGGL((dequant_kernel<kMcg, R>), grid, block, 0, s, trellis, w_hat, out, n, wbits);
+        else hipLaunchKernelGGL((dequant_kernel<kMul1, R>), grid, block, 0, s, trellis, w_hat, out, n, wbits);
+    });
     return hipGetLastError();
 }
 
@@ -92,9 +92,10 @@ hipError_t launch_test_codebooks(uint16_t* mcg, uint16_t* mul1, uint16_t* t, hip
 
 hipError_t launch_test_lane(const uint32_t* trellis, uint32_t n, uint32_t wbits, uint32_t tiles, uint16_t* cw,
                             uint16_t* mcg, uint16_t* mul1, hipStream_t s) {
-    if (quad_needs_wide(n))
-        hipLaunchKernelGGL(test_lane_kernel<true>, dim3(tiles), dim3(64), 0, s, trellis, n, wbits, cw, mcg, mul1);
-    else hipLaunchKernelGGL(test_lane_kernel<false>, dim3(tiles), dim3(64), 0, s, trellis, n, wbits, cw, mcg, mul1);
+    with_reader(n, [&](auto reader) {
+        hipLaunchKernelGGL(test_lane_kernel<decltype(reader)::value>, dim3(tiles), dim3(64), 0, s, trellis, n, wbits, cw,
+                           mcg, mul1);
+    });
     return hipGetLastError();
 }
 

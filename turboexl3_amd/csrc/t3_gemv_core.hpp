@@ -50,7 +50,7 @@ struct XLds {               // the wave's own [per + 1][kXldsRows][64 bytes], wr
 // xoff[r]: the lane's byte offset of block r's activation row plus its quad, inside a row (XGlobal) or inside a tile
 // row's kXldsRows x 64 bytes (XLds). stage: the wave's own LDS bytes (gemv_stage_bytes<BT>()), 16-byte aligned.
 // run(): acc[r][t] += the 16 x 16 product of activation block r and tile t, summed over the wave's tile rows in order.
-template <int CB, bool WIDE, int RB, int BT, int ST, typename XSrc>
+template <int CB, int WIDE, int RB, int BT, int ST, typename XSrc>
 struct GemvStream {
     static constexpr bool kXLds = __is_same(XSrc, XLds);
     static_assert(ST % 2 == 0, "stage buffers and word sets alternate by ring slot parity");
@@ -104,7 +104,17 @@ struct GemvStream {
         }
     }
 
+    // A tile of whole 16-byte pieces (n a multiple of 8: every standard rate) takes a lane's load into the stage with one
+    // 128-bit store; otherwise a lane's four dwords may lie in two tiles and go one by one (four stores at a stride of
+    // four banks: each a four-way bank conflict, which the wide rates' LDS traffic has no room for). Two copies of the
+    // loop rather than a branch inside it.
     __device__ __forceinline__ void run(float4v (&acc)[RB][BT]) {
+        if ((n & 7u) == 0u) run_as<true>(acc);
+        else run_as<false>(acc);
+    }
+
+    template <bool W16>
+    __device__ __forceinline__ void run_as(float4v (&acc)[RB][BT]) {
         const uint32_t tile_bytes = 2u * n;
         const uint32_t chunk_bytes = static_cast<uint32_t>(BT) * tile_bytes;
         // The loads are in flight; everything a lane needs to decode is worked out under their latency.
@@ -126,9 +136,13 @@ struct GemvStream {
         const uint32_t get_ap = plan.ia_prev * 4u, get_al = plan.ia_last * 4u;
 
         auto stage_chunk = [&](const uint4v& v, uint32_t parity) {
+            if constexpr (W16) {
+                *reinterpret_cast<uint4v*>(stage + parity * (BT * kTileSlot) + put[0]) = v;
+            } else {
 #pragma unroll
-            for (uint32_t j = 0; j < 4u; ++j)
-                *reinterpret_cast<uint32_t*>(stage + parity * (BT * kTileSlot) + put[j]) = v[j];
+                for (uint32_t j = 0; j < 4u; ++j)
+                    *reinterpret_cast<uint32_t*>(stage + parity * (BT * kTileSlot) + put[j]) = v[j];
+            }
         };
         // a tile row's words, read back from the stage into registers one row ahead of their decode
         auto fetch = [&](uint32_t parity, uint32_t row, QuadWords<WIDE>(&wd)[BT], uint4v(&xv)[RB]) {
@@ -138,7 +152,7 @@ struct GemvStream {
                 const unsigned char* slot = buf + static_cast<uint32_t>(t) * kTileSlot;
                 wd[t].b_prev = *reinterpret_cast<const uint32_t*>(slot + get_bp);
                 wd[t].b_last = *reinterpret_cast<const uint32_t*>(slot + get_bl);
-                if constexpr (WIDE) {
+                if constexpr (WIDE == kWide) {
                     wd[t].a_prev = *reinterpret_cast<const uint32_t*>(slot + get_ap);
                     wd[t].a_last = *reinterpret_cast<const uint32_t*>(slot + get_al);
                 }

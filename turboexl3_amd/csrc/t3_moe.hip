@@ -51,7 +51,7 @@ constexpr uint32_t role_lds_bytes() {
     return stage > red ? stage : red;
 }
 
-template <int CB, bool WIDE, int BT, int NPROJ, bool XLDS, bool ARRIVE>
+template <int CB, int WIDE, int BT, int NPROJ, bool XLDS, bool ARRIVE>
 __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint32_t yidx, uint32_t ksl,
                                           unsigned char* smem, uint32_t& last_flag, uint32_t* cinfo, float* cscore) {
     // Two tile rows in flight a wave (measured: all 8 in flight is no faster; a call's time is its chain of dependent
@@ -241,7 +241,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
     }
 }
 
-template <int CB, bool WIDE, int BT, int NPROJ, bool XLDS, bool ARRIVE>
+template <int CB, int WIDE, int BT, int NPROJ, bool XLDS, bool ARRIVE>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ? 2 : 4))) moe_gemv(const MoeLaunch a) {
     __shared__ __attribute__((aligned(16))) unsigned char smem[role_lds_bytes<BT>()];
     __shared__ uint32_t last_flag, cinfo[64];
@@ -263,35 +263,35 @@ __global__ void __launch_bounds__(64) moe_combine(const MoeLaunch a) {
     else routed_slots_block<false>(a, blockIdx.y, blockIdx.x, threadIdx.x);
 }
 
-template <int CB, bool WIDE, int NPROJ, bool XLDS, bool ARRIVE>
+template <int CB, int WIDE, int NPROJ, bool XLDS, bool ARRIVE>
 hipError_t launch_gemv_bt(const MoeLaunch& a, hipStream_t s) {
     const uint32_t out = NPROJ == 2 ? a.inter : a.hidden;
     const uint32_t bt = NPROJ == 2 ? a.bt_gu : a.bt_dn, ks = NPROJ == 2 ? a.ks_gu : a.ks_dn;
     const uint32_t rkt = a.rows * (a.topk + a.shared_slots);
     const dim3 grid((out / 16u) / bt, rkt * NPROJ, ks), block(256);
     const size_t dyn = XLDS ? 4u * ((NPROJ == 2 ? a.per_gu : a.per_dn) + 1u) * (kXldsRows * 64u) : 0u;
-    if (bt == 8u) hipLaunchKernelGGL((moe_gemv<CB, WIDE, 8, NPROJ, XLDS, ARRIVE>), grid, block, dyn, s, a);
-    else hipLaunchKernelGGL((moe_gemv<CB, WIDE, 4, NPROJ, XLDS, ARRIVE>), grid, block, dyn, s, a);
+    if constexpr (WIDE == kNarrow) {
+        if (bt == 8u) {
+            hipLaunchKernelGGL((moe_gemv<CB, WIDE, 8, NPROJ, XLDS, ARRIVE>), grid, block, dyn, s, a);
+            return hipGetLastError();
+        }
+    }
+    if (bt != 4u) return hipErrorInvalidValue;  // a wide rate's eight tiles never fit a load
+    hipLaunchKernelGGL((moe_gemv<CB, WIDE, 4, NPROJ, XLDS, ARRIVE>), grid, block, dyn, s, a);
     return hipGetLastError();
 }
 
 template <int NPROJ, bool XLDS, bool ARRIVE>
 hipError_t launch_gemv_cb(const MoeLaunch& a, hipStream_t s) {
-    const bool wide = quad_needs_wide(NPROJ == 2 ? a.n_gu : a.n_dn);
-    switch (a.codebook) {
-        case kMul1:
-            return wide ? launch_gemv_bt<kMul1, true, NPROJ, XLDS, ARRIVE>(a, s)
-                        : launch_gemv_bt<kMul1, false, NPROJ, XLDS, ARRIVE>(a, s);
-        case kMcg:
-            return wide ? launch_gemv_bt<kMcg, true, NPROJ, XLDS, ARRIVE>(a, s)
-                        : launch_gemv_bt<kMcg, false, NPROJ, XLDS, ARRIVE>(a, s);
-        case kMul1Defer:
-            return wide ? launch_gemv_bt<kMul1Defer, true, NPROJ, XLDS, ARRIVE>(a, s)
-                        : launch_gemv_bt<kMul1Defer, false, NPROJ, XLDS, ARRIVE>(a, s);
-        default:
-            return wide ? launch_gemv_bt<kMcgPair, true, NPROJ, XLDS, ARRIVE>(a, s)
-                        : launch_gemv_bt<kMcgPair, false, NPROJ, XLDS, ARRIVE>(a, s);
-    }
+    return with_reader(NPROJ == 2 ? a.n_gu : a.n_dn, [&](auto reader) {
+        constexpr int R = decltype(reader)::value;
+        switch (a.codebook) {
+            case kMul1: return launch_gemv_bt<kMul1, R, NPROJ, XLDS, ARRIVE>(a, s);
+            case kMcg: return launch_gemv_bt<kMcg, R, NPROJ, XLDS, ARRIVE>(a, s);
+            case kMul1Defer: return launch_gemv_bt<kMul1Defer, R, NPROJ, XLDS, ARRIVE>(a, s);
+            default: return launch_gemv_bt<kMcgPair, R, NPROJ, XLDS, ARRIVE>(a, s);
+        }
+    });
 }
 
 }  // namespace

@@ -111,7 +111,7 @@ __device__ __forceinline__ void wait_loads() {
 // LBMAX < RB (the 128-row shape only): the same kernel with accumulators for LBMAX live row blocks (16 LBMAX registers
 // a lane instead of 128) and rings three steps deep, which fits three waves a SIMD where the full shape fits two. It
 // serves routings whose items the route cuts at 16 LBMAX = 96 rows (src: `moe_item_rows`).
-template <int CB, bool WIDE, int RB, int LBMAX = RB>
+template <int CB, int WIDE, int RB, int LBMAX = RB>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(LBMAX < RB ? 3 : 1, 8))) pf_gemm(const PfGemm a) {
     constexpr bool kShort = LBMAX < RB;
     constexpr uint32_t D = (RB == 2 || kShort) ? 3u : 4u;    // steps in flight + 1
@@ -191,7 +191,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(LBMAX 
                 const unsigned char* tile = st + (r * kPfTiles + t) * kPfSlot;
                 wd[r][t].b_prev = *reinterpret_cast<const uint32_t*>(tile + get_bp);
                 wd[r][t].b_last = *reinterpret_cast<const uint32_t*>(tile + get_bl);
-                if constexpr (WIDE) {
+                if constexpr (WIDE == kWide) {
                     wd[r][t].a_prev = *reinterpret_cast<const uint32_t*>(tile + get_ap);
                     wd[r][t].a_last = *reinterpret_cast<const uint32_t*>(tile + get_al);
                 }
@@ -656,7 +656,7 @@ inline uint32_t gemm_nblk(uint32_t out, uint32_t item_rows) {
     return (out + 255u) / 256u;
 }
 
-template <int CB, bool WIDE>
+template <int CB, int WIDE>
 hipError_t launch_gemm_rb(PfGemm g, uint32_t max_items, uint32_t nproj, uint32_t item_rows, hipStream_t s) {
     g.nblk = gemm_nblk(g.out, item_rows);
     g.spread = gemm_spread(max_items);  // 8 / spread items share the dies
@@ -672,18 +672,14 @@ hipError_t launch_gemm_rb(PfGemm g, uint32_t max_items, uint32_t nproj, uint32_t
 // The GEMM decodes exactly whatever form the GEMV runs: MCG's pair form has no use here (it would double K).
 hipError_t launch_gemm(const PfGemm& g, int codebook, uint32_t max_items, uint32_t nproj, uint32_t item_rows,
                        hipStream_t s) {
-    const bool wide = quad_needs_wide(g.n);
-    switch (codebook) {
-        case kMul1:
-            return wide ? launch_gemm_rb<kMul1, true>(g, max_items, nproj, item_rows, s)
-                        : launch_gemm_rb<kMul1, false>(g, max_items, nproj, item_rows, s);
-        case kMul1Defer:
-            return wide ? launch_gemm_rb<kMul1Defer, true>(g, max_items, nproj, item_rows, s)
-                        : launch_gemm_rb<kMul1Defer, false>(g, max_items, nproj, item_rows, s);
-        default:
-            return wide ? launch_gemm_rb<kMcg, true>(g, max_items, nproj, item_rows, s)
-                        : launch_gemm_rb<kMcg, false>(g, max_items, nproj, item_rows, s);
-    }
+    return with_reader(g.n, [&](auto reader) {
+        constexpr int R = decltype(reader)::value;
+        switch (codebook) {
+            case kMul1: return launch_gemm_rb<kMul1, R>(g, max_items, nproj, item_rows, s);
+            case kMul1Defer: return launch_gemm_rb<kMul1Defer, R>(g, max_items, nproj, item_rows, s);
+            default: return launch_gemm_rb<kMcg, R>(g, max_items, nproj, item_rows, s);
+        }
+    });
 }
 
 }  // namespace
