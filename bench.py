@@ -11,7 +11,8 @@ captures its calls once into a HIP graph and brackets a replay with events on th
 
 Prints ONE JSON line. `value`: the whole call's rate as GB/s of trellis code bytes. `roofline`: the kernel that call
 launches (one launch at one row: the call's time is that kernel's), its algorithmic code bytes over its duration
-against 8 TB/s; `gemv_launch_alone` is the chain's GEMV launch without prepare and finish, for comparison. Beside
+against 8 TB/s; `gemv_launch_alone` is the chain's GEMV launch without prepare and finish, for comparison, and
+`launch_floor` what the chain's two small launches cost alone (what any launch costs in a replayed graph). Beside
 them, unless --quick: `sweep` (the metric's K = 3, 4, 5 x rows = 1, 4, 16, 32), `lm_head` (4096 -> 151936 at K6, 1 and
 256 rows), `moe_decode` (config 3 at 1 and 8 tokens, each launch timed alone as well), `moe_prefill` (config 4, each
 stage timed alone; TFLOP/s against the 2.5 PFLOP/s f16 MFMA figure and against a dense f16 GEMM measured in this
@@ -42,7 +43,7 @@ MIN_ROTATION_BYTES = 512 << 20
 # HBM bytes one launch of the served one-row kernel (the one-launch form) moves, from the profiler's FETCH_SIZE and
 # WRITE_SIZE counters scaled by a 256 MiB copy (profiles/dense_gemv_in4096_out12288_k4_rows1.txt): keyed by
 # (in, out, n, rows); others report null
-MEASURED_TRAFFIC = {(4096, 12288, 64, 1): 27_476_518}
+MEASURED_TRAFFIC = {(4096, 12288, 64, 1): 27_503_399}
 F32_BAR, BF16_DENSE_BAR, BF16_MOE_BAR = 5e-3, 2.5e-2, 1.5e-2
 
 MCG_CB, MUL1_CB = 1, 0
@@ -399,6 +400,13 @@ def main() -> int:
                               "achieved": head.get("gemv_gbps"), "unit": "GB/s", "frac": head.get("gemv_frac_of_hbm")},
     }
 
+    # what a launch costs here whatever it computes: the chain's prepare and finish launches alone (32 and 96 one-wave
+    # workgroups), each replayed back to back in a graph like every other cell
+    d.bind(args.rows)
+    out["launch_floor"] = {"prepare_launch_alone_us": d.time(sub_steps, 10, stages=1) * 1e6,
+                           "finish_launch_alone_us": d.time(sub_steps, 10, stages=4) * 1e6,
+                           "chain_three_launches_us": d.time(sub_steps, 10, stages=7) * 1e6}
+
     if "sweep" in sections:
         out["sweep"] = []
         for k in (3, 4, 5):
@@ -449,7 +457,7 @@ def main() -> int:
         in_f, out_f, n = 4096, 151936, 96
         dl = Dense(torch, api, in_f, out_f, n, MCG_CB, 256, torch.bfloat16, seed=6, copies=2, outliers=False)
         one = dense_cell(dl, 1, 40, 4, todo, "lm_head K6 rows 1", gemv_alone=True)
-        one["roofline"] = {"bound": "hbm", "kernel": "t3::dense_gemv<kMcgPair, wide, 1, 4 tiles>", "us_per_launch": one.get("gemv_us"),
+        one["roofline"] = {"bound": "hbm", "kernel": "t3::dense_gemv<kMcgPair, two-word wide reader, 1 row block, 4 tiles>", "us_per_launch": one.get("gemv_us"),
                            "algorithmic_bytes_per_launch": dl.cb, "achieved": one.get("gemv_gbps"), "peak": HBM_PEAK / 1e9,
                            "unit": "GB/s", "frac": one.get("gemv_frac_of_hbm")}
         many = dense_cell(dl, 256, 10, 2, todo, "lm_head K6 rows 256")

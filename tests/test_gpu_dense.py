@@ -51,6 +51,8 @@ CASES = [
     (2560, 640, 80, MUL1, 16, torch.bfloat16),
     (4096, 2048, 64, MCG, 16, torch.bfloat16),
     (1024, 512, 96, MUL1, 16, torch.float16),
+    (512, 256, 112, MCG, 16, torch.float32),     # K7: the four-word wide reader (K6 and K8 read two words)
+    (512, 256, 88, MUL1, 16, torch.float32),     # a fractional wide rate on the two-word reader
 ]
 
 

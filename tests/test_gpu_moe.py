@@ -153,7 +153,7 @@ def test_launch_forms_give_the_same_bytes(oracle, t3):
 
 
 @pytest.mark.parametrize("hidden,inter,experts,topk,n", [(128, 128, 1, 1, 64), (128, 256, 3, 2, 16), (384, 128, 5, 3, 128),
-                                                         (256, 384, 4, 4, 34)])
+                                                         (256, 384, 4, 4, 34), (256, 256, 3, 2, 112), (256, 128, 3, 2, 96)])
 def test_smallest_and_odd_banks(oracle, t3, hidden, inter, experts, topk, n):
     # one 128-block either side, a single expert, the extreme rates, a fractional one, three-block widths: decode rows
     # (waves past the last K part idle), the row boundary of the chains, and the prefill chain

@@ -30,6 +30,7 @@ DENSE = [
     (512, 256, 128, MCG, 12, torch.float32),
     (1024, 512, 96, MUL1, 16, torch.float16),
     (2560, 640, 80, MUL1, 16, torch.bfloat16),
+    (512, 256, 112, MCG, 16, torch.float32),     # K7: the four-word wide reader
 ]
 
 
