@@ -31,8 +31,10 @@ namespace {
 
 enum Fuse : int { kChain = 0, kArrive = 1, kOne = 2 };
 
-// Grid (in / 128, rows), 64 threads. xq: uint32 [rows][in], word (tk 16 + quad_slot(r)) = the f16 value of input
-// tk 16 + r in both halves. xs: f32 [rows][in / 128].
+// Grid (in / 128, rows), 64 threads. xq: uint32 [in / 16][rows][16], word quad_slot(r) of (tile tk, row) = the f16 value of
+// input tk 16 + r in both halves: the rows of one input tile lie side by side, so the GEMV's fragment of a tile row (64 bytes
+// a row) is one contiguous piece of whole cache lines (with a row's tiles adjacent instead, a 16-row fragment touched 16
+// lines for half of each, and 32 rows cost the K5 GEMV a third of its time). xs: f32 [rows][in / 128].
 __global__ void __launch_bounds__(64) dense_prep(const void* x, const uint16_t* suh, uint32_t* xq, float* xs,
                                                  uint32_t in, int dt) {
     const uint32_t b = blockIdx.x, row = blockIdx.y, lane = threadIdx.x;
@@ -42,7 +44,7 @@ __global__ void __launch_bounds__(64) dense_prep(const void* x, const uint16_t* 
 #pragma unroll
     for (uint32_t j = 0; j < 2u; ++j) {
         const uint32_t i = b * 128u + lane + 64u * j;
-        xq[static_cast<size_t>(row) * in + (i & ~15u) + quad_slot(i & 15u)] = hv[j] | (hv[j] << 16);
+        xq[(static_cast<size_t>(i >> 4) * gridDim.y + row) * 16u + quad_slot(i & 15u)] = hv[j] | (hv[j] << 16);
     }
     if (lane == 0u) xs[static_cast<size_t>(row) * (in / 128u) + b] = sum;
 }
@@ -216,10 +218,10 @@ __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
 #pragma unroll
         for (int r = 0; r < RB; ++r) {
             const uint32_t row = static_cast<uint32_t>(r) * 16u + (lane & 15u);
-            xoff[r] = ((row < rows ? row : 0u) * a.in + 4u * (lane >> 4)) * 4u;
+            xoff[r] = ((row < rows ? row : 0u) * 16u + 4u * (lane >> 4)) * 4u;
         }
         GemvStream<CB, WIDE, RB, BT, ST, XGlobal> stream(
-            wbase, wstep, per, a.n, a.wbits, XGlobal{a.xq, static_cast<uint64_t>(rows) * a.in * 4u, tk0 * 64u}, xoff,
+            wbase, wstep, per, a.n, a.wbits, XGlobal{a.xq, static_cast<uint64_t>(rows) * a.in * 4u, tk0 * rows * 64u, rows * 64u}, xoff,
             smem + sg * kStage, lane);
         stream.issue();
         stream.run(acc);

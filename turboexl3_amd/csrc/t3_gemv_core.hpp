@@ -34,10 +34,13 @@ constexpr uint32_t gemv_stage_bytes() {
 }
 
 // Where a wave's prepared activations come from.
-struct XGlobal {            // u32 [rows][in], doubled f16 in quad order
+struct XGlobal {            // doubled f16 in quad order, 64 bytes a (row, input tile)
     const uint32_t* base;
     uint64_t bytes;
-    uint32_t first;         // byte offset of the wave's first input tile inside a row (a tile: 64 bytes)
+    uint32_t first;         // byte offset of the wave's first input tile
+    uint32_t step;          // bytes from one input tile to the next: 64 where a row's tiles are adjacent ([rows][in]),
+                            // rows x 64 where a tile's rows are ([in / 16][rows][16]: the fragment of one tile row is one
+                            // contiguous piece, whole cache lines whatever the rows)
 };
 struct XLds {               // the wave's own [per + 1][kXldsRows][64 bytes], written by the in-kernel prepare;
     const unsigned char* base;  // the last tile row all zeros: what a row past the wave's last multiplies by
@@ -89,7 +92,7 @@ struct GemvStream {
     __device__ __forceinline__ void load_x(uint32_t row, uint4v (&dst)[RB]) const {
         if constexpr (!kXLds) {
             const __amdgpu_buffer_rsrc_t res = make_rsrc(xs.base, row < per ? xs.bytes : 0u);
-            const uint32_t soff = xs.first + row * 64u;
+            const uint32_t soff = xs.first + row * xs.step;
 #pragma unroll
             for (int r = 0; r < RB; ++r) dst[r] = buf_load_u128(res, xoff[r], soff);
         }

@@ -69,7 +69,7 @@ int32_t check_dense(const t3_array* x, const t3_array* trellis, const t3_array* 
     return T3_OK;
 }
 
-// arrival counters u32 [out / 128] (fixed place), xq u32 [rows][in], xs f32 [rows][in / 128], z f32 [ks][rows][out]
+// arrival counters u32 [out / 128] (fixed place), xq u32 [in / 16][rows][16], xs f32 [rows][in / 128], z f32 [ks][rows][out]
 void carve_dense(DenseCall* call, void* workspace) {
     DenseLaunch& l = call->launch;
     Carver c(workspace);

@@ -150,7 +150,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
             const uint32_t* xq = NPROJ == 1 ? a.hd : (proj ? a.xu : a.xg);
             xoff[0] = (rk * in + 4u * (lane >> 4)) * 4u;
             GemvStream<CB, WIDE, 1, BT, ST, XGlobal> stream(
-                wbase, wstep, per, n, a.wbits, XGlobal{xq, static_cast<uint64_t>(rkt) * in * 4u, tk0 * 64u}, xoff,
+                wbase, wstep, per, n, a.wbits, XGlobal{xq, static_cast<uint64_t>(rkt) * in * 4u, tk0 * 64u, 64u}, xoff,
                 smem + sg * kStage, lane);
             stream.issue();
             stream.run(acc);
