@@ -45,6 +45,10 @@ __device__ __forceinline__ void store_coherent(float* p, float v) {
 __device__ __forceinline__ float load_coherent(const float* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// four adjacent floats (16-byte aligned) in one device-coherent store
+__device__ __forceinline__ void store_coherent4(float* p, float4v v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+}
 // every store this lane has issued is acknowledged at its coherence level (with store_coherent: device-wide)
 __device__ __forceinline__ void wait_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 

@@ -243,8 +243,7 @@ __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
         if constexpr (FUSE == kChain) {
             *reinterpret_cast<float4v*>(dst) = s;
         } else {
-#pragma unroll
-            for (int c = 0; c < 4; ++c) store_coherent(dst + c, s[c]);
+            store_coherent4(dst, s);
         }
     }
 

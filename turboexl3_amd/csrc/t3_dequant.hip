@@ -8,25 +8,53 @@
 namespace t3 {
 namespace {
 
-// Grid (out / 64, in / 16), 256 threads: wave sg decodes tile (tk, 4 blockIdx.x + sg); the four tiles' rows leave
-// through LDS as 128-byte row segments.
+// Grid (ceil(out / 128 / kDqSteps), in / 16), 256 threads: a workgroup walks kDqSteps 128-column pieces of tile row tk; at
+// every piece wave sg decodes tiles 8 piece + 2 sg and + 1, and the eight tiles' rows leave through LDS as 256-byte row
+// segments, 16 bytes a thread. The lane plan is made once a workgroup, the next piece's words are fetched before the
+// current piece is staged, and the stage alternates between two buffers: one barrier a piece.
+constexpr uint32_t kDqSteps = 4u;
 template <int CB, int WIDE>
 __global__ void __launch_bounds__(256) dequant_kernel(const uint32_t* __restrict__ w, uint16_t* __restrict__ w_hat,
                                                       uint32_t out, uint32_t n, uint32_t wbits) {
-    __shared__ __attribute__((aligned(16))) uint16_t stage[16][64 + 8];
+    __shared__ __attribute__((aligned(16))) uint16_t stage[2][16][128 + 8];
     const uint32_t sg = threadIdx.x >> 6, lane = threadIdx.x & 63u;
-    const uint32_t tk = blockIdx.y, tn = blockIdx.x * 4u + sg;
+    const uint32_t tk = blockIdx.y;
     const uint32_t out_tiles = out >> 4, nw = n >> 1;
     const QuadPlan<WIDE> plan = quad_plan<WIDE>(n, lane);
-    const QuadWords<WIDE> words = quad_load<WIDE>(w + (static_cast<size_t>(tk) * out_tiles + tn) * nw, plan);
-    uint32_t cw[4];
-    quad_codewords<WIDE>(words, plan, wbits, cw);
+    const uint32_t* row = w + static_cast<size_t>(tk) * out_tiles * nw;
+    const uint32_t first = blockIdx.x * kDqSteps;  // 128-column pieces
+    // a tile past the row's last reads tile 0 again: decoded, staged and never stored
+    auto fetch = [&](uint32_t piece, QuadWords<WIDE>(&wd)[2]) {
 #pragma unroll
-    for (uint32_t m = 0; m < 4u; ++m) stage[quad_row(lane, m)][sg * 16u + quad_col(lane)] = decode_exact<CB>(cw[m]);
-    __syncthreads();
-    const uint32_t r = threadIdx.x >> 4, c4 = (threadIdx.x & 15u) * 4u;
-    const uint2 v = *reinterpret_cast<const uint2*>(&stage[r][c4]);
-    *reinterpret_cast<uint2*>(w_hat + (static_cast<size_t>(tk) * 16u + r) * out + blockIdx.x * 64u + c4) = v;
+        for (uint32_t t = 0; t < 2u; ++t) {
+            const uint32_t tn = piece * 8u + 2u * sg + t;
+            wd[t] = quad_load<WIDE>(row + static_cast<size_t>(tn < out_tiles ? tn : 0u) * nw, plan);
+        }
+    };
+    QuadWords<WIDE> cur[2], nxt[2];
+    fetch(first, cur);
+    const uint32_t r = threadIdx.x >> 4, c8 = (threadIdx.x & 15u) * 8u;
+    for (uint32_t s = 0; s < kDqSteps; ++s) {
+        const uint32_t piece = first + s;
+        if (piece * 128u >= out) break;  // uniform over the workgroup
+        if (s + 1u < kDqSteps) fetch(piece + 1u, nxt);
+        uint16_t(*st)[128 + 8] = stage[s & 1u];
+#pragma unroll
+        for (uint32_t t = 0; t < 2u; ++t) {
+            uint32_t cw[4];
+            quad_codewords<WIDE>(cur[t], plan, wbits, cw);
+#pragma unroll
+            for (uint32_t m = 0; m < 4u; ++m)
+                st[quad_row(lane, m)][(2u * sg + t) * 16u + quad_col(lane)] = decode_exact<CB>(cw[m]);
+        }
+        __syncthreads();
+        const uint32_t col = piece * 128u + c8;
+        if (col < out)  // out is a multiple of 64: a piece's second half may lie past the end
+            *reinterpret_cast<uint4*>(w_hat + (static_cast<size_t>(tk) * 16u + r) * out + col) =
+                *reinterpret_cast<const uint4*>(&st[r][c8]);
+#pragma unroll
+        for (uint32_t t = 0; t < 2u; ++t) cur[t] = nxt[t];
+    }
 }
 
 __global__ void __launch_bounds__(256) test_codebooks_kernel(uint16_t* mcg, uint16_t* mul1, uint16_t* t) {
@@ -75,7 +103,7 @@ __global__ void __launch_bounds__(64) test_mfma_kernel(const uint16_t* a, const 
 
 hipError_t launch_dequant(const uint32_t* trellis, uint16_t* w_hat, uint32_t in, uint32_t out, uint32_t n,
                           uint32_t wbits, int codebook, hipStream_t s) {
-    const dim3 grid(out / 64u, in / 16u), block(256);
+    const dim3 grid((out + 128u * kDqSteps - 1u) / (128u * kDqSteps), in / 16u), block(256);
     const bool mcg = codebook == kMcg || codebook == kMcgPair;
     with_reader(n, [&](auto reader) {
         constexpr int R = decltype(reader)::value;

@@ -168,9 +168,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
         const float4v v = ((red[0][i] + red[1][i]) + red[2][i]) + red[3][i];
         float* dst = z + (static_cast<size_t>(ksl) * rkt + rk) * out + (blk * BT + t) * 16u + 4u * (i & 3u);
         if constexpr (ARRIVE) {
-            if (s.live)
-#pragma unroll
-                for (int c = 0; c < 4; ++c) store_coherent(dst + c, v[c]);
+            if (s.live) store_coherent4(dst, v);
         } else {
             *reinterpret_cast<float4v*>(dst) = v;
         }
