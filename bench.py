@@ -488,12 +488,12 @@ def main() -> int:
                 # the launch that reads two thirds of the code bytes; up to two rows the mid stage runs inside the down
                 # launch, above that the gate|up launch's last arriver at a block runs it
                 "roofline": {"bound": "hbm",
-                             "kernel": "t3::moe_gemv<gate|up, prepare in LDS" + (">" if tokens <= 2 else ", arriving mid>"),
+                             "kernel": "t3::moe_gemv<gate|up, prepare in LDS" + (">" if tokens <= 4 else ", arriving mid>"),
                              "us_per_launch": t_gu * 1e6, "algorithmic_bytes_per_launch": gu_bytes,
                              "achieved": gu_bytes / t_gu / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                              "frac": gu_bytes / t_gu / HBM_PEAK},
-                "launches": {("gate_up_us" if tokens <= 2 else "gate_up_mid_us"): t_gu * 1e6,
-                             ("mid_down_combine_us" if tokens <= 2 else "down_combine_us"): t_dn * 1e6}})
+                "launches": {("gate_up_us" if tokens <= 4 else "gate_up_mid_us"): t_gu * 1e6,
+                             ("mid_down_combine_us" if tokens <= 4 else "down_combine_us"): t_dn * 1e6}})
             del m
             torch.cuda.empty_cache()
 

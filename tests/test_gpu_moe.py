@@ -121,8 +121,8 @@ def test_launch_forms_give_the_same_bytes(oracle, t3):
     # row (the arrival counters go back to zero), with skipped slots, a clamp and a shared expert in
     # the same launches
     rng = np.random.default_rng(9)
-    # one and two rows: the two-launch form runs the mid stage inside the down launch there
-    for codebook, n, rows, topk in ((MCG, 64, 5, 4), (MUL1, 48, 16, 4), (MUL1, 96, 3, 2), (MCG, 48, 1, 4), (MUL1, 64, 2, 3),
+    # up to four rows the two-launch form runs the mid stage inside the down launch
+    for codebook, n, rows, topk in ((MCG, 64, 5, 4), (MUL1, 48, 16, 4), (MUL1, 96, 3, 2), (MCG, 48, 1, 4), (MUL1, 64, 2, 3), (MCG, 64, 4, 3),
                                     (MUL1, 96, 1, 2)):
         bank = oracle.synth_bank(rng, 8, 512, 256, n)
         shared = oracle.synth_bank(rng, 1, 512, 256, n)

@@ -75,7 +75,7 @@ struct MoeLaunch {
     float* zd = nullptr;         // f32 [ks_dn][RKT][hidden]
     uint32_t hidden = 0, inter = 0, rows = 0, topk = 0, shared_slots = 0;
     uint32_t n_gu = 0, n_dn = 0, wbits = 16;
-    uint32_t per_gu = 8, per_dn = 4, parts_gu = 0, parts_dn = 0, ks_gu = 1, ks_dn = 1, bt_gu = 8, bt_dn = 8;
+    uint32_t per_gu = 8, per_dn = 8, parts_gu = 0, parts_dn = 0, ks_gu = 1, ks_dn = 1, bt_gu = 8, bt_dn = 8;
     int codebook = 0, dtype = 0, score_dt = 0, defer = 0;
     float limit = 0.0f;
     int clamp_at = 0;  // format.ClampAt: 0 gate_in (the gate clamped before its SiLU), 1 silu_out (the SiLU's output)

@@ -123,13 +123,15 @@ int32_t check_moe(const t3_array* x, const t3_bank* bank, const t3_array* inds, 
     l.limit = static_cast<float>(limit);
     l.clamp_at = clamp_at;
     // Partitions: functions of the bank's shapes alone. gate|up: a part is one 128-block of the input (8 tiles), so a
-    // wave can prepare its own block; down: 4 tiles a part, its input being prepared by the mid launch.
+    // wave can prepare its own block; down: the same (up to four rows a down wave runs the mid stage of its block
+    // itself). Four tiles a down part were measured too: twice the workgroups of half the length, 2-5 % slower from three
+    // rows up (8 tokens 63.5 against 62.0 us), because a down wave's 32 tiles are short against its launch's round trips.
     l.bt_gu = gemv_bt(l.n_gu);
     l.bt_dn = gemv_bt(l.n_dn);
     l.per_gu = 8;
     l.parts_gu = (l.hidden / 16u) / l.per_gu;
     l.ks_gu = (l.parts_gu + 3u) / 4u;
-    l.per_dn = 4;
+    l.per_dn = 8;
     l.parts_dn = (l.inter / 16u) / l.per_dn;
     l.ks_dn = (l.parts_dn + 3u) / 4u;
     return T3_OK;

@@ -42,7 +42,7 @@ __global__ void __launch_bounds__(64) moe_prep(const MoeLaunch a) {
 // itself in at its 128-column block, and the last to arrive runs that block's next stage on the complete planes:
 // gate|up -> the slot's mid block (counter a (row-slot, block of inter)); down -> the row's combine block (counter a
 // (row, block of hidden); skipped slots count themselves in too). The statements are the chain's, so are the bytes.
-constexpr uint32_t kMidInDownRows = 2u;
+constexpr uint32_t kMidInDownRows = 4u;
 
 // a workgroup's static LDS: the four waves' stages while they stream, their partial sums afterwards
 template <int BT>
@@ -96,9 +96,8 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
     if (part < parts && s.live) {  // uniform over the wave; a wave past the last part adds zeros below
         uint32_t xoff[1];
         if constexpr (XLDS && NPROJ == 1) {
-            // The down's input made here: the wave runs the mid stage of the 128-block its four input tiles lie in
-            // (the block's other half is the next wave's, which does the same) over the gate|up launch's planes and
-            // keeps its own half in LDS.
+            // The down's input made here: the wave runs the mid stage of its own 128-block (its eight input tiles) over
+            // the gate|up launch's planes and keeps the prepared block in LDS.
             extern __shared__ __attribute__((aligned(16))) unsigned char xdyn[];
             unsigned char* xst = xdyn + sg * ((per + 1u) * (kXldsRows * 64u));
             xoff[0] = (lane >> 4) * 16u;
@@ -108,9 +107,11 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
             uint32_t hh[2];
             float sum;
             routed_mid_values<false, false, 0>(a, s, rk, tk0 >> 3, lane, hh, sum);
-            const uint32_t mine = (tk0 >> 2) & 1u ? hh[1] : hh[0];  // elements 64 half + lane of the block
-            *reinterpret_cast<uint32_t*>(xst + ((lane >> 4) * kXldsRows) * 64u + quad_slot(lane & 15u) * 4u) =
-                mine | (mine << 16);
+            // element 64 j + lane of the block belongs to its tile row 4 j + lane / 16
+#pragma unroll
+            for (uint32_t j = 0; j < 2u; ++j)
+                *reinterpret_cast<uint32_t*>(xst + ((4u * j + (lane >> 4)) * kXldsRows) * 64u + quad_slot(lane & 15u) * 4u) =
+                    hh[j] | (hh[j] << 16);
             // every column workgroup of the slot stores the same sum; the row's combine, later in this launch, reads it
             if (a.defer && lane == 0u) store_coherent(a.hs + static_cast<size_t>(rk) * (a.inter / 128u) + (tk0 >> 3), sum);
             for (uint32_t i = lane; i < kXldsRows * 16u; i += 64u)
