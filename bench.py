@@ -54,10 +54,11 @@ def code_bytes(in_f: int, out_f: int, n: int) -> int:
     return (in_f // 16) * (out_f // 16) * n * 2
 
 
-def graph_time(torch, call, steps: int, warmup: int) -> float:
+def graph_time(torch, call, steps: int, warmup: int, replays: int = 1) -> float:
     """Seconds a call over exactly `steps` back-to-back calls `call(i, stream)`, captured once into a HIP graph (as a
     serving loop would hold its decode step) so the host's per-launch cost stays out of the GPU's timeline; events
-    bracket one replay on the launch stream."""
+    bracket one replay on the launch stream. `replays` > 1 (the cells beside the headline, which time fewer steps): the
+    median of that many timed replays of the same `steps` calls."""
     cur = torch.cuda.current_stream().cuda_stream
     for i in range(max(warmup, 1)):
         call(i, cur)
@@ -71,12 +72,15 @@ def graph_time(torch, call, steps: int, warmup: int) -> float:
         torch.cuda.synchronize()
         graph.replay()  # untimed: the graph's first replay uploads it
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(side)
-        graph.replay()
-        e1.record(side)
-        torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e-3 / steps
+        took = []
+        for _ in range(replays):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(side)
+            graph.replay()
+            e1.record(side)
+            torch.cuda.synchronize()
+            took.append(e0.elapsed_time(e1))
+    return sorted(took)[len(took) // 2] * 1e-3 / steps
 
 
 def host_u16(t) -> np.ndarray:
@@ -149,17 +153,18 @@ class Dense:
                 "x": self.xr[rows_to_check].to(torch.float32).cpu().numpy(),
                 "y": self.y[rows_to_check, 128 * blk:128 * blk + 128].to(torch.float32).cpu().numpy()}
 
-    def time(self, steps: int, warmup: int, stages: int = 0) -> float:
-        return graph_time(self.torch, lambda i, s: self.call(i, s, stages), steps, warmup)
+    def time(self, steps: int, warmup: int, stages: int = 0, replays: int = 3) -> float:
+        return graph_time(self.torch, lambda i, s: self.call(i, s, stages), steps, warmup, replays)
 
 
-def dense_cell(d: Dense, rows: int, steps: int, warmup: int, todo: list, name: str, gemv_alone: bool = False) -> dict:
+def dense_cell(d: Dense, rows: int, steps: int, warmup: int, todo: list, name: str, gemv_alone: bool = False,
+               replays: int = 3) -> dict:
     import torch
     d.bind(rows)
     bf16 = d.x.dtype == torch.bfloat16
     todo.append(d.sample(name, blk=(d.out_f // 128) // 3, rows_to_check=[0, rows - 1],
                          bar=BF16_DENSE_BAR if bf16 else F32_BAR, half_ulp=2.0 ** -8 if bf16 else 2.0 ** -11))
-    t = d.time(steps, warmup)
+    t = d.time(steps, warmup, replays=replays)
     out = {"n": d.n, "k": d.n / 16, "rows": rows, "code_bytes": d.cb, "copies": d.copies, "us_per_call": t * 1e6,
            "call_gbps": d.cb / t / 1e9, "frac_of_hbm": d.cb / t / HBM_PEAK,
            "plan": {key: d.plan[key] for key in ("path", "launches", "tiles_a_load", "k_slices", "tiles_a_wave", "workgroups")}}
@@ -226,8 +231,8 @@ class Moe:
         if st != 0:
             raise RuntimeError(self.L.t3_error_name(st).decode())
 
-    def time(self, steps: int, warmup: int, stages: int = 63) -> float:
-        return graph_time(self.torch, lambda i, s: self.call(i, s, stages), steps, warmup)
+    def time(self, steps: int, warmup: int, stages: int = 63, replays: int = 3) -> float:
+        return graph_time(self.torch, lambda i, s: self.call(i, s, stages), steps, warmup, replays)
 
     def sample(self, name: str, token: int, bar: float):
         """One eager call over routing 0, and the chosen token's experts for ref.moeRowClamped on the host."""
@@ -378,7 +383,8 @@ def main() -> int:
     # ---- the headline: one row of the q|k|v shape --------------------------------------------------------------
     n_head = 16 * args.k
     d = Dense(torch, api, IN_F, OUT_F, n_head, MCG_CB, 32, torch.float16, seed=1000 + args.k)
-    head = dense_cell(d, args.rows, args.steps, args.warmup, todo, f"headline K{args.k} rows {args.rows}", gemv_alone=True)
+    head = dense_cell(d, args.rows, args.steps, args.warmup, todo, f"headline K{args.k} rows {args.rows}", gemv_alone=True,
+                      replays=1)  # the headline: exactly --steps calls, timed once
     one_launch = head["plan"]["launches"] == 1
     out = {
         "metric": "EXL3 GEMV HBM GB/s (% of 8 TB/s) at decode rows; MoE prefill GEMM TFLOP/s",
