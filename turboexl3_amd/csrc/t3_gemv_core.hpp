@@ -5,8 +5,9 @@
 // Memory path. A tile row's BT tiles are contiguous (BT * 2n bytes <= 1 KB), so the wave fetches them with ONE
 // 128-bit buffer load, 16 consecutive bytes a lane: the texture unit sees a fully coalesced stream (a gather of each
 // lane's own words costs it many times the cycles, measured). The loaded registers go to a wave-private LDS stage,
-// one 256-byte slot a tile, and every lane reads back the two (or four) words its quad needs. ST such loads stay in
-// flight in a register ring, fully unrolled, with scalar row offsets: the loop spends no vector ALU on addresses.
+// one 256-byte slot a tile, and every lane reads back the two words its quad needs (four at the wide rates whose quads
+// pass two words). ST such loads stay in flight in a register ring, fully unrolled, with scalar row offsets: the loop
+// spends no vector ALU on addresses.
 // A row past the wave's last is read through a zero-sized buffer: the hardware returns zeros without touching memory.
 // LDS operations of one wave complete in order, so the stage needs no barrier.
 //

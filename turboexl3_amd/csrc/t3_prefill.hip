@@ -101,7 +101,8 @@ __device__ __forceinline__ void wait_loads() {
 //
 // The operands reach LDS without passing through registers, D steps deep (a step = K 32 = two tile rows):
 //   weights      a wave's four tiles of a tile row, one load: lane L brings bytes 16 (L % 16).. of tile L / 16 to the
-//                tile's 256-byte slot; each lane then reads back the two (four) words its quad's windows span;
+//                tile's 256-byte slot; each lane then reads back the two words its quad's windows span (four where a wide
+//                rate's quads pass two words);
 //   activations  the item's rows, 64 bytes a row a step, 16 rows a load. Row r's 16-byte piece p is kept at position
 //                p ^ ((r >> 1) & 3) of the row, which spreads a B fragment's reads (16 rows, one piece each) over the
 //                banks at row stride 64 (measured: 4.2 cycles a wave's read, 8 unswizzled).
