@@ -21,6 +21,7 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
 
 // A raw buffer over `bytes` bytes from p: loads take a per-lane byte offset (VGPR) plus a uniform byte offset (SGPR),
 // so a streaming loop spends no vector ALU on addresses, and a read past the end returns zero instead of faulting.

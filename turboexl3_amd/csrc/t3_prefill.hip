@@ -36,6 +36,8 @@ struct PfGemm {
     uint32_t spread;  // dies one item's column blocks go round: 1 with eight items or more a launch, up to 8 with one
     uint32_t kparts;  // K parts (grid z): part k multiplies its share of the tile rows into plane k of z
     uint32_t plane;   // elements between z's planes
+    uint32_t zhalf;   // z holds f16 [positions][out] (the sums rounded at the launch's end) instead of f32: one K part, and
+                      // a finish that starts by rounding them (no deferred map, not GLM's profile)
 };
 
 // The weight a GEMM feeds the matrix core as one f16: exact, or MUL1's h = 1024 + t when its map is deferred.
@@ -267,10 +269,21 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(LBMAX 
         for (int mb = 0; mb < LB; ++mb) {
             const uint32_t row = static_cast<uint32_t>(mb) * 16u + (lane & 15u);
             if (row >= count) continue;
+            const size_t at = static_cast<size_t>(first + row) * a.out + col0 * 16u + 4u * (lane >> 4);
+            if (a.zhalf) {  // uniform
+                uint16_t* zh = reinterpret_cast<uint16_t*>(z);
 #pragma unroll
-            for (uint32_t t = 0; t < kPfTiles; ++t)
-                *reinterpret_cast<float4v*>(z + static_cast<size_t>(first + row) * a.out + (col0 + t) * 16u +
-                                            4u * (lane >> 4)) = acc[mb][t];
+                for (uint32_t t = 0; t < kPfTiles; ++t) {
+                    const float4v v = acc[mb][t];
+                    uint2v h;
+                    h[0] = static_cast<uint32_t>(half_bits(v[0])) | (static_cast<uint32_t>(half_bits(v[1])) << 16);
+                    h[1] = static_cast<uint32_t>(half_bits(v[2])) | (static_cast<uint32_t>(half_bits(v[3])) << 16);
+                    *reinterpret_cast<uint2v*>(zh + at + t * 16u) = h;
+                }
+            } else {
+#pragma unroll
+                for (uint32_t t = 0; t < kPfTiles; ++t) *reinterpret_cast<float4v*>(z + at + t * 16u) = acc[mb][t];
+            }
         }
     };
 
@@ -453,8 +466,9 @@ __global__ void __launch_bounds__(256) pf_mid(const MoeLaunch a) {
     const size_t eo = static_cast<size_t>(s.e) * a.inter, qo = static_cast<size_t>(pos) * a.inter;
     const Row16 g16 = row16(lane);
     float gt[8], up[8], svg[8], svu[8], sdn[8];
-    load8_f32(a.zg, qo + i, gt);
-    load8_f32(a.zu, qo + i, up);
+    const bool zhalf = PROF == 0 && !a.defer;
+    load8_plane(a.zg, qo + i, zhalf, gt);
+    load8_plane(a.zu, qo + i, zhalf, up);
     load8_half(bank.gate_svh, eo + i, svg);
     load8_half(bank.up_svh, eo + i, svu);
     load8_half(bank.down_suh, eo + i, sdn);
@@ -535,7 +549,7 @@ __global__ void __launch_bounds__(256) pf_combine(const MoeLaunch a) {
         const uint32_t pos = a.inv[rk];
         const RoutedBank& bank = s.shared ? a.shared : a.bank;
         float v[8], sv[8];
-        load8_f32(a.zd, static_cast<size_t>(pos) * a.hidden + i, v);
+        load8_plane(a.zd, static_cast<size_t>(pos) * a.hidden + i, !a.defer, v);
         load8_half(bank.down_svh, static_cast<size_t>(s.e) * a.hidden + i, sv);
         if (a.defer) {
             float xsum = 0.0f;
@@ -608,7 +622,7 @@ __global__ void __launch_bounds__(256) pf_dense_finish(const float* z, const flo
     const Row16 g16 = row16(lane);
     const size_t at = static_cast<size_t>(row) * out + i;
     float v[8], sv[8];
-    load8_f32(z, at, v);
+    load8_plane(z, at, ks == 1u && !defer, v);
     const size_t plane = static_cast<size_t>(rows) * out;
     for (uint32_t k = 1; k < ks; ++k) {
         float part[8];
@@ -723,6 +737,7 @@ hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s) {
     g.wbits = a.wbits;
     g.positions = p;
     g.experts = a.bank.experts;
+    g.zhalf = !a.defer && !a.glm;
     if (a.stages & 4u)
         if ((e = launch_gemm(g, a.codebook, a.max_items, 2u, a.item_rows, s)) != hipSuccess) return e;
 
@@ -772,6 +787,7 @@ hipError_t launch_dense_prefill(const DenseLaunch& d, hipStream_t s) {
     g.experts = 1u;
     g.kparts = d.ks;
     g.plane = d.rows * d.out;
+    g.zhalf = d.ks == 1u && d.codebook != kMul1Defer;
     const uint32_t item_rows = d.rows <= 64u ? 64u : 128u;
     if ((e = launch_gemm(g, d.codebook, (d.rows + item_rows - 1u) / item_rows, 1u, item_rows, s)) != hipSuccess) return e;
     return launch_pf_dense_finish(d, d.z, s);

@@ -241,6 +241,14 @@ __device__ __forceinline__ void load8_half(const uint16_t* p, size_t i, float (&
         o[2u * k + 1u] = half_value(w[k] >> 16);
     }
 }
+// Eight adjacent sums of a GEMM's output plane: f32, or already rounded to f16 where the plane is the chain's z itself
+// (one K part and no deferred map: the rounding the finish would start with was done at the GEMM's end).
+__device__ __forceinline__ void load8_f32(const float* p, size_t i, float (&o)[8]);
+__device__ __forceinline__ void load8_half(const uint16_t* p, size_t i, float (&o)[8]);
+__device__ __forceinline__ void load8_plane(const float* p, size_t i, bool half, float (&o)[8]) {
+    if (half) load8_half(reinterpret_cast<const uint16_t*>(p), i, o);
+    else load8_f32(p, i, o);
+}
 __device__ __forceinline__ void load8_f32(const float* p, size_t i, float (&o)[8]) {
     const float4v a = *reinterpret_cast<const float4v*>(p + i), b = *reinterpret_cast<const float4v*>(p + i + 4);
 #pragma unroll
