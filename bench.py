@@ -15,7 +15,8 @@ against 8 TB/s; `gemv_launch_alone` is the chain's GEMV launch without prepare a
 `launch_floor` what the chain's two small launches cost alone (what any launch costs in a replayed graph). Beside
 them, unless --quick: `sweep` (the metric's K = 3, 4, 5 x rows = 1, 4, 16, 32), `lm_head` (4096 -> 151936 at K6, 1 and
 256 rows), `moe_decode` (config 3 at 1 and 8 tokens, each launch timed alone as well), `moe_prefill` (config 4, each
-stage timed alone; TFLOP/s against the 2.5 PFLOP/s f16 MFMA figure and against a dense f16 GEMM measured in this
+stage timed alone, and the same call over MUL1's codebook; TFLOP/s against the 2.5 PFLOP/s f16 MFMA figure and against a
+dense f16 GEMM measured in this
 process, `measured_dense_f16_peak`), `dense_prefill` (config 5's 4096 rows and its resident-weight forms),
 `codebook_forms` (the price of exact f16 weights in the GEMV), `rates` (a fractional narrow rate and a wide one) and
 `dense_rows` (few-row dense calls with and without the rows-alone partition). `cpu_baseline`: the CPU oracle
@@ -250,7 +251,7 @@ class Moe:
             arrays[nm + "_suh"] = side(p.suh, q.suh if s else None)
             arrays[nm + "_svh"] = side(p.svh, q.svh if s else None)
         scores = self.scores[0, token].tolist() + ([1.0] if s else [])
-        return {"kind": "moe", "cell": name, "hidden": self.hidden, "inter": self.inter, "n_gu": self.n_gu, "n_dn": self.n_dn,
+        return {"kind": "moe", "cell": name, "codebook": self.dec.codebook, "hidden": self.hidden, "inter": self.inter, "n_gu": self.n_gu, "n_dn": self.n_dn,
                 "limit": float(self.limit), "bar": bar, "arrays": arrays, "scores": np.asarray(scores, dtype=np.float32),
                 "x": self.x[0, token].to(torch.float32).cpu().numpy(), "y": self.y[0, token].to(torch.float32).cpu().numpy()}
 
@@ -326,7 +327,7 @@ def cpu_leg(n: int, seed: int, todo: list, budget_s: float = 20.0):
             a = s["arrays"]
             bank = oracle.Bank(a["gate_t"].shape[0], s["hidden"], s["inter"], s["n_gu"], s["n_dn"], a["gate_t"], a["gate_suh"],
                                a["gate_svh"], a["up_t"], a["up_suh"], a["up_svh"], a["down_t"], a["down_suh"], a["down_svh"])
-            want, _ = oracle.moe_row(bank, s["x"], np.arange(len(s["scores"]), dtype=np.int32), s["scores"], oracle.MCG,
+            want, _ = oracle.moe_row(bank, s["x"], np.arange(len(s["scores"]), dtype=np.int32), s["scores"], s["codebook"],
                                      0xFFFF, s["limit"])
             err = oracle.compare(s["y"], want, 2.0 ** -8)
         checks.append({"cell": s["cell"], "err_over_rms": err, "bar": s["bar"], "ok": bool(err <= s["bar"])})
@@ -522,6 +523,12 @@ def main() -> int:
                          "peak": MFMA_F16_PEAK / 1e12, "unit": "TFLOP/s", "frac": gu_flops / t_gu / MFMA_F16_PEAK,
                          "frac_of_measured_f16_peak": (gu_flops / t_gu / 1e12 / peak_meas) if peak_meas else None},
             "stages_us": {nm: v * 1e6 for nm, v in stage_t.items()}}
+        # the same call over the same codes read as MUL1 (the deferred map: h = 1024 + t as the weight, three vector
+        # operations a weight in the GEMM's decode instead of MCG's four)
+        m.dec = api.Decode(MUL1_CB, 16)
+        todo.append(m.sample("moe_prefill MUL1 token 0", 0, BF16_MOE_BAR))
+        t1 = m.time(5, 2)
+        out["moe_prefill"]["mul1_codebook"] = {"ms_per_call": t1 * 1e3, **both(m.flops, t1)}
         del m
         torch.cuda.empty_cache()
 

@@ -58,8 +58,12 @@ __device__ __forceinline__ void finish_block(int dt, const float* z, const float
                                              uint32_t row, uint32_t b, uint32_t lane) {
     auto get_z = [](const float* p) { return ZCOH ? load_coherent(p) : *p; };
     auto get_x = [](const float* p) { return XCOH ? load_coherent(p) : *p; };
-    float xsum = 0.0f;
-    if (defer)
+    // The deferred map's sum of the row's block sums, 0 + s[0] + s[1] + ... in block order. Up to 64 blocks: one load
+    // across the wave's lanes, in flight beside the planes' loads, added up lane by lane afterwards; more: eight at a time.
+    float xsum = 0.0f, xmine = 0.0f;
+    const bool xwave = defer && inblk <= 64u;
+    if (xwave && lane < inblk) xmine = get_x(xs_row + lane);
+    if (defer && !xwave)
         for (uint32_t q0 = 0; q0 < inblk; q0 += 8u) {
             float part[8];
 #pragma unroll
@@ -86,6 +90,9 @@ __device__ __forceinline__ void finish_block(int dt, const float* z, const float
                 acc[1] = k0 + k == 0u ? part[k][1] : acc[1] + part[k][1];
             }
     }
+    if (xwave)
+        for (uint32_t q = 0; q < inblk; ++q)
+            xsum += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, xmine), static_cast<int>(q)));
 #pragma unroll
     for (uint32_t j = 0; j < 2u; ++j) {
         float s = acc[j];

@@ -473,11 +473,8 @@ __global__ void __launch_bounds__(256) pf_mid(const MoeLaunch a) {
     load8_half(bank.up_svh, eo + i, svu);
     load8_half(bank.down_suh, eo + i, sdn);
     if (a.defer) {
-        float xg = 0.0f, xu = 0.0f;
-        for (uint32_t t = 0; t < nbh; ++t) {
-            xg += a.sg[static_cast<size_t>(pos) * nbh + t];
-            xu += a.su[static_cast<size_t>(pos) * nbh + t];
-        }
+        const float xg = wave_ordered_sum(a.sg + static_cast<size_t>(pos) * nbh, nbh, lane);
+        const float xu = wave_ordered_sum(a.su + static_cast<size_t>(pos) * nbh, nbh, lane);
 #pragma unroll
         for (uint32_t r = 0; r < 8u; ++r) {
             gt[r] = __builtin_fmaf(gt[r], mul1_a(), mul1_b() * xg);
@@ -520,8 +517,7 @@ __global__ void __launch_bounds__(256) pf_slots(const MoeLaunch a) {
     load8_f32(a.zd, static_cast<size_t>(pos) * a.hidden + i, v);
     load8_half(a.bank.down_svh, static_cast<size_t>(s.e) * a.hidden + i, sv);
     if (a.defer) {
-        float xsum = 0.0f;
-        for (uint32_t t = 0; t < nbi; ++t) xsum += a.hs[static_cast<size_t>(pos) * nbi + t];
+        const float xsum = wave_ordered_sum(a.hs + static_cast<size_t>(pos) * nbi, nbi, lane);
 #pragma unroll
         for (uint32_t r = 0; r < 8u; ++r) v[r] = __builtin_fmaf(v[r], mul1_a(), mul1_b() * xsum);
     }
@@ -552,8 +548,7 @@ __global__ void __launch_bounds__(256) pf_combine(const MoeLaunch a) {
         load8_plane(a.zd, static_cast<size_t>(pos) * a.hidden + i, !a.defer, v);
         load8_half(bank.down_svh, static_cast<size_t>(s.e) * a.hidden + i, sv);
         if (a.defer) {
-            float xsum = 0.0f;
-            for (uint32_t t = 0; t < nbi; ++t) xsum += a.hs[static_cast<size_t>(pos) * nbi + t];
+            const float xsum = wave_ordered_sum(a.hs + static_cast<size_t>(pos) * nbi, nbi, lane);
 #pragma unroll
             for (uint32_t r = 0; r < 8u; ++r) v[r] = __builtin_fmaf(v[r], mul1_a(), mul1_b() * xsum);
         }
@@ -632,8 +627,7 @@ __global__ void __launch_bounds__(256) pf_dense_finish(const float* z, const flo
     }
     load8_half(svh, i, sv);
     if (defer) {
-        float xsum = 0.0f;
-        for (uint32_t t = 0; t < inblk; ++t) xsum += xs[static_cast<size_t>(row) * inblk + t];
+        const float xsum = wave_ordered_sum(xs + static_cast<size_t>(row) * inblk, inblk, lane);
 #pragma unroll
         for (uint32_t r = 0; r < 8u; ++r) v[r] = __builtin_fmaf(v[r], mul1_a(), mul1_b() * xsum);
     }

@@ -241,6 +241,20 @@ __device__ __forceinline__ void load8_half(const uint16_t* p, size_t i, float (&
         o[2u * k + 1u] = half_value(w[k] >> 16);
     }
 }
+// 0 + p[0] + p[1] + ... + p[count - 1] in that order, the same value in every lane: up to 64 terms come with one load across
+// the wave's lanes (one round trip, not one a term) and are added lane by lane; more go one by one.
+__device__ __forceinline__ float wave_ordered_sum(const float* p, uint32_t count, uint32_t lane) {
+    float acc = 0.0f;
+    if (count <= 64u) {
+        const float mine = lane < count ? p[lane] : 0.0f;
+        for (uint32_t q = 0; q < count; ++q)
+            acc += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), static_cast<int>(q)));
+    } else {
+        for (uint32_t q = 0; q < count; ++q) acc += p[q];
+    }
+    return acc;
+}
+
 // Eight adjacent sums of a GEMM's output plane: f32, or already rounded to f16 where the plane is the chain's z itself
 // (one K part and no deferred map: the rounding the finish would start with was done at the GEMM's end).
 __device__ __forceinline__ void load8_f32(const float* p, size_t i, float (&o)[8]);
