@@ -16,8 +16,8 @@ against 8 TB/s; `gemv_launch_alone` is the chain's GEMV launch without prepare a
 them, unless --quick: `sweep` (the metric's K = 3, 4, 5 x rows = 1, 4, 16, 32), `lm_head` (4096 -> 151936 at K6, 1 and
 256 rows), `moe_decode` (config 3 at 1 and 8 tokens, each launch timed alone as well), `moe_prefill` (config 4, each
 stage timed alone, and the same call over MUL1's codebook; TFLOP/s against the 2.5 PFLOP/s f16 MFMA figure and against a
-dense f16 GEMM measured in this
-process, `measured_dense_f16_peak`), `dense_prefill` (config 5's 4096 rows and its resident-weight forms),
+dense f16 GEMM measured in this process, `measured_dense_f16_peak`), `dense_prefill` (config 5's 4096 rows and its
+resident-weight forms),
 `codebook_forms` (the price of exact f16 weights in the GEMV), `rates` (a fractional narrow rate and a wide one) and
 `dense_rows` (few-row dense calls with and without the rows-alone partition). `cpu_baseline`: the CPU oracle
 (`format.project` restated in C) timed on this box's host cores, and, in the same leg, one sampled output block (or row)
