@@ -152,6 +152,29 @@ def test_launch_forms_give_the_same_bytes(oracle, t3):
         assert not ws[:65536].any()
 
 
+def test_launch_forms_give_the_same_bytes_at_the_reference_rows(oracle, t3):
+    # src/hip_tests.zig:891-895,907: the reference's model-sized case (2560 x 640, 16 experts, top-10, K3, MUL1's deferred
+    # map, bf16) at its rows 1-5, 8 and 16
+    rng = np.random.default_rng(0x909)
+    hidden, inter, experts, topk = 2560, 640, 16, 10
+    bank = oracle.synth_bank(rng, experts, hidden, inter, 48)
+    dbank = dev_bank(t3, bank)
+    x_dev, _ = make_x(rng, 16, hidden, torch.bfloat16)
+    slots, scores = routing(rng, 16, topk, experts)
+    dec = t3.Decode(MUL1, 16)
+    for rows in (1, 2, 3, 4, 5, 8, 16):
+        args = (x_dev[:rows].reshape(1, rows, hidden), dbank, torch.from_numpy(slots[:rows]).cuda().reshape(1, rows, topk),
+                torch.from_numpy(scores[:rows]).cuda().reshape(1, rows, topk), dec)
+        nine = t3.moe(*args)
+        for form in (3, 4):
+            t3.configure(decode_form=form)
+            try:
+                other = t3.moe(*args)
+            finally:
+                t3.configure()
+            assert bytes_of(nine) == bytes_of(other), f"rows {rows}: form 9 differs from form {form}"
+
+
 @pytest.mark.parametrize("hidden,inter,experts,topk,n", [(128, 128, 1, 1, 64), (128, 256, 3, 2, 16), (384, 128, 5, 3, 128),
                                                          (256, 384, 4, 4, 34), (256, 256, 3, 2, 112), (256, 128, 3, 2, 96)])
 def test_smallest_and_odd_banks(oracle, t3, hidden, inter, experts, topk, n):
@@ -511,12 +534,14 @@ def _w_std64(oracle, trellis, suh, svh, in_f, out_f, n, codebook):
     return w * svh.view(np.float16).astype(np.float64)[None, :]
 
 
-@pytest.mark.parametrize("rows", [1, 4, 8, 40])
-def test_glm_profile_slots_against_float64(oracle, t3, rows):
-    # src/hip_tests.zig:576-671: every routed slot's f32 output within sum |a w| / 64 + 1e-6 of float64 under GLM's
-    # roundings, the slot past the experts (the host's shared expert) left alone; 40 rows take the prefill chain
+@pytest.mark.parametrize("hidden,inter,experts,rows", [(512, 256, 12, 1), (512, 256, 12, 4), (512, 256, 12, 8),
+                                                        (512, 256, 12, 40), (4096, 2048, 9, 8), (4096, 2048, 9, 40)])
+def test_glm_profile_slots_against_float64(oracle, t3, hidden, inter, experts, rows):
+    # src/hip_tests.zig:576-671,762-797 (both of its shapes): every routed slot's f32 output within
+    # sum |a w| / 64 + 1e-6 of float64 under GLM's roundings, the slot past the experts (the host's shared expert) left
+    # alone; 40 rows take the prefill chain, where the reference samples rows 0, 1, 20 and 39
     rng = np.random.default_rng(0x61A)
-    hidden, inter, experts, topk, n, limit = 512, 256, 12, 8, 64, 7.0
+    topk, n, limit = 8, 64, 7.0
     bank = oracle.synth_bank(rng, experts, hidden, inter, n)
     dbank = dev_bank(t3, bank)
     k = topk + 1
@@ -528,7 +553,8 @@ def test_glm_profile_slots_against_float64(oracle, t3, rows):
     assert np.isnan(got[:, topk]).all(), "the slot past the experts was written"
     worst = 0.0
     w64 = {}
-    for r in range(rows if rows <= 8 else 6):
+    sampled = range(rows) if rows <= 8 and hidden <= 512 else sorted({0, 1, rows // 2, rows - 1})
+    for r in sampled:
         xr = x_f32[r].astype(np.float64)
         for j in range(topk):
             e = int(slots[r, j])
@@ -545,4 +571,4 @@ def test_glm_profile_slots_against_float64(oracle, t3, rows):
             q = (np.abs(got[r, j] - want) / tol).max()
             assert q <= 1.0, f"rows {rows} row {r} slot {j}: {q:.3f} of its tolerance"
             worst = max(worst, q)
-    print(f"GLM profile rows {rows}: worst {worst:.3f} of the float64 tolerance")
+    print(f"GLM profile hidden {hidden} rows {rows}: worst {worst:.3f} of the float64 tolerance")
