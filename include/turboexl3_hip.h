@@ -105,7 +105,9 @@ typedef struct t3_bank {
 
 typedef struct t3_config {
     int32_t decode_form;   /* 3: the five-launch chain; 4: four launches (prepare inside gate|up); 9 (default): two
-                            * launches (mid and combine run by the last workgroup to arrive); others refused */
+                            * launches (mid and combine run by the last workgroup to arrive) while the gate|up launch
+                            * stays within 8192 workgroups, the five launches past that (large experts at many rows,
+                            * where they are faster); the same bytes whichever runs; others refused */
     int32_t dec_one;       /* 1 (default): dense decode rows in one launch; 0: the three-launch chain */
     int32_t prefill;       /* 1 (default); 0: routed calls above 16 rows refuse Exl3EngineNotImplemented */
     int32_t mcg_pair;      /* 1 (default): MCG's GEMV feeds the hashed pair to the matrix core unrounded; 0: the f16 weight */
@@ -234,7 +236,8 @@ int32_t t3_linear_unrot(t3_stream stream, const t3_array* x, const t3_array* w_s
 
 /* x [B, S, D]; inds (U32/I32) and scores (F32/BF16/F16) [B, S, K], K <= 32; y [B, S, D] in x's dtype.
  * `verify_rows` is accepted and ignored, as in the reference (src/root.zig:822-825). Up to 16 rows: the split-K GEMV
- * chain, two launches (four or five under decode_form 4 or 3, the same bytes). A routed id outside [0, E) is skipped. Gate and up
+ * chain, two launches (five for large experts at many rows; four or five under decode_form 4 or 3; the same bytes, and
+ * t3_moe_plan_of says which). A routed id outside [0, E) is skipped. Gate and up
  * must share a rate (T3_Exl3GateUpRateMismatch); the down's rate may differ (the reference refuses that,
  * src/root.zig:841; this library's kernels take a rate a launch). */
 int32_t t3_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
@@ -343,8 +346,9 @@ int32_t t3_moe_plan_of(const t3_array* x, const t3_bank* bank, const t3_array* i
  * src/kernels/hip/decode/decode.hip:8-13): x BF16 times suh in f32 (no f16 rounding of x), the inner products stay f32,
  * gate and up round to bf16 and are limited (limit 0: not), the SiLU rounds to bf16, the product rounds to bf16; y F32
  * [B, S, K, D]: each routed slot's own down finish, no score (the host combines a row's slots and its shared expert). A
- * slot whose id is outside [0, E) is skipped and its output left as it is. Any row count: the decode chain's five
- * launches up to 16 rows, the prefill chain above. Workspace: t3_moe_workspace_bytes (shared_bank NULL). */
+ * slot whose id is outside [0, E) is skipped and its output left as it is. Any row count: the decode chain up to 16 rows
+ * (the launch forms of t3_moe, the same bytes; the exact codebook forms and decode_form 4 take the five launches), the
+ * prefill chain above. Workspace: t3_moe_workspace_bytes (shared_bank NULL). */
 int32_t t3_moe_glm(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds, t3_decode dec,
                    int32_t limit, t3_array* y, void* workspace, size_t workspace_bytes);
 /* shared_bank: NULL, or the bank `t3_moe_shared_expert` will take (its slots need scratch too). */

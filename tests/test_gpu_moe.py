@@ -519,6 +519,32 @@ def test_fused_gated_shared_expert_with_the_gate_vector(oracle, t3, hidden, rows
         assert err.value.name == name, (kwargs.keys(), name)
 
 
+def test_glm_profile_launch_forms_give_the_same_bytes(oracle, t3):
+    # src/hip_tests.zig:896,900-913: form 9's bytes are form 3's under GLM's profile too (4096 x 2048, 9 experts, K4, MCG,
+    # bf16, the last slot of a row the host's shared expert), rows 1-5, 8 and 16; and with MUL1's deferred map
+    rng = np.random.default_rng(0x90A)
+    for hidden, inter, experts, n, codebook in ((4096, 2048, 9, 64, MCG), (512, 384, 6, 48, MUL1)):
+        topk = min(8, experts - 1)
+        k = topk + 1
+        bank = oracle.synth_bank(rng, experts, hidden, inter, n)
+        dbank = dev_bank(t3, bank)
+        x_dev, _ = make_x(rng, 16, hidden, torch.bfloat16)
+        slots = np.stack([np.concatenate([rng.permutation(experts)[:topk], [experts]]) for _ in range(16)]).astype(np.int32)
+        for rows in (1, 2, 3, 4, 5, 8, 16):
+            args = (x_dev[:rows].reshape(1, rows, hidden), dbank, torch.from_numpy(slots[:rows]).cuda().reshape(1, rows, k),
+                    t3.Decode(codebook, 16), 7)
+            two = t3.moe_glm(*args, fill=float("nan"))
+            again = t3.moe_glm(*args, fill=float("nan"))
+            assert bytes_of(two) == bytes_of(again)
+            t3.configure(decode_form=3)
+            try:
+                five = t3.moe_glm(*args, fill=float("nan"))
+            finally:
+                t3.configure()
+            assert bytes_of(two) == bytes_of(five), f"hidden {hidden} rows {rows}: two launches differ from five"
+            assert torch.isnan(two.reshape(rows, k, hidden)[:, topk]).all(), "the slot past the experts was written"
+
+
 def _bf16_round64(v):
     return torch.from_numpy(np.asarray(v, dtype=np.float32)).to(torch.bfloat16).to(torch.float64).numpy()
 

@@ -145,6 +145,17 @@ def test_decode_forms_by_configuration(lib):
             assert lib.t3_configure(C.byref(cfg)) == 0
 
 
+def test_decode_form_by_the_gate_up_launch_size(lib):
+    # two launches while the gate|up launch stays within 8192 workgroups (column groups x row-slots x 2 x K slices), five
+    # past that: 4096 x 2048 K4 top-8 has 16 x 8 r x 2 x 8 = 2048 r of them
+    for rows, launches in ((1, 2), (4, 2), (5, 5), (16, 5)):
+        assert moe_plan(lib, rows, 64, 4096, 2048, 8, 64, 64).launches == launches
+    # 7168 x 2048 K3 top-8: 16 x 8 r x 2 x 14 = 3584 r
+    assert [moe_plan(lib, rows, 256, 7168, 2048, 8, 48, 48).launches for rows in (1, 2, 3)] == [2, 2, 5]
+    # four tiles a load (K5) doubles the column groups: 4096 x 1024 has 16 x 8 r x 2 x 8 = 2048 r as well
+    assert [moe_plan(lib, rows, 64, 4096, 1024, 8, 80, 80).launches for rows in (4, 5)] == [2, 5]
+
+
 def test_plan_refusals(lib):
     p = LinearPlan()
     st = lib.t3_linear_plan_of(C.byref(arr(F16, 1, 4000)), C.byref(arr(U16, 256, 768, 64)), Decode(1, 16), C.byref(p))

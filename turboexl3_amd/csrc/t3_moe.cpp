@@ -197,13 +197,23 @@ int32_t admit_prefill(const MoeCall& call) {
 }
 
 // decode_form 3: the five-launch chain; 4: four launches; 9: two launches while a counter a (row-slot, 128-block) fits
-// the workspace's counter area, else four
+// the workspace's counter area (else four) and the gate|up launch stays within kTwoLaunchGroups workgroups (else five).
+// The two launches save three launch boundaries (~12 us of the chain) and pay with every gate|up workgroup's own prepare
+// of its block (once a column workgroup instead of once) and the coherent hand-offs, ~8 % of the decode at eight tiles a
+// load and twice that at four: past eight rounds of the GPU's resident workgroups the five launches are faster. Measured
+// (two against five, us): 4096 x 2048 K4 top-8 at 4 / 5 / 8 / 16 rows 148.7 / 177.0 / 270.8 / 515.5 against 148.5 / 175.3 /
+// 256.1 / 477.5; 7168 x 2048 K3 at 2 / 3 / 8 rows 131.9 / 189.0 / 449.4 against 133.9 / 180.1 / 415.6; 4096 x 1024 K5 at
+// 4 / 8 rows 96.6 / 170.9 against 95.7 / 159.2; 2048 x 512 K3 top-10 at 16 rows 97.1 against 103.1. Every form gives the
+// same bytes, so a row's bytes do not depend on which one its call took.
+constexpr uint64_t kTwoLaunchGroups = 8192u;
 int decode_form_of(const MoeLaunch& l) {
+    const uint64_t rkt = static_cast<uint64_t>(l.rows) * (l.topk + l.shared_slots);
     const size_t widest = (l.hidden > l.inter ? l.hidden : l.inter) / 128u;
-    const size_t counters = static_cast<size_t>(l.rows) * (l.topk + l.shared_slots) * widest;
-    return config().decode_form == 3 ? kMoeFiveLaunches
-           : config().decode_form == 4 || counters * 4u > kCounterBytes ? kMoeFourLaunches
-                                                                         : kMoeTwoLaunches;
+    const size_t counters = rkt * widest;
+    if (config().decode_form == 3) return kMoeFiveLaunches;
+    if (config().decode_form == 4 || counters * 4u > kCounterBytes) return kMoeFourLaunches;
+    const uint64_t gu_groups = static_cast<uint64_t>(l.inter / 16u / l.bt_gu) * rkt * 2u * l.ks_gu;
+    return gu_groups > kTwoLaunchGroups ? kMoeFiveLaunches : kMoeTwoLaunches;
 }
 
 int32_t run_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
@@ -370,7 +380,9 @@ int32_t t3_moe_glm(t3_stream stream, const t3_array* x, const t3_bank* bank, con
     }
     t3::carve_moe(&call, workspace);
     if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
-    return t3::hip_status(t3::launch_moe_decode(l, t3::kMoeFiveLaunches, s));
+    // the four-launch form has no GLM statements of its own: the five launches stand in for it
+    const int form = t3::decode_form_of(l);
+    return t3::hip_status(t3::launch_moe_decode(l, form == t3::kMoeFourLaunches ? t3::kMoeFiveLaunches : form, s));
 }
 
 namespace {

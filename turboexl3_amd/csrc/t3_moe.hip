@@ -51,7 +51,7 @@ constexpr uint32_t role_lds_bytes() {
     return stage > red ? stage : red;
 }
 
-template <int CB, int WIDE, int BT, int NPROJ, bool XLDS, bool ARRIVE>
+template <int CB, int WIDE, int BT, int NPROJ, bool XLDS, bool ARRIVE, int PROF>
 __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint32_t yidx, uint32_t ksl,
                                           unsigned char* smem, uint32_t& last_flag, uint32_t* cinfo, float* cscore) {
     // Two tile rows in flight a wave (measured: all 8 in flight is no faster; a call's time is its chain of dependent
@@ -72,7 +72,8 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
         if (threadIdx.x < kt) {
             const SlotRef sk = resolve_slot(a, s.row * kt + threadIdx.x);
             cinfo[threadIdx.x] = !sk.live ? 0xFFFFFFFFu : (sk.shared ? 0x80000000u | sk.e : sk.e);
-            cscore[threadIdx.x] = sk.shared ? 1.0f : (sk.live ? score_of(a, s.row, threadIdx.x) : 0.0f);
+            // GLM's profile has no scores: every slot's output is stored by itself
+            if constexpr (PROF == 0) cscore[threadIdx.x] = sk.shared ? 1.0f : (sk.live ? score_of(a, s.row, threadIdx.x) : 0.0f);
         }
     }
     const RoutedBank& bank = s.shared ? a.shared : a.bank;
@@ -106,7 +107,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
             stream.issue();
             uint32_t hh[2];
             float sum;
-            routed_mid_values<false, false, 0>(a, s, rk, tk0 >> 3, lane, hh, sum);
+            routed_mid_values<false, false, PROF>(a, s, rk, tk0 >> 3, lane, hh, sum);
             // element 64 j + lane of the block belongs to its tile row 4 j + lane / 16
 #pragma unroll
             for (uint32_t j = 0; j < 2u; ++j)
@@ -129,7 +130,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
             for (uint32_t b = 0; b < blocks; ++b) {
                 uint32_t hv[2];
                 float sum;
-                prep_values(a.dtype, a.x, suh, a.hidden, s.row, (tk0 >> 3) + b, lane, hv, sum);
+                prep_values(a.dtype, a.x, suh, a.hidden, s.row, (tk0 >> 3) + b, lane, hv, sum, PROF == 0);
 #pragma unroll
                 for (uint32_t j = 0; j < 2u; ++j) {
                     const uint32_t i = lane + 64u * j;
@@ -193,7 +194,33 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
         if (threadIdx.x == 0u)  // zero again for the next call
             __hip_atomic_store(a.arrive + counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if constexpr (NPROJ == 2) {
-            if (sg == 0u) routed_mid_block<false, true>(a, s, rk, b128, lane);
+            if (sg == 0u) routed_mid_block<false, true, PROF>(a, s, rk, b128, lane);
+        } else if constexpr (PROF == 1) {
+            // GLM's profile ends with each live slot's own finished output, f32 [row-slot][hidden]: four slots a wave,
+            // every load of the four in flight together, nothing to add up
+            for (uint32_t k0 = 0; k0 < kt; k0 += 16u) {
+                SlotRef sk[4];
+                uint32_t qk[4];
+                float v[4][2];
+#pragma unroll
+                for (uint32_t r = 0; r < 4u; ++r) {
+                    const uint32_t k = k0 + 4u * r + sg;
+                    const uint32_t info = k < kt ? cinfo[k] : 0xFFFFFFFFu;
+                    sk[r].row = s.row;
+                    sk[r].live = info != 0xFFFFFFFFu;
+                    sk[r].shared = false;
+                    sk[r].e = info & 0x7FFFFFFFu;
+                    qk[r] = s.row * kt + (k < kt ? k : 0u);
+                }
+                routed_down_finish_many<true, XLDS, 4, 1>(a, sk, qk, b128, lane, v, ks);
+#pragma unroll
+                for (uint32_t r = 0; r < 4u; ++r)
+                    if (sk[r].live) {
+                        float* o = static_cast<float*>(a.y) + static_cast<size_t>(qk[r]) * a.hidden + b128 * 128u + lane;
+                        o[0] = v[r][0];
+                        o[64] = v[r][1];
+                    }
+            }
         } else {
             // The slots' finishes sixteen at a time, four a wave (slot k0 + 4 r + wave) with every load of the four in
             // flight together; wave 0 adds them in slot order.
@@ -213,7 +240,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
                     sk[r].e = info & 0x7FFFFFFFu;
                     qk[r] = s.row * kt + (k < kt ? k : 0u);
                 }
-                routed_down_finish_many<true, XLDS, 4>(a, sk, qk, b128, lane, v, ks);
+                routed_down_finish_many<true, XLDS, 4, 0>(a, sk, qk, b128, lane, v, ks);
 #pragma unroll
                 for (uint32_t r = 0; r < 4u; ++r)
                     if (sk[r].live) {
@@ -240,13 +267,13 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
     }
 }
 
-template <int CB, int WIDE, int BT, int NPROJ, bool XLDS, bool ARRIVE>
+template <int CB, int WIDE, int BT, int NPROJ, bool XLDS, bool ARRIVE, int PROF>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ? 2 : 4))) moe_gemv(const MoeLaunch a) {
     __shared__ __attribute__((aligned(16))) unsigned char smem[role_lds_bytes<BT>()];
     __shared__ uint32_t last_flag, cinfo[64];
     __shared__ float cscore[64];
-    gemv_role<CB, WIDE, BT, NPROJ, XLDS, ARRIVE>(a, blockIdx.x, blockIdx.y, blockIdx.z, smem, last_flag, cinfo,
-                                                        cscore);
+    gemv_role<CB, WIDE, BT, NPROJ, XLDS, ARRIVE, PROF>(a, blockIdx.x, blockIdx.y, blockIdx.z, smem, last_flag, cinfo,
+                                                       cscore);
 }
 
 // Grid (inter / 128, RKT), 64 threads.
@@ -262,7 +289,7 @@ __global__ void __launch_bounds__(64) moe_combine(const MoeLaunch a) {
     else routed_slots_block<false>(a, blockIdx.y, blockIdx.x, threadIdx.x);
 }
 
-template <int CB, int WIDE, int NPROJ, bool XLDS, bool ARRIVE>
+template <int CB, int WIDE, int NPROJ, bool XLDS, bool ARRIVE, int PROF>
 hipError_t launch_gemv_bt(const MoeLaunch& a, hipStream_t s) {
     const uint32_t out = NPROJ == 2 ? a.inter : a.hidden;
     const uint32_t bt = NPROJ == 2 ? a.bt_gu : a.bt_dn, ks = NPROJ == 2 ? a.ks_gu : a.ks_dn;
@@ -271,24 +298,33 @@ hipError_t launch_gemv_bt(const MoeLaunch& a, hipStream_t s) {
     const size_t dyn = XLDS ? 4u * ((NPROJ == 2 ? a.per_gu : a.per_dn) + 1u) * (kXldsRows * 64u) : 0u;
     if constexpr (WIDE == kNarrow) {
         if (bt == 8u) {
-            hipLaunchKernelGGL((moe_gemv<CB, WIDE, 8, NPROJ, XLDS, ARRIVE>), grid, block, dyn, s, a);
+            hipLaunchKernelGGL((moe_gemv<CB, WIDE, 8, NPROJ, XLDS, ARRIVE, PROF>), grid, block, dyn, s, a);
             return hipGetLastError();
         }
     }
     if (bt != 4u) return hipErrorInvalidValue;  // a wide rate's eight tiles never fit a load
-    hipLaunchKernelGGL((moe_gemv<CB, WIDE, 4, NPROJ, XLDS, ARRIVE>), grid, block, dyn, s, a);
+    hipLaunchKernelGGL((moe_gemv<CB, WIDE, 4, NPROJ, XLDS, ARRIVE, PROF>), grid, block, dyn, s, a);
     return hipGetLastError();
 }
 
-template <int NPROJ, bool XLDS, bool ARRIVE>
+// PROF 1 (GLM's roundings in the stages a launch runs itself) exists for the served codebook forms only
+template <int NPROJ, bool XLDS, bool ARRIVE, int PROF = 0>
 hipError_t launch_gemv_cb(const MoeLaunch& a, hipStream_t s) {
     return with_reader(NPROJ == 2 ? a.n_gu : a.n_dn, [&](auto reader) {
         constexpr int R = decltype(reader)::value;
-        switch (a.codebook) {
-            case kMul1: return launch_gemv_bt<kMul1, R, NPROJ, XLDS, ARRIVE>(a, s);
-            case kMcg: return launch_gemv_bt<kMcg, R, NPROJ, XLDS, ARRIVE>(a, s);
-            case kMul1Defer: return launch_gemv_bt<kMul1Defer, R, NPROJ, XLDS, ARRIVE>(a, s);
-            default: return launch_gemv_bt<kMcgPair, R, NPROJ, XLDS, ARRIVE>(a, s);
+        if constexpr (PROF == 0) {
+            switch (a.codebook) {
+                case kMul1: return launch_gemv_bt<kMul1, R, NPROJ, XLDS, ARRIVE, 0>(a, s);
+                case kMcg: return launch_gemv_bt<kMcg, R, NPROJ, XLDS, ARRIVE, 0>(a, s);
+                case kMul1Defer: return launch_gemv_bt<kMul1Defer, R, NPROJ, XLDS, ARRIVE, 0>(a, s);
+                default: return launch_gemv_bt<kMcgPair, R, NPROJ, XLDS, ARRIVE, 0>(a, s);
+            }
+        } else {
+            switch (a.codebook) {
+                case kMul1Defer: return launch_gemv_bt<kMul1Defer, R, NPROJ, XLDS, ARRIVE, 1>(a, s);
+                case kMcgPair: return launch_gemv_bt<kMcgPair, R, NPROJ, XLDS, ARRIVE, 1>(a, s);
+                default: return hipErrorInvalidValue;
+            }
         }
     });
 }
@@ -298,19 +334,27 @@ hipError_t launch_gemv_cb(const MoeLaunch& a, hipStream_t s) {
 hipError_t launch_moe_decode(const MoeLaunch& a, int form, hipStream_t s) {
     const uint32_t rkt = a.rows * (a.topk + a.shared_slots);
     hipError_t e;
+    // Up to kMidInDownRows rows, every down wave runs the mid stage of its own 128-block first (the two launches hand
+    // over at their boundary; the stage is run once a column workgroup). More rows: the gate|up launch's last arriver
+    // at a block runs it once.
+    const bool mid_in_down = a.rows <= kMidInDownRows;
     if (form == kMoeTwoLaunches && !a.glm) {
-        // Up to kMidInDownRows rows, every down wave runs the mid stage of its own 128-block first (the two launches
-        // hand over at their boundary; the stage is run once a column workgroup). More rows: the gate|up launch's last
-        // arriver at a block runs it once.
-        const bool mid_in_down = a.rows <= kMidInDownRows;
         if (a.stages & 1u)
             if ((e = mid_in_down ? launch_gemv_cb<2, true, false>(a, s) : launch_gemv_cb<2, true, true>(a, s)) != hipSuccess)
                 return e;
         if (a.stages & 2u) return mid_in_down ? launch_gemv_cb<1, true, true>(a, s) : launch_gemv_cb<1, false, true>(a, s);
         return hipSuccess;
     }
+    if (form == kMoeTwoLaunches && (a.codebook == kMcgPair || a.codebook == kMul1Defer)) {
+        // GLM's profile in the same two launches (src/hip/plan.zig's form 9 under Profile.glm), its own roundings in the
+        // stages the launches run themselves
+        if ((e = mid_in_down ? launch_gemv_cb<2, true, false, 1>(a, s) : launch_gemv_cb<2, true, true, 1>(a, s)) != hipSuccess)
+            return e;
+        return mid_in_down ? launch_gemv_cb<1, true, true, 1>(a, s) : launch_gemv_cb<1, false, true, 1>(a, s);
+    }
     if (a.glm) {
-        // GLM's profile runs the five launches with its own roundings in the stages between the GEMVs
+        // GLM's profile on the five launches (the exact codebook forms, or a configured decode_form): its own roundings
+        // in the stages between the GEMVs
         hipLaunchKernelGGL(moe_prep<1>, dim3(a.hidden / 128u, rkt), dim3(64), 0, s, a);
         if ((e = hipGetLastError()) != hipSuccess) return e;
         if ((e = launch_gemv_cb<2, false, false>(a, s)) != hipSuccess) return e;

@@ -260,7 +260,7 @@ __device__ __forceinline__ bool routed_down_finish(const MoeLaunch& a, const Slo
 
 // R slots' finished down outputs of block b at once (a skipped slot's entry is left alone): all their planes, scales
 // and block sums are fetched together. q[r]: where slot r's scratch lives.
-template <bool COH, bool HS_COH, int R>
+template <bool COH, bool HS_COH, int R, int PROF = 0>
 __device__ __forceinline__ void routed_down_finish_many(const MoeLaunch& a, const SlotRef (&s)[R], const uint32_t (&q)[R],
                                                         uint32_t b, uint32_t lane, float (&v)[R][2], uint32_t ks) {
     const uint32_t rkt = a.rows * (a.topk + a.shared_slots), nbi = a.inter / 128u;
@@ -290,7 +290,8 @@ __device__ __forceinline__ void routed_down_finish_many(const MoeLaunch& a, cons
         if (a.defer)
 #pragma unroll
             for (uint32_t j = 0; j < 2u; ++j) v[r][j] = __builtin_fmaf(v[r][j], mul1_a(), mul1_b() * xsum[r]);
-        finish_core(v[r], sv[r], lane);
+        if constexpr (PROF == 0) finish_core(v[r], sv[r], lane);
+        else finish_core_glm(v[r], sv[r], lane, false);
     }
 }
 
