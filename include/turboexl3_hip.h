@@ -113,13 +113,18 @@ typedef struct t3_config {
     int32_t mcg_pair;      /* 1 (default): MCG's GEMV feeds the hashed pair to the matrix core unrounded; 0: the f16 weight */
     int32_t mul1_defer;    /* 1 (default): MUL1's affine map applied once an output (src/core/dense.zig deferFor); 0: per weight */
     int32_t dense_gemm_rows; /* dense calls of this many rows or more decode W_hat once into the workspace and run this
-                              * library's plain f16 GEMM, which ends with the finish. Default 512; 0: never */
+                              * library's plain f16 GEMM, which ends with the finish (where dense_gemm_fill allows).
+                              * Default 512; 0: never */
     int32_t dense_rows_alone; /* 0 (default): rows 17..32 run the GEMV and above 32 rows a dense call's launch shape follows
                                * its rows (K parts at few rows, the W_hat form at many), so a row's bytes can differ between
                                * calls of different row counts (each within the bars). 1: every call above 16 rows takes the
                                * trellis GEMM with one K part, and a row's bytes ignore the call's other rows, as the
                                * reference's own GEMM holds them for 17, 40, 129 and 200 rows (src/hip_tests.zig:866-880);
                                * few-row calls then run up to twice as long */
+    int32_t dense_gemm_fill;  /* 1 (default): the W_hat form serves only where its GEMM's grid fills the GPU: tiles =
+                               * ceil(rows / 256) * ceil(out / 256) (a 256 x 256 tile a workgroup, no K split) at least 120
+                               * and at least in / 56 (below that the trellis GEMM's K parts are faster, measured); 0: from
+                               * dense_gemm_rows rows whatever the shape */
 } t3_config;
 
 /* The served configuration. */
@@ -186,7 +191,8 @@ enum {
     T3_DENSE_ARRIVE = 1,       /* prepare launch, then the GEMV whose last workgroup a block runs the finish */
     T3_DENSE_CHAIN = 2,        /* prepare, GEMV, finish */
     T3_DENSE_TRELLIS_GEMM = 3, /* above 32 rows: prepare, the GEMM that decodes in registers, finish */
-    T3_DENSE_W_HAT_GEMM = 4    /* from dense_gemm_rows rows: W_hat decode, prepare, plain f16 GEMM, finish */
+    T3_DENSE_W_HAT_GEMM = 4    /* from dense_gemm_rows rows, where the GEMM's grid fills the GPU (dense_gemm_fill): W_hat
+                                * decode, prepare, plain f16 GEMM, finish */
 };
 typedef struct t3_linear_plan {
     int32_t path;            /* T3_DENSE_* */

@@ -55,7 +55,7 @@ def test_configure_refuses_unserved_values(lib):
     cfg = Config()
     lib.t3_config_default(C.byref(cfg))
     assert (cfg.decode_form, cfg.dec_one, cfg.prefill, cfg.mcg_pair, cfg.mul1_defer, cfg.dense_gemm_rows,
-            cfg.dense_rows_alone) == (9, 1, 1, 1, 1, 512, 0)
+            cfg.dense_rows_alone, cfg.dense_gemm_fill) == (9, 1, 1, 1, 1, 512, 0, 1)
     cfg.decode_form = 5
     assert lib.t3_error_name(lib.t3_configure(C.byref(cfg))).decode() == "InvalidTurboexl3Config"
     cfg.decode_form, cfg.dense_gemm_rows = 9, -1

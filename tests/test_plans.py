@@ -91,17 +91,23 @@ def test_few_rows_share_the_tile_rows_out(lib):
     p = linear_plan(lib, 64, 4096, 14336, 64, BF16)
     assert (p.path, p.launches, p.k_slices) == (3, 3, 16)
     assert p.workgroups == 56 * 16
-    q = linear_plan(lib, 300, 4096, 14336, 64, BF16)   # three items
-    assert (q.path, q.k_slices) == (3, 4)
+    q = linear_plan(lib, 300, 4096, 14336, 64, BF16)   # three items: 168 workgroups a part, two parts fit the 512 resident
+    assert (q.path, q.k_slices) == (3, 2)
     # from dense_gemm_rows (512) rows the W_hat form serves: decode once, prepare, the f16 GEMM that ends with the finish
     w = linear_plan(lib, 600, 4096, 14336, 64, BF16)
     assert (w.path, w.launches, w.k_slices) == (4, 3, 1)
+    # ... where its GEMM's 256 x 256 tiles fill the GPU (at least 120 of them, and in / 64): 512 rows of this shape are
+    # 2 x 56 = 112 tiles and stay on the trellis GEMM; a narrow out needs many rows; a long K more tiles (in / 56)
+    assert linear_plan(lib, 512, 4096, 14336, 64, BF16).path == 3
+    assert [linear_plan(lib, r, 7168, 2048, 48, BF16).path for r in (1024, 2048, 4096)] == [3, 3, 4]
+    assert [linear_plan(lib, r, 4096, 4096, 64, BF16).path for r in (1024, 1536, 2048)] == [3, 3, 4]
+    assert [linear_plan(lib, r, 14336, 4096, 64, BF16).path for r in (2048, 4096)] == [3, 4]
     cfg = Config()
     lib.t3_config_default(C.byref(cfg))
     cfg.dense_gemm_rows = 0
     assert lib.t3_configure(C.byref(cfg)) == 0
     try:
-        assert linear_plan(lib, 600, 4096, 14336, 64, BF16).k_slices == 2   # kept on the trellis GEMM: five items
+        assert linear_plan(lib, 600, 4096, 14336, 64, BF16).k_slices == 1   # kept on the trellis GEMM: five items, 280 workgroups
     finally:
         lib.t3_config_default(C.byref(cfg))
         assert lib.t3_configure(C.byref(cfg)) == 0

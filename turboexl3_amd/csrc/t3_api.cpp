@@ -61,7 +61,7 @@ const char* t3_error_name(int32_t status) {
 
 void t3_config_default(t3_config* out) {
     if (!out) return;
-    const t3_config d = {9, 1, 1, 1, 1, 512, 0};
+    const t3_config d = {9, 1, 1, 1, 1, 512, 0, 1};
     *out = d;
 }
 
@@ -69,7 +69,8 @@ int32_t t3_configure(const t3_config* cfg) {
     if (!cfg) return T3_BadArgs;
     const bool flags_ok = (cfg->dec_one == 0 || cfg->dec_one == 1) && (cfg->prefill == 0 || cfg->prefill == 1) &&
                           (cfg->mcg_pair == 0 || cfg->mcg_pair == 1) && (cfg->mul1_defer == 0 || cfg->mul1_defer == 1) &&
-                          cfg->dense_gemm_rows >= 0 && (cfg->dense_rows_alone == 0 || cfg->dense_rows_alone == 1);
+                          cfg->dense_gemm_rows >= 0 && (cfg->dense_rows_alone == 0 || cfg->dense_rows_alone == 1) &&
+                          (cfg->dense_gemm_fill == 0 || cfg->dense_gemm_fill == 1);
     if ((cfg->decode_form != 3 && cfg->decode_form != 4 && cfg->decode_form != 9) || !flags_ok) return T3_InvalidTurboexl3Config;
     std::lock_guard<std::mutex> lock(g_config_write);
     const uint32_t next = g_config_at.load(std::memory_order_relaxed) + 1u;

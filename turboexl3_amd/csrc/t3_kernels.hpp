@@ -128,12 +128,19 @@ hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s);
 hipError_t launch_dense_prefill(const DenseLaunch& d, hipStream_t s);
 // Its K parts (d.ks; z then holds that many planes, summed in part order by the finish): a call of few rows decodes the
 // matrix once, and a workgroup per 256 columns alone would leave most of the GPU idle, so the tile rows are shared out
-// until the launch has two workgroups a compute unit. Each part keeps an even number of K = 32 steps, at least eight.
+// while the launch stays within the workgroups the GPU holds at once. Each part keeps an even number of K = 32 steps, at
+// least eight. Measured against the rule that grew the parts until the launch had at least 512 workgroups (us): 4096 x 4096
+// at 300 / 640 / 1536 rows 59 / 78 / 113 -> 44 / 63 / 100, 2048 x 7168 at 512 / 1024 rows 64 / 82 -> 48 / 66, 4096 x 14336 at
+// 128 / 256 / 512 rows 62 / 80 / 115 -> 45 / 61 / 100, 8192 x 8192 at 300 rows 107 -> 94.
 inline uint32_t dense_prefill_kparts(uint32_t rows, uint32_t in, uint32_t out) {
     const uint32_t item_rows = rows <= 64u ? 64u : 128u, items = (rows + item_rows - 1u) / item_rows;
     const uint32_t nblk = (out + 255u) / 256u, steps = in / 32u;
+    // the most parts that still fit one round of the workgroups the GPU holds at once (two a compute unit with a 128-row
+    // item's accumulators, four with a 64-row item's): a launch that spills into a second round takes that round's whole
+    // time for its few workgroups
+    const uint32_t slots = item_rows == 64u ? 1024u : 512u;
     uint32_t k = 1;
-    while (items * nblk * k < 512u && k < 16u && steps % (4u * k) == 0u && steps / (2u * k) >= 8u) k *= 2u;
+    while (k < 16u && steps % (4u * k) == 0u && steps / (2u * k) >= 8u && items * nblk * 2u * k <= slots) k *= 2u;
     return k;
 }
 

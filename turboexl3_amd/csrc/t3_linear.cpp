@@ -101,10 +101,22 @@ constexpr uint32_t kGemvRowsMax = 32;
 uint32_t gemv_rows_max() { return config().dense_rows_alone ? 16u : kGemvRowsMax; }
 
 // From dense_gemm_rows rows up a dense call decodes W_hat once and multiplies plainly (src/core/dense.zig:909-922,
-// 1290-1302): the decode is paid once a call, not once a 64-row item.
+// 1290-1302): the decode is paid once a call, not once a 128-row item. The plain GEMM takes a 256 x 256 tile a workgroup
+// over the whole K, so it only pays where its grid fills the GPU: with few tiles (a narrow out, or rows in the hundreds)
+// a handful of workgroups walk K while the trellis GEMM shares the tile rows out into K parts. Measured (trellis GEMM
+// against W_hat form, us): 7168 x 2048 at 1024 / 4096 rows 66 / 156 and 173 / 170, 14336 x 4096 at 512 / 2048 / 4096 rows
+// 97 / 290, 297 / 322 and 570 / 459, 4096 x 4096 at 1024 / 2048 / 4096 rows 67 / 104, 105 / 106 and 182 / 140, 8192 x 8192 at
+// 1024 / 1536 rows 177 / 194 and 320 / 226, 5120 x 5120 at 1024 / 1536 rows 105 / 126 and 161 / 127, 4096 x 14336 at 512 / 640 /
+// 2048 rows 111 / 116, 170 / 123 and 316 / 244, 2048 x 7168 at 1024 rows 80 / 70. Across ten shapes and eight row counts
+// from 256 to 4096 the W_hat form wins from about 120 tiles (half the compute units), a long K asking for more (tiles x 56
+// >= in: 8192 x 8192 at 1024 rows, 128 tiles, 172 / 195); the rule below is within 10 % of the better form in every cell
+// measured.
 bool takes_w_hat(const DenseLaunch& l) {
     const int32_t from = config().dense_gemm_rows;
-    return !config().dense_rows_alone && from > 0 && l.rows >= static_cast<uint32_t>(from) && gemm_half_ok(l.in, l.out);
+    if (config().dense_rows_alone || from <= 0 || l.rows < static_cast<uint32_t>(from) || !gemm_half_ok(l.in, l.out))
+        return false;
+    const uint64_t tiles = static_cast<uint64_t>((l.rows + 255u) / 256u) * ((l.out + 255u) / 256u);
+    return !config().dense_gemm_fill || (tiles >= 120u && tiles * 56u >= l.in);
 }
 
 struct WhatScratch {
