@@ -100,6 +100,21 @@ inline uint32_t gemv_slices(uint32_t in_tiles, uint32_t groups) {
     return 1;
 }
 
+// A dense GEMV's tiles a load and K slices. A small matrix cannot reach the target workgroup count at eight tiles a load
+// (2560 x 640: 25 workgroups), and each of its few waves then walks its 64 tiles alone on a SIMD: with up to 128 workgroups
+// the same rows are cut at four tiles a load, twice the workgroups of half the length. Measured (one row, us a call, eight
+// against four tiles): 2560 x 640 8.2 / 7.1, 1024 x 4096 8.1 / 7.1, 2048 x 512 8.2 / 7.1, 2048 x 2048 8.4 / 8.0 (32 rows
+// 11.2 / 9.9), 2048 x 4096 8.8 / 8.3; from about 144 workgroups up four tiles lose (4096 x 4096 9.6 / 10.0, 5120 x 5120
+// 11.5 / 12.9). A column's sums do not depend on the tiles a load; the shape alone decides, so a row's bytes stay its own.
+inline void dense_gemv_partition(uint32_t n, uint32_t in, uint32_t out, uint32_t* bt, uint32_t* ks) {
+    *bt = gemv_bt(n);
+    *ks = gemv_slices(in / 16u, (out / 16u) / *bt);
+    if (*bt == 8u && (out / 128u) * *ks <= 128u) {
+        *bt = 4u;
+        *ks = gemv_slices(in / 16u, (out / 16u) / 4u);
+    }
+}
+
 // The caller's workspace starts with the arrival counters of the fused launches, at a fixed place and size whatever
 // the call's shapes: zero when the workspace is first passed, and zero again after every call.
 constexpr size_t kCounterBytes = 65536;

@@ -64,8 +64,7 @@ int32_t check_dense(const t3_array* x, const t3_array* trellis, const t3_array* 
     l.wbits = d.wbits;
     l.codebook = d.gemv_form;
     l.dtype = x->dtype;
-    l.bt = gemv_bt(l.n);
-    l.ks = gemv_slices(l.in / 16u, (l.out / 16u) / l.bt);
+    dense_gemv_partition(l.n, l.in, l.out, &l.bt, &l.ks);
     return T3_OK;
 }
 
