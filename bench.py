@@ -19,7 +19,8 @@ stage timed alone, and the same call over MUL1's codebook; TFLOP/s against the 2
 dense f16 GEMM measured in this process, `measured_dense_f16_peak`), `dense_prefill` (config 5's 4096 rows and its
 resident-weight forms),
 `codebook_forms` (the price of exact f16 weights in the GEMV), `rates` (a fractional narrow rate and a wide one) and
-`dense_rows` (few-row dense calls with and without the rows-alone partition). `cpu_baseline`: the CPU oracle
+`dense_rows` (few-row dense calls with and without the rows-alone partition), `shapes` (shapes beside the metric's own:
+what the rules that pick a path from the shape serve, beside the other path). `cpu_baseline`: the CPU oracle
 (`format.project` restated in C) timed on this box's host cores, and, in the same leg, one sampled output block (or row)
 of every timed cell held against the oracle by the reference's bars (`parity_checks`).
 """
@@ -289,6 +290,84 @@ def eager_time(torch, fn, reps: int = 5) -> float:
     return e0.elapsed_time(e1) * 1e-3 / reps
 
 
+def shapes_section(torch, api) -> dict:
+    """Shapes beside the metric's own, one cell each for a rule that picks a path from the shape: what the served call
+    takes and what the other path would (the same bytes either way, or the same bars)."""
+    out = {}
+    # a small matrix: four tiles a load while eight would leave at most 128 workgroups
+    cells = []
+    for in_f, out_f, n, rows in ((2560, 640, 64, 1), (2048, 2048, 64, 1), (2048, 2048, 64, 32)):
+        d = Dense(torch, api, in_f, out_f, n, MCG_CB, 32, torch.float16, seed=77)
+        d.bind(rows)
+        cells.append({"in": in_f, "out": out_f, "n": n, "rows": rows, "us_per_call": d.time(96, 8) * 1e6,
+                      "plan": {k: d.plan[k] for k in ("launches", "tiles_a_load", "k_slices", "workgroups")}})
+        del d
+    out["dense_small"] = cells
+    # above 32 rows: the trellis GEMM (K parts within one round of resident workgroups) or the W_hat form (where its
+    # GEMM's tiles fill the GPU)
+    cells = []
+    for in_f, out_f, n, rows in ((7168, 2048, 48, 1024), (4096, 4096, 64, 640), (4096, 14336, 64, 640), (8192, 8192, 64, 1536)):
+        d = Dense(torch, api, in_f, out_f, n, MCG_CB, rows, torch.bfloat16, seed=78, copies=2, outliers=False)
+        took = {}
+        for name, cfg in (("served", {}), ("trellis_gemm", {"dense_gemm_rows": 0}),
+                          ("w_hat_form", {"dense_gemm_rows": 1, "dense_gemm_fill": 0})):
+            api.configure(**cfg)
+            try:
+                d.bind(rows)
+                took[name + "_us"] = d.time(8, 2) * 1e6
+                if name == "served":
+                    took["served_plan"] = {k: d.plan[k] for k in ("path", "k_slices", "workgroups")}
+            finally:
+                api.configure()
+        cells.append({"in": in_f, "out": out_f, "n": n, "rows": rows, **took})
+        del d
+    out["dense_above_32_rows"] = cells
+    # routed decode over large experts: two launches up to 8192 gate|up workgroups, five past it; GLM's profile
+    cells = []
+    m = None
+    for tokens in (1, 4, 8, 16):
+        m = Moe(torch, api, 64, 4096, 2048, 4, 4, 8, tokens, 7, shared=False, sets=8, seed=79)
+        took = {}
+        for name, form in (("served", 9), ("five_launches", 3)):
+            api.configure(decode_form=form)
+            try:
+                took[name + "_us"] = m.time(48, 6) * 1e6
+            finally:
+                api.configure()
+        cells.append({"experts": 64, "hidden": 4096, "inter": 2048, "k": 4, "topk": 8, "tokens": tokens, **took,
+                      "served_launches": m.plan["launches"]})
+        if tokens != 1:
+            del m
+            m = None
+        else:
+            # GLM's profile over the same bank at one token (the last slot of the row is the host's shared expert)
+            y = torch.zeros(1, 1, m.topk, m.hidden, dtype=torch.float32, device="cuda")
+            ay = api._arr(y)
+            inds = [torch.cat([m.inds[j, :, :m.topk - 1], torch.full((1, 1), m.E, dtype=torch.int32, device="cuda")], dim=1)
+                    .reshape(1, 1, m.topk).contiguous() for j in range(m.sets)]
+            ai = [api._arr(t) for t in inds]
+
+            def glm_call(i, stream, m=m, ai=ai, ay=ay):
+                st = m.L.t3_moe_glm(stream, C.byref(m.ax), C.byref(m.cb), C.byref(ai[i % m.sets]), m.dec.c(), 7, C.byref(ay),
+                                    m.ws.data_ptr(), m.ws.numel())
+                if st != 0:
+                    raise RuntimeError(m.L.t3_error_name(st).decode())
+
+            glm = {}
+            for name, form in (("two_launches", 9), ("five_launches", 3)):
+                api.configure(decode_form=form)
+                try:
+                    glm[name + "_us"] = graph_time(torch, glm_call, 48, 6, 3) * 1e6
+                finally:
+                    api.configure()
+            out["moe_glm_one_token"] = {"experts": 64, "hidden": 4096, "inter": 2048, "k": 4, "topk": 7, **glm}
+            del m, y, inds, ai
+            m = None
+    out["moe_decode_large_experts"] = cells
+    torch.cuda.empty_cache()
+    return out
+
+
 def cpu_leg(n: int, seed: int, todo: list, budget_s: float = 20.0):
     """The only place this program touches the CPU oracle. (1) format.project (the C restatement) timed on the host: the
     headline workload's shape and seeded distributions, one row, one thread, re-decoding every tile as the reference does;
@@ -344,7 +423,7 @@ def main() -> int:
     ap.add_argument("--rows", type=int, default=1)
     ap.add_argument("--quick", action="store_true", help="the headline workload only")
     ap.add_argument("--only", default="", help="comma-separated sections to run beside the headline: sweep, forms, rates, "
-                                               "lm_head, moe_decode, moe_prefill, dense_prefill, dense_rows, peak")
+                                               "lm_head, moe_decode, moe_prefill, dense_prefill, dense_rows, peak, shapes")
     ap.add_argument("--sweep", action="store_true", help="(default on) K = 3, 4, 5 x rows = 1, 4, 16, 32")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run one 256 MiB device copy, the known-size kernel that scales the profiler's "
@@ -358,7 +437,7 @@ def main() -> int:
         print(f"bench.py: this build measures one GPU (the path has no collective); --gpus {args.gpus} is not served",
               file=sys.stderr)
         return 2
-    sections = {"sweep", "forms", "rates", "lm_head", "moe_decode", "moe_prefill", "dense_prefill", "dense_rows", "peak"}
+    sections = {"sweep", "forms", "rates", "lm_head", "moe_decode", "moe_prefill", "dense_prefill", "dense_rows", "peak", "shapes"}
     if args.quick:
         sections = set()
     elif args.only:
@@ -579,6 +658,9 @@ def main() -> int:
                                                           if k in ("path", "k_slices", "workgroups")}})
         del dp
         torch.cuda.empty_cache()
+
+    if "shapes" in sections:
+        out["shapes"] = shapes_section(torch, api)
 
     if not args.no_cpu:
         out["cpu_baseline"], checks = cpu_leg(n_head, seed=11, todo=todo)
