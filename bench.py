@@ -322,7 +322,8 @@ def shapes_section(torch, api) -> dict:
         cells.append({"in": in_f, "out": out_f, "n": n, "rows": rows, **took})
         del d
     out["dense_above_32_rows"] = cells
-    # routed decode over large experts: two launches up to 8192 gate|up workgroups, five past it; GLM's profile
+    # routed decode over large experts: two launches up to 8192 gate|up workgroups; past it the five launches behind a
+    # grouping launch (the row-slots of one expert served together); GLM's profile
     cells = []
     m = None
     for tokens in (1, 4, 8, 16):
@@ -335,7 +336,7 @@ def shapes_section(torch, api) -> dict:
             finally:
                 api.configure()
         cells.append({"experts": 64, "hidden": 4096, "inter": 2048, "k": 4, "topk": 8, "tokens": tokens, **took,
-                      "served_launches": m.plan["launches"]})
+                      "served_launches": m.plan["launches"], "distinct_experts": m.distinct})
         if tokens != 1:
             del m
             m = None
@@ -363,6 +364,19 @@ def shapes_section(torch, api) -> dict:
             out["moe_glm_one_token"] = {"experts": 64, "hidden": 4096, "inter": 2048, "k": 4, "topk": 7, **glm}
             del m, y, inds, ai
             m = None
+    # few experts, each very large (eight of 4096 x 14336, top-2): most row-slots of a call share their expert
+    for tokens in (4, 16):
+        m = Moe(torch, api, 8, 4096, 14336, 4, 4, 2, tokens, 0, shared=False, sets=8, seed=80)
+        took = {}
+        for name, form in (("served", 9), ("five_launches", 3)):
+            api.configure(decode_form=form)
+            try:
+                took[name + "_us"] = m.time(24, 4) * 1e6
+            finally:
+                api.configure()
+        cells.append({"experts": 8, "hidden": 4096, "inter": 14336, "k": 4, "topk": 2, "tokens": tokens, **took,
+                      "served_launches": m.plan["launches"], "distinct_experts": m.distinct})
+        del m
     out["moe_decode_large_experts"] = cells
     torch.cuda.empty_cache()
     return out

@@ -104,10 +104,12 @@ typedef struct t3_bank {
 /* ---- configuration (src/core/config.zig; only the fields this path reads) --------------------------------- */
 
 typedef struct t3_config {
-    int32_t decode_form;   /* 3: the five-launch chain; 4: four launches (prepare inside gate|up); 9 (default): two
+    int32_t decode_form;   /* 3: the five-launch chain; 4: four launches (prepare inside gate|up); 6 (this library's own):
+                            * the grouped six launches whatever the size; 9 (default): two
                             * launches (mid and combine run by the last workgroup to arrive) while the gate|up launch
-                            * stays within 8192 workgroups, the five launches past that (large experts at many rows,
-                            * where they are faster); the same bytes whichever runs; others refused */
+                            * stays within 8192 workgroups; past that (large experts at several rows, where the decode
+                            * dominates) six: the five behind a grouping launch that serves the row-slots of one expert
+                            * together; the same bytes whichever runs; others refused */
     int32_t dec_one;       /* 1 (default): dense decode rows in one launch; 0: the three-launch chain */
     int32_t prefill;       /* 1 (default); 0: routed calls above 16 rows refuse Exl3EngineNotImplemented */
     int32_t mcg_pair;      /* 1 (default): MCG's GEMV feeds the hashed pair to the matrix core unrounded; 0: the f16 weight */
@@ -242,8 +244,8 @@ int32_t t3_linear_unrot(t3_stream stream, const t3_array* x, const t3_array* w_s
 
 /* x [B, S, D]; inds (U32/I32) and scores (F32/BF16/F16) [B, S, K], K <= 32; y [B, S, D] in x's dtype.
  * `verify_rows` is accepted and ignored, as in the reference (src/root.zig:822-825). Up to 16 rows: the split-K GEMV
- * chain, two launches (five for large experts at many rows; four or five under decode_form 4 or 3; the same bytes, and
- * t3_moe_plan_of says which). A routed id outside [0, E) is skipped. Gate and up
+ * chain, two launches (six for large experts at several rows; four or five under decode_form 4 or 3; the same bytes,
+ * and t3_moe_plan_of says which). A routed id outside [0, E) is skipped. Gate and up
  * must share a rate (T3_Exl3GateUpRateMismatch); the down's rate may differ (the reference refuses that,
  * src/root.zig:841; this library's kernels take a rate a launch). */
 int32_t t3_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
@@ -327,6 +329,8 @@ enum {
     T3_MOE_TWO_LAUNCHES = 0,   /* gate|up + mid, down + combine */
     T3_MOE_FOUR_LAUNCHES = 1,  /* gate|up (prepare inside), mid, down, combine */
     T3_MOE_FIVE_LAUNCHES = 2,  /* prepare, gate|up, mid, down, combine */
+    T3_MOE_GROUPED = 4,        /* group, prepare, gate|up, mid, down, combine: the row-slots that read one expert served
+                                * together (large experts at two rows or more), the same bytes */
     T3_MOE_PREFILL = 3         /* above 16 rows: route (clear, histogram, scan, place), prepare, gate|up GEMM, mid, down
                                 * GEMM, combine */
 };

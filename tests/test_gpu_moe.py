@@ -140,7 +140,7 @@ def test_launch_forms_give_the_same_bytes(oracle, t3):
             nine = call()
             again = call()
             assert bytes_of(nine) == bytes_of(again)
-            for form in (3, 4):
+            for form in (3, 4, 6):
                 t3.configure(decode_form=form)
                 try:
                     other = call()
@@ -166,7 +166,7 @@ def test_launch_forms_give_the_same_bytes_at_the_reference_rows(oracle, t3):
         args = (x_dev[:rows].reshape(1, rows, hidden), dbank, torch.from_numpy(slots[:rows]).cuda().reshape(1, rows, topk),
                 torch.from_numpy(scores[:rows]).cuda().reshape(1, rows, topk), dec)
         nine = t3.moe(*args)
-        for form in (3, 4):
+        for form in (3, 4, 6):
             t3.configure(decode_form=form)
             try:
                 other = t3.moe(*args)
@@ -373,7 +373,7 @@ def test_fused_gated_shared_expert(oracle, t3, codebook, n, dtype):
     # `moe` has one, and a step of bf16 at 4 rms is 3e-2 of rms: the dense bar (src/hip_tests.zig:326), not the routed
     # one. f16: two steps of f16 at 4 rms (8e-3 of rms) on top of the f32 bar's share
     bar = 2.5e-2 if dtype == torch.bfloat16 else 1e-2
-    for form in (9, 4, 3):
+    for form in (9, 4, 3, 6):
         t3.configure(decode_form=form)
         try:
             for count in (1, 3, 4):
@@ -519,6 +519,59 @@ def test_fused_gated_shared_expert_with_the_gate_vector(oracle, t3, hidden, rows
         assert err.value.name == name, (kwargs.keys(), name)
 
 
+def test_grouped_form_serves_an_experts_row_slots_together(oracle, t3):
+    """The six-launch form (the row-slots that read one expert served by one set of workgroups, up to sixteen a group):
+    the bytes of the five launches, where every row reads the same experts (full groups), where a row names an expert
+    twice (more than sixteen readers: a second group), with skipped ids and a shared expert (one group of every row), at
+    four tiles a load as well; and where the default configuration picks it by itself (large experts, several rows)."""
+    rng = np.random.default_rng(0x6E0)
+    hidden, inter = 512, 256
+    for experts, topk, n, rows, how in ((2, 2, 64, 16, "same"), (3, 2, 48, 16, "twice"), (12, 4, 80, 9, "mixed"),
+                                        (5, 3, 96, 2, "mixed")):
+        bank = oracle.synth_bank(rng, experts, hidden, inter, n)
+        shared = oracle.synth_bank(rng, 1, hidden, inter, n)
+        dbank, dshared = dev_bank(t3, bank), dev_bank(t3, shared)
+        x_dev, _ = make_x(rng, rows, hidden, torch.bfloat16)
+        slots, scores = routing(rng, rows, topk, experts)
+        if how == "same":
+            slots[:] = np.arange(topk, dtype=np.int32)[None, :]
+        elif how == "twice":
+            slots[:] = 1                                   # expert 1 read 32 times: two groups of sixteen
+        else:
+            slots[0, 1] = -1
+            slots[rows - 1, 0] = experts + 3
+        args = (x_dev.reshape(1, rows, hidden), dbank, torch.from_numpy(slots).cuda().reshape(1, rows, topk),
+                torch.from_numpy(scores).cuda().reshape(1, rows, topk), t3.Decode(MUL1 if n == 48 else MCG, 16))
+        for call in (lambda: t3.moe_clamped(*args, 7), lambda: t3.moe_shared_expert(*args, 1, dshared)):
+            t3.configure(decode_form=3)
+            try:
+                five = call()
+            finally:
+                t3.configure()
+            t3.configure(decode_form=6)
+            try:
+                six, again = call(), call()
+            finally:
+                t3.configure()
+            assert bytes_of(six) == bytes_of(five), f"{how} E {experts} top-{topk} n {n} rows {rows}: grouped differs"
+            assert bytes_of(six) == bytes_of(again)
+    # the default's own choice: 4096 x 2048, sixteen rows over few experts
+    hidden, inter, experts, topk = 4096, 2048, 4, 3
+    bank = dev_bank(t3, oracle.synth_bank(rng, experts, hidden, inter, 64))
+    x_dev, _ = make_x(rng, 16, hidden, torch.bfloat16)
+    slots, scores = routing(rng, 16, topk, experts)
+    args = (x_dev.reshape(1, 16, hidden), bank, torch.from_numpy(slots).cuda().reshape(1, 16, topk),
+            torch.from_numpy(scores).cuda().reshape(1, 16, topk), t3.Decode.mcg)
+    assert t3.moe_plan(args[0], bank, args[2])["launches"] == 6
+    served = t3.moe(*args)
+    t3.configure(decode_form=3)
+    try:
+        five = t3.moe(*args)
+    finally:
+        t3.configure()
+    assert bytes_of(served) == bytes_of(five)
+
+
 def test_glm_profile_launch_forms_give_the_same_bytes(oracle, t3):
     # src/hip_tests.zig:896,900-913: form 9's bytes are form 3's under GLM's profile too (4096 x 2048, 9 experts, K4, MCG,
     # bf16, the last slot of a row the host's shared expert), rows 1-5, 8 and 16; and with MUL1's deferred map
@@ -536,12 +589,13 @@ def test_glm_profile_launch_forms_give_the_same_bytes(oracle, t3):
             two = t3.moe_glm(*args, fill=float("nan"))
             again = t3.moe_glm(*args, fill=float("nan"))
             assert bytes_of(two) == bytes_of(again)
-            t3.configure(decode_form=3)
-            try:
-                five = t3.moe_glm(*args, fill=float("nan"))
-            finally:
-                t3.configure()
-            assert bytes_of(two) == bytes_of(five), f"hidden {hidden} rows {rows}: two launches differ from five"
+            for form in (3, 6):
+                t3.configure(decode_form=form)
+                try:
+                    five = t3.moe_glm(*args, fill=float("nan"))
+                finally:
+                    t3.configure()
+                assert bytes_of(two) == bytes_of(five), f"hidden {hidden} rows {rows}: the served form differs from form {form}"
             assert torch.isnan(two.reshape(rows, k, hidden)[:, topk]).all(), "the slot past the experts was written"
 
 

@@ -139,7 +139,7 @@ def test_config4_prefill_items(lib):
 
 def test_decode_forms_by_configuration(lib):
     cfg = Config()
-    for form, path, launches in ((3, 2, 5), (4, 1, 4), (9, 0, 2)):
+    for form, path, launches in ((3, 2, 5), (4, 1, 4), (6, 4, 6), (9, 0, 2)):
         lib.t3_config_default(C.byref(cfg))
         cfg.decode_form = form
         assert lib.t3_configure(C.byref(cfg)) == 0
@@ -154,12 +154,15 @@ def test_decode_forms_by_configuration(lib):
 def test_decode_form_by_the_gate_up_launch_size(lib):
     # two launches while the gate|up launch stays within 8192 workgroups (column groups x row-slots x 2 x K slices), five
     # past that: 4096 x 2048 K4 top-8 has 16 x 8 r x 2 x 8 = 2048 r of them
-    for rows, launches in ((1, 2), (4, 2), (5, 5), (16, 5)):
+    # (past it: the five launches behind a grouping launch, six in all)
+    for rows, launches in ((1, 2), (4, 2), (5, 6), (16, 6)):
         assert moe_plan(lib, rows, 64, 4096, 2048, 8, 64, 64).launches == launches
     # 7168 x 2048 K3 top-8: 16 x 8 r x 2 x 14 = 3584 r
-    assert [moe_plan(lib, rows, 256, 7168, 2048, 8, 48, 48).launches for rows in (1, 2, 3)] == [2, 2, 5]
+    assert [moe_plan(lib, rows, 256, 7168, 2048, 8, 48, 48).launches for rows in (1, 2, 3)] == [2, 2, 6]
     # four tiles a load (K5) doubles the column groups: 4096 x 1024 has 16 x 8 r x 2 x 8 = 2048 r as well
-    assert [moe_plan(lib, rows, 64, 4096, 1024, 8, 80, 80).launches for rows in (4, 5)] == [2, 5]
+    assert [moe_plan(lib, rows, 64, 4096, 1024, 8, 80, 80).launches for rows in (4, 5)] == [2, 6]
+    # one row of a top-k wide enough to pass the bound has nothing to group: the five launches
+    assert moe_plan(lib, 1, 64, 8192, 4096, 32, 64, 64).launches == 5
 
 
 def test_plan_refusals(lib):

@@ -64,6 +64,9 @@ struct MoeLaunch {
     int glm = 0;
     void* y = nullptr;
     uint32_t* arrive = nullptr;  // the two-launch form's arrival counters
+    // the grouped form's table: [0] the number of groups; then {key, members} a group (key: the expert, bit 31 for a
+    // shared slot); then 16 member row-slots a group. RKT groups at most.
+    uint32_t* groups = nullptr;
     uint32_t* xg = nullptr;      // u32 [RKT][hidden]
     uint32_t* xu = nullptr;
     uint32_t* hd = nullptr;      // u32 [RKT][inter]
@@ -97,7 +100,10 @@ struct MoeLaunch {
 
 // Five launches (prepare, gate|up, mid, down, combine); four (each gate|up wave prepares its own 128-block in LDS);
 // or two (gate|up + mid, down + combine: the last workgroup to arrive at a block runs the next stage). The same bytes.
-enum MoeForm : int { kMoeFiveLaunches = 0, kMoeFourLaunches = 1, kMoeTwoLaunches = 2 };
+// Or six: the five behind a grouping launch, the row-slots that read one expert served together (up to 16 a group), so
+// the expert's tiles are decoded once for all of them. The same bytes again: an output column of the matrix core depends
+// on its own activation row alone.
+enum MoeForm : int { kMoeFiveLaunches = 0, kMoeFourLaunches = 1, kMoeTwoLaunches = 2, kMoeGrouped = 3 };
 hipError_t launch_moe_decode(const MoeLaunch& a, int form, hipStream_t s);
 // a row's top-k experts by logit (ties to the lowest id) and their renormalised softmax weights in the logits' dtype
 hipError_t launch_route_softmax(const void* logits, int32_t* inds, void* scores, uint32_t rows, uint32_t experts, uint32_t k,

@@ -151,6 +151,7 @@ void carve_moe(MoeCall* call, void* workspace) {
     l.zg = c.take<float>(static_cast<size_t>(l.ks_gu) * rkt * l.inter * 4u);
     l.zu = c.take<float>(static_cast<size_t>(l.ks_gu) * rkt * l.inter * 4u);
     l.zd = c.take<float>(static_cast<size_t>(l.ks_dn) * rkt * l.hidden * 4u);
+    l.groups = c.take<uint32_t>((1u + 2u * rkt + 16u * rkt) * 4u);  // the grouped form's table
     call->workspace = c.used;
 }
 
@@ -211,9 +212,13 @@ int decode_form_of(const MoeLaunch& l) {
     const size_t widest = (l.hidden > l.inter ? l.hidden : l.inter) / 128u;
     const size_t counters = rkt * widest;
     if (config().decode_form == 3) return kMoeFiveLaunches;
+    if (config().decode_form == 6) return kMoeGrouped;
     if (config().decode_form == 4 || counters * 4u > kCounterBytes) return kMoeFourLaunches;
     const uint64_t gu_groups = static_cast<uint64_t>(l.inter / 16u / l.bt_gu) * rkt * 2u * l.ks_gu;
-    return gu_groups > kTwoLaunchGroups ? kMoeFiveLaunches : kMoeTwoLaunches;
+    if (gu_groups <= kTwoLaunchGroups) return kMoeTwoLaunches;
+    // where the decode dominates, the row-slots that read one expert are served together (a grouping launch in front):
+    // every row-slot alone at worst, an expert's tiles decoded once for up to sixteen rows at best
+    return l.rows >= 2u ? kMoeGrouped : kMoeFiveLaunches;
 }
 
 int32_t run_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
@@ -294,8 +299,9 @@ int32_t t3_moe_plan_of(const t3_array* x, const t3_bank* bank, const t3_array* i
         t3::carve_moe(&call, nullptr);
         const int form = t3::decode_form_of(l);
         p.path = form == t3::kMoeTwoLaunches ? T3_MOE_TWO_LAUNCHES
-                 : form == t3::kMoeFourLaunches ? T3_MOE_FOUR_LAUNCHES : T3_MOE_FIVE_LAUNCHES;
-        p.launches = form == t3::kMoeTwoLaunches ? 2 : form == t3::kMoeFourLaunches ? 4 : 5;
+                 : form == t3::kMoeFourLaunches ? T3_MOE_FOUR_LAUNCHES
+                 : form == t3::kMoeGrouped ? T3_MOE_GROUPED : T3_MOE_FIVE_LAUNCHES;
+        p.launches = form == t3::kMoeTwoLaunches ? 2 : form == t3::kMoeFourLaunches ? 4 : form == t3::kMoeGrouped ? 6 : 5;
         p.tiles_a_wave_gu = l.per_gu;
         p.k_slices_gu = l.ks_gu;
         p.tiles_a_load_gu = l.bt_gu;

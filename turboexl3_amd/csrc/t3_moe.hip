@@ -276,6 +276,115 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ?
                                                        cscore);
 }
 
+// ---- the grouped form ------------------------------------------------------------------------------------------
+// Row-slots that read the same expert (or the same shared slot) are served by one set of workgroups: lane L's activation
+// row of the matrix-core fragment is member L % 16's, so a tile decoded once multiplies up to sixteen rows. A column of
+// the product depends on its own activation row alone, so a member's sums are the ones it gets alone. Worth a launch of
+// its own where the decode dominates the call (large experts at several rows).
+constexpr uint32_t kGroupRows = 16u, kMaxRowSlots = 1024u;  // 16 rows x (top-k + shared slots <= 64)
+
+// One workgroup, 256 threads. Members of a group in ascending row-slot order, groups in the order of their first member;
+// an expert read more than sixteen times starts a new group.
+__global__ void __launch_bounds__(256) moe_group(const MoeLaunch a) {
+    __shared__ uint32_t key[kMaxRowSlots], rank[kMaxRowSlots], leaders;
+    const uint32_t rkt = a.rows * (a.topk + a.shared_slots);
+    uint32_t* info = a.groups + 1;
+    uint32_t* member = a.groups + 1u + 2u * rkt;
+    for (uint32_t rk = threadIdx.x; rk < rkt; rk += 256u) {
+        const SlotRef s = resolve_slot(a, rk);
+        key[rk] = !s.live ? 0xFFFFFFFFu : (s.shared ? 0x80000000u | s.e : s.e);
+    }
+    if (threadIdx.x == 0u) leaders = 0u;
+    __syncthreads();
+    for (uint32_t rk = threadIdx.x; rk < rkt; rk += 256u) {
+        uint32_t r = 0;
+        for (uint32_t j = 0; j < rk; ++j) r += key[j] == key[rk] ? 1u : 0u;
+        rank[rk] = r;
+    }
+    __syncthreads();
+    for (uint32_t rk = threadIdx.x; rk < rkt; rk += 256u) {
+        if (key[rk] == 0xFFFFFFFFu) continue;
+        const uint32_t first = rank[rk] / kGroupRows * kGroupRows, pos = rank[rk] - first;
+        uint32_t leader = rk;
+        for (uint32_t j = 0; j < rk; ++j)
+            if (key[j] == key[rk] && rank[j] == first) leader = j;
+        uint32_t g = 0;
+        for (uint32_t j = 0; j < leader; ++j) g += key[j] != 0xFFFFFFFFu && rank[j] % kGroupRows == 0u ? 1u : 0u;
+        member[g * kGroupRows + pos] = rk;
+        if (pos == 0u) {
+            uint32_t count = 0;
+            for (uint32_t j = rk; j < rkt; ++j) count += key[j] == key[rk] && rank[j] < first + kGroupRows ? 1u : 0u;
+            info[2u * g] = key[rk];
+            info[2u * g + 1u] = count;
+            atomicAdd(&leaders, 1u);
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0u) a.groups[0] = leaders;
+}
+
+template <int BT>
+constexpr uint32_t group_lds_bytes() {
+    constexpr uint32_t stage = 4u * gemv_stage_bytes<BT>(), red = 4u * kGroupRows * BT * 4u * 16u;
+    return stage > red ? stage : red;
+}
+
+// Grid (out / 16 / BT, RKT * NPROJ, KS), 256 threads: workgroup row y serves group y / NPROJ (none past the table's count)
+// as moe_gemv serves a row-slot, from the prepared rows of the five-launch form, z [KS][RKT][out] by member.
+template <int CB, int WIDE, int BT, int NPROJ>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ? 2 : 4))) moe_gemv_grouped(const MoeLaunch a) {
+    __shared__ __attribute__((aligned(16))) unsigned char smem[group_lds_bytes<BT>()];
+    constexpr int ST = 2;
+    constexpr uint32_t kStage = gemv_stage_bytes<BT>();
+    const uint32_t g = blockIdx.y / NPROJ, proj = blockIdx.y % NPROJ, blk = blockIdx.x, ksl = blockIdx.z;
+    if (g >= a.groups[0]) return;  // uniform over the workgroup
+    const uint32_t rkt = a.rows * (a.topk + a.shared_slots);
+    const uint32_t key = a.groups[1u + 2u * g], count = a.groups[2u + 2u * g];
+    const uint32_t* member = a.groups + 1u + 2u * rkt + g * kGroupRows;
+    const uint32_t sg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
+    const RoutedBank& bank = (key >> 31) != 0u ? a.shared : a.bank;
+    const uint32_t e = key & 0x7FFFFFFFu;
+    const uint32_t in = NPROJ == 2 ? a.hidden : a.inter, out = NPROJ == 2 ? a.inter : a.hidden;
+    const uint32_t n = NPROJ == 2 ? a.n_gu : a.n_dn;
+    const uint32_t per = NPROJ == 2 ? a.per_gu : a.per_dn, parts = NPROJ == 2 ? a.parts_gu : a.parts_dn;
+    const uint32_t in_tiles = in >> 4, out_tiles = out >> 4, nw = n >> 1;
+    const uint32_t* wmat = (NPROJ == 1 ? bank.down_t : (proj ? bank.up_t : bank.gate_t)) +
+                           static_cast<size_t>(e) * in_tiles * out_tiles * nw;
+    const uint32_t part = ksl * 4u + sg, tk0 = part * per;
+    const uint64_t wstride = static_cast<uint64_t>(out_tiles) * nw;
+    const uint32_t* wbase = wmat + static_cast<uint64_t>(blk) * BT * nw + tk0 * wstride;
+    // the lane's activation row: member lane % 16's (a lane past the members reads the first member's: valid memory, its
+    // sums are dropped)
+    const uint32_t m = lane & 15u;
+    const uint32_t rk = member[m < count ? m : 0u];
+
+    float4v acc[1][BT];
+#pragma unroll
+    for (int t = 0; t < BT; ++t) acc[0][t] = float4v{0.f, 0.f, 0.f, 0.f};
+    if (part < parts) {  // uniform over the wave; a wave past the last part adds zeros below
+        const uint32_t* xq = NPROJ == 1 ? a.hd : (proj ? a.xu : a.xg);
+        uint32_t xoff[1] = {(rk * in + 4u * (lane >> 4)) * 4u};
+        GemvStream<CB, WIDE, 1, BT, ST, XGlobal> stream(
+            wbase, static_cast<uint32_t>(wstride) * 4u, per, n, a.wbits,
+            XGlobal{xq, static_cast<uint64_t>(rkt) * in * 4u, tk0 * 64u, 64u}, xoff, smem + sg * kStage, lane);
+        stream.issue();
+        stream.run(acc);
+    }
+    __syncthreads();
+    float4v(*red)[kGroupRows][BT * 4] = reinterpret_cast<float4v(*)[kGroupRows][BT * 4]>(smem);
+    if (m < count)
+#pragma unroll
+        for (int t = 0; t < BT; ++t) red[sg][m][t * 4 + (lane >> 4)] = acc[0][t];
+    __syncthreads();
+    float* z = NPROJ == 1 ? a.zd : (proj ? a.zu : a.zg);
+    for (uint32_t idx = threadIdx.x; idx < count * (BT * 4u); idx += 256u) {
+        const uint32_t mm = idx / (BT * 4u), i = idx % (BT * 4u), t = i >> 2;
+        const float4v v = ((red[0][mm][i] + red[1][mm][i]) + red[2][mm][i]) + red[3][mm][i];
+        float* dst = z + (static_cast<size_t>(ksl) * rkt + member[mm]) * out + (blk * BT + t) * 16u + 4u * (i & 3u);
+        *reinterpret_cast<float4v*>(dst) = v;
+    }
+}
+
 // Grid (inter / 128, RKT), 64 threads.
 template <int PROF>
 __global__ void __launch_bounds__(64) moe_mid(const MoeLaunch a) {
@@ -329,6 +438,36 @@ hipError_t launch_gemv_cb(const MoeLaunch& a, hipStream_t s) {
     });
 }
 
+template <int CB, int WIDE, int NPROJ>
+hipError_t launch_grouped_bt(const MoeLaunch& a, hipStream_t s) {
+    const uint32_t out = NPROJ == 2 ? a.inter : a.hidden;
+    const uint32_t bt = NPROJ == 2 ? a.bt_gu : a.bt_dn, ks = NPROJ == 2 ? a.ks_gu : a.ks_dn;
+    const uint32_t rkt = a.rows * (a.topk + a.shared_slots);
+    const dim3 grid((out / 16u) / bt, rkt * NPROJ, ks), block(256);
+    if constexpr (WIDE == kNarrow) {
+        if (bt == 8u) {
+            hipLaunchKernelGGL((moe_gemv_grouped<CB, WIDE, 8, NPROJ>), grid, block, 0, s, a);
+            return hipGetLastError();
+        }
+    }
+    if (bt != 4u) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((moe_gemv_grouped<CB, WIDE, 4, NPROJ>), grid, block, 0, s, a);
+    return hipGetLastError();
+}
+
+template <int NPROJ>
+hipError_t launch_grouped_cb(const MoeLaunch& a, hipStream_t s) {
+    return with_reader(NPROJ == 2 ? a.n_gu : a.n_dn, [&](auto reader) {
+        constexpr int R = decltype(reader)::value;
+        switch (a.codebook) {
+            case kMul1: return launch_grouped_bt<kMul1, R, NPROJ>(a, s);
+            case kMcg: return launch_grouped_bt<kMcg, R, NPROJ>(a, s);
+            case kMul1Defer: return launch_grouped_bt<kMul1Defer, R, NPROJ>(a, s);
+            default: return launch_grouped_bt<kMcgPair, R, NPROJ>(a, s);
+        }
+    });
+}
+
 }  // namespace
 
 hipError_t launch_moe_decode(const MoeLaunch& a, int form, hipStream_t s) {
@@ -351,6 +490,22 @@ hipError_t launch_moe_decode(const MoeLaunch& a, int form, hipStream_t s) {
         if ((e = mid_in_down ? launch_gemv_cb<2, true, false, 1>(a, s) : launch_gemv_cb<2, true, true, 1>(a, s)) != hipSuccess)
             return e;
         return mid_in_down ? launch_gemv_cb<1, true, true, 1>(a, s) : launch_gemv_cb<1, false, true, 1>(a, s);
+    }
+    if (form == kMoeGrouped) {
+        // the five launches behind the grouping launch, either profile's stages around the grouped GEMVs
+        hipLaunchKernelGGL(moe_group, dim3(1), dim3(256), 0, s, a);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        if (a.glm) hipLaunchKernelGGL(moe_prep<1>, dim3(a.hidden / 128u, rkt), dim3(64), 0, s, a);
+        else hipLaunchKernelGGL(moe_prep<0>, dim3(a.hidden / 128u, rkt), dim3(64), 0, s, a);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        if ((e = launch_grouped_cb<2>(a, s)) != hipSuccess) return e;
+        if (a.glm) hipLaunchKernelGGL(moe_mid<1>, dim3(a.inter / 128u, rkt), dim3(64), 0, s, a);
+        else hipLaunchKernelGGL(moe_mid<0>, dim3(a.inter / 128u, rkt), dim3(64), 0, s, a);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        if ((e = launch_grouped_cb<1>(a, s)) != hipSuccess) return e;
+        if (a.glm) hipLaunchKernelGGL(moe_combine<1>, dim3(a.hidden / 128u, a.rows), dim3(64), 0, s, a);
+        else hipLaunchKernelGGL(moe_combine<0>, dim3(a.hidden / 128u, a.rows), dim3(64), 0, s, a);
+        return hipGetLastError();
     }
     if (a.glm) {
         // GLM's profile on the five launches (the exact codebook forms, or a configured decode_form): its own roundings
