@@ -87,3 +87,47 @@ def test_captured_calls_replay_to_the_eager_bytes(oracle, t3, w_hat_form_at_any_
         torch.cuda.synchronize()
         for i, (g, w) in enumerate(zip(got, want)):
             assert g == w, f"replay with inputs {seed}: call {i} differs from the eager call"
+
+
+def test_the_grouped_routed_form_under_capture(oracle, t3):
+    """The six-launch grouped form (its grouping launch builds the table on the device from the call's ids): captured once,
+    replayed on new activations AND new routings, every replay the eager bytes."""
+    rng = np.random.default_rng(0x64AA)
+    hidden, inter, experts, topk, rows = 512, 256, 6, 3, 12
+    bank = dev_bank(t3, oracle.synth_bank(rng, experts, hidden, inter, 64))
+    dec = t3.Decode(MCG, 16)
+    x = torch.zeros(1, rows, hidden, dtype=torch.bfloat16, device="cuda")
+    slots = torch.zeros(1, rows, topk, dtype=torch.int32, device="cuda")
+    scores = torch.zeros(1, rows, topk, dtype=torch.float32, device="cuda")
+
+    def new_inputs(seed):
+        r = np.random.default_rng(seed)
+        xm, _ = make_x(r, rows, hidden, torch.bfloat16)
+        s, w = routing(r, rows, topk, experts)
+        s[seed % rows, 0] = -1  # a skipped id, somewhere else every time
+        x.copy_(xm.reshape(1, rows, hidden))
+        slots.copy_(torch.from_numpy(s).reshape(1, rows, topk))
+        scores.copy_(torch.from_numpy(w).reshape(1, rows, topk))
+
+    t3.configure(decode_form=6)
+    try:
+        new_inputs(1)
+        t3.moe_clamped(x, bank, slots, scores, dec, 7)
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                captured = t3.moe_clamped(x, bank, slots, scores, dec, 7)
+        torch.cuda.synchronize()
+        for seed in (2, 3, 4):
+            new_inputs(seed)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            got = bytes_of(captured)
+            want = bytes_of(t3.moe_clamped(x, bank, slots, scores, dec, 7))
+            torch.cuda.synchronize()
+            assert got == want, f"replay with inputs {seed} differs from the eager call"
+    finally:
+        t3.configure()
