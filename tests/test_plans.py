@@ -226,3 +226,22 @@ def test_configure_publishes_whole_snapshots(lib):
         cfg = Config()
         lib.t3_config_default(C.byref(cfg))
         assert lib.t3_configure(C.byref(cfg)) == 0
+
+
+def test_a_process_that_never_configures_runs_the_defaults():
+    """The configuration a library starts with is the one t3_config_default hands out: a fresh process that asks for a
+    plan without ever configuring gets the default's paths (the W_hat form only where its GEMM's tiles fill the GPU)."""
+    import subprocess
+    import sys
+    code = (
+        "import ctypes as C\n"
+        "from tests.test_plans import linear_plan, BF16\n"
+        "from turboexl3_amd import _lib\n"
+        "lib = _lib.lib()\n"
+        "print(linear_plan(lib, 512, 4096, 4096, 64, BF16).path, linear_plan(lib, 600, 4096, 14336, 64, BF16).path)\n"
+    )
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, cwd=root, timeout=120)
+    assert out.returncode == 0, out.stderr
+    assert out.stdout.split() == ["3", "4"]

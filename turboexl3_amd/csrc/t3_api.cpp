@@ -17,7 +17,9 @@ namespace {
 // (The reference sets its configuration once before the first call, src/core/config.zig:175-178; a slot is reused only
 // after 63 further t3_configure calls, by which time no call that started under it is still reading.)
 constexpr uint32_t kConfigSlots = 64;
-t3_config g_configs[kConfigSlots] = {{9, 1, 1, 1, 1, 512, 0}};
+// what a process that never configures runs with, and what t3_config_default hands out
+constexpr t3_config kDefaultConfig = {9, 1, 1, 1, 1, 512, 0, 1};
+t3_config g_configs[kConfigSlots] = {kDefaultConfig};
 std::atomic<uint32_t> g_config_at{0};
 std::mutex g_config_write;
 
@@ -61,8 +63,7 @@ const char* t3_error_name(int32_t status) {
 
 void t3_config_default(t3_config* out) {
     if (!out) return;
-    const t3_config d = {9, 1, 1, 1, 1, 512, 0, 1};
-    *out = d;
+    *out = kDefaultConfig;
 }
 
 int32_t t3_configure(const t3_config* cfg) {
