@@ -217,7 +217,11 @@ int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_
  * t3_config.dense_gemm_rows rows decodes the whole trellis to W_hat on every call; a host that keeps the W_hat of
  * `t3_dequant` calls this instead: prepare, then one plain f16 GEMM that ends with the finish, the same launches on the
  * same operands, so y is `t3_linear`'s W_hat form byte for byte. w_hat F16 [in, out]. Up to 32 rows it refuses with
- * T3_Exl3EngineNotImplemented: decode and verify rows never read a W_hat (dense.zig:1309). */
+ * T3_Exl3EngineNotImplemented: decode and verify rows never read a W_hat (dense.zig:1309). The plain GEMM takes a
+ * 256 x 256 tile a workgroup over the whole K, so this pays where ceil(rows / 256) * ceil(out / 256) reaches about a
+ * hundred tiles; a call of few rows is faster through `t3_linear`'s trellis GEMM, which shares K out (measured at
+ * 4096 -> 14336, us: 64 rows 87 against 42, 512 rows 97 against 123; at 7168 -> 2048: 64 rows 136 against 27,
+ * 2048 rows 153 against 164). The same holds for `t3_linear_unrot`. */
 int32_t t3_linear_resident_workspace_bytes(const t3_array* x, const t3_array* w_hat, size_t* bytes);
 int32_t t3_linear_resident(t3_stream stream, const t3_array* x, const t3_array* w_hat, const t3_array* suh,
                            const t3_array* svh, t3_array* y, void* workspace, size_t workspace_bytes);
