@@ -197,15 +197,18 @@ int32_t admit_prefill(const MoeCall& call) {
     return T3_OK;
 }
 
-// decode_form 3: the five-launch chain; 4: four launches; 9: two launches while a counter a (row-slot, 128-block) fits
-// the workspace's counter area (else four) and the gate|up launch stays within kTwoLaunchGroups workgroups (else five).
+// decode_form 3: the five-launch chain; 4: four launches; 6: the grouped six; 9: two launches while a counter a (row-slot,
+// 128-block) fits the workspace's counter area (else four) and the gate|up launch stays within kTwoLaunchGroups workgroups
+// (else the grouped six from two rows, the five at one).
 // The two launches save three launch boundaries (~12 us of the chain) and pay with every gate|up workgroup's own prepare
 // of its block (once a column workgroup instead of once) and the coherent hand-offs, ~8 % of the decode at eight tiles a
 // load and twice that at four: past eight rounds of the GPU's resident workgroups the five launches are faster. Measured
 // (two against five, us): 4096 x 2048 K4 top-8 at 4 / 5 / 8 / 16 rows 148.7 / 177.0 / 270.8 / 515.5 against 148.5 / 175.3 /
 // 256.1 / 477.5; 7168 x 2048 K3 at 2 / 3 / 8 rows 131.9 / 189.0 / 449.4 against 133.9 / 180.1 / 415.6; 4096 x 1024 K5 at
-// 4 / 8 rows 96.6 / 170.9 against 95.7 / 159.2; 2048 x 512 K3 top-10 at 16 rows 97.1 against 103.1. Every form gives the
-// same bytes, so a row's bytes do not depend on which one its call took.
+// 4 / 8 rows 96.6 / 170.9 against 95.7 / 159.2; 2048 x 512 K3 top-10 at 16 rows 97.1 against 103.1. Past the bound the decode
+// is what the call waits for, and serving the row-slots of one expert together pays (five against grouped, us: 4096 x 2048
+// top-8 of 64 at 8 / 16 rows 256 / 468 against 208 / 274; eight experts of 4096 x 14336 top-2 at 16 rows 754 against 254).
+// Every form gives the same bytes, so a row's bytes do not depend on which one its call took.
 constexpr uint64_t kTwoLaunchGroups = 8192u;
 int decode_form_of(const MoeLaunch& l) {
     const uint64_t rkt = static_cast<uint64_t>(l.rows) * (l.topk + l.shared_slots);

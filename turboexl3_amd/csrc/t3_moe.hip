@@ -11,8 +11,10 @@
 //   combine   per row: acc = fma(score_k, finish(zd_k), acc) in slot order, then y's dtype.
 // A shared expert rides the same launches as slots K..KT-1 of every row, read from its own bank at weight 1.
 // One wave serves one row-slot's K part with the dense path's streaming core; the matrix core runs one live row of 16.
-// Launch forms: five launches (prepare apart) or four (each gate|up wave prepares its own 128-block in LDS): the same
-// statements in the same order, so the same bytes.
+// Launch forms: five launches (prepare apart), four (each gate|up wave prepares its own 128-block in LDS), two (the mid
+// stage and the combine run by the last workgroup to arrive at a block, or the mid stage by the down launch's own waves),
+// or six (the five behind a grouping launch: the row-slots that read one expert served together). The same statements in
+// the same order a row-slot, so the same bytes.
 
 #include "t3_gemv_core.hpp"
 #include "t3_kernels.hpp"
