@@ -53,6 +53,10 @@ CASES = [
     (1024, 512, 96, MUL1, 16, torch.float16),
     (512, 256, 112, MCG, 16, torch.float32),     # K7: the four-word wide reader (K6 and K8 read two words)
     (512, 256, 88, MUL1, 16, torch.float32),     # a fractional wide rate on the two-word reader
+    # the shapes above are small enough for four tiles a load (at most 128 workgroups at eight); these two keep eight,
+    # the benchmark shapes' partition: 66 x 2 and 34 x 4 workgroups
+    (1024, 8448, 64, MCG, 16, torch.float32),
+    (2048, 4352, 48, MUL1, 16, torch.bfloat16),
 ]
 
 
@@ -89,12 +93,16 @@ def test_dense_chain_rows_1_to_32(oracle, t3, in_f, out_f, n, codebook, wbits, d
     (2560, 640, 80, MUL1, 16, torch.float32),    # per = 40 > 16: prepare + arriving GEMV at every row count
     (512, 256, 36, MCG, 16, torch.float32),      # a K part that is not whole 128-blocks
     (1024, 512, 96, MCG, 12, torch.float16),     # wide reader, BT 4: two workgroup columns a 128-column block
+    (1024, 8448, 64, MCG, 16, torch.float16),    # eight tiles a load (132 workgroups), per = 8
+    (2048, 4352, 48, MUL1, 16, torch.bfloat16),  # eight tiles a load, the deferred map
 ])
 def test_fused_launches_equal_the_chain_bytes(oracle, t3, in_f, out_f, n, codebook, wbits, dtype):
     # the served `linear` (one launch up to 4 rows, else prepare + arriving GEMV) against the three-launch chain,
     # byte for byte, twice in a row (the arrival counters must come back to zero)
     case = DenseCase(oracle, t3, 0xF00D + in_f + n, in_f, out_f, n, codebook, wbits)
     x_dev, _ = make_x(case.rng, 32, in_f, dtype)
+    eight = n <= 64 and (out_f // 128) * t3.linear_plan(x_dev[:1], case.d_trellis, case.dec)["k_slices"] > 128
+    assert t3.linear_plan(x_dev[:1], case.d_trellis, case.dec)["tiles_a_load"] == (8 if eight else 4)
     for rows in (1, 2, 4, 5, 16, 17, 32):
         chain = t3.linear_chain(x_dev[:rows], case.d_trellis, case.d_suh, case.d_svh, case.dec)
         for _ in range(2):
