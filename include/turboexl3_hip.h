@@ -104,8 +104,10 @@ typedef struct t3_bank {
 /* ---- configuration (src/core/config.zig; only the fields this path reads) --------------------------------- */
 
 typedef struct t3_config {
-    int32_t decode_form;   /* 3: the five-launch chain; 4: four launches (prepare inside gate|up); 6 (this library's own):
-                            * the grouped six launches whatever the size; 9 (default): two
+    int32_t decode_form;   /* the reference's values (src/core/config.zig:8-12: 3, 5, 6, 7, 8 or 9, each with form 3's bytes),
+                            * mapped to this library's forms: 3, 7: the five-launch chain; 5, 6 (one decode shared among the
+                            * row-slots that chose an expert): the grouped six launches whatever the size; 8: four launches
+                            * (the prepare inside gate|up); 9 (default): two
                             * launches (mid and combine run by the last workgroup to arrive) while the gate|up launch
                             * stays within 8192 workgroups; past that (large experts at several rows, where the decode
                             * dominates) six: the five behind a grouping launch that serves the row-slots of one expert
@@ -248,7 +250,7 @@ int32_t t3_linear_unrot(t3_stream stream, const t3_array* x, const t3_array* w_s
 
 /* x [B, S, D]; inds (U32/I32) and scores (F32/BF16/F16) [B, S, K], K <= 32; y [B, S, D] in x's dtype.
  * `verify_rows` is accepted and ignored, as in the reference (src/root.zig:822-825). Up to 16 rows: the split-K GEMV
- * chain, two launches (six for large experts at several rows; four or five under decode_form 4 or 3; the same bytes,
+ * chain, two launches (six for large experts at several rows; four or five under decode_form 8 or 3; the same bytes,
  * and t3_moe_plan_of says which). A routed id outside [0, E) is skipped. Gate and up
  * must share a rate (T3_Exl3GateUpRateMismatch); the down's rate may differ (the reference refuses that,
  * src/root.zig:841; this library's kernels take a rate a launch). */
@@ -361,7 +363,7 @@ int32_t t3_moe_plan_of(const t3_array* x, const t3_bank* bank, const t3_array* i
  * gate and up round to bf16 and are limited (limit 0: not), the SiLU rounds to bf16, the product rounds to bf16; y F32
  * [B, S, K, D]: each routed slot's own down finish, no score (the host combines a row's slots and its shared expert). A
  * slot whose id is outside [0, E) is skipped and its output left as it is. Any row count: the decode chain up to 16 rows
- * (the launch forms of t3_moe, the same bytes; the exact codebook forms and decode_form 4 take the five launches), the
+ * (the launch forms of t3_moe, the same bytes; the exact codebook forms and decode_form 8 take the five launches), the
  * prefill chain above. Workspace: t3_moe_workspace_bytes (shared_bank NULL). */
 int32_t t3_moe_glm(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds, t3_decode dec,
                    int32_t limit, t3_array* y, void* workspace, size_t workspace_bytes);

@@ -140,7 +140,7 @@ def test_launch_forms_give_the_same_bytes(oracle, t3):
             nine = call()
             again = call()
             assert bytes_of(nine) == bytes_of(again)
-            for form in (3, 4, 6):
+            for form in (3, 8, 6):
                 t3.configure(decode_form=form)
                 try:
                     other = call()
@@ -166,7 +166,7 @@ def test_launch_forms_give_the_same_bytes_at_the_reference_rows(oracle, t3):
         args = (x_dev[:rows].reshape(1, rows, hidden), dbank, torch.from_numpy(slots[:rows]).cuda().reshape(1, rows, topk),
                 torch.from_numpy(scores[:rows]).cuda().reshape(1, rows, topk), dec)
         nine = t3.moe(*args)
-        for form in (3, 4, 6):
+        for form in (3, 8, 6):
             t3.configure(decode_form=form)
             try:
                 other = t3.moe(*args)
@@ -373,7 +373,7 @@ def test_fused_gated_shared_expert(oracle, t3, codebook, n, dtype):
     # `moe` has one, and a step of bf16 at 4 rms is 3e-2 of rms: the dense bar (src/hip_tests.zig:326), not the routed
     # one. f16: two steps of f16 at 4 rms (8e-3 of rms) on top of the f32 bar's share
     bar = 2.5e-2 if dtype == torch.bfloat16 else 1e-2
-    for form in (9, 4, 3, 6):
+    for form in (9, 8, 3, 6, 5, 7):
         t3.configure(decode_form=form)
         try:
             for count in (1, 3, 4):

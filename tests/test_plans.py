@@ -139,7 +139,8 @@ def test_config4_prefill_items(lib):
 
 def test_decode_forms_by_configuration(lib):
     cfg = Config()
-    for form, path, launches in ((3, 2, 5), (4, 1, 4), (6, 4, 6), (9, 0, 2)):
+    # the reference's values (src/core/config.zig:140), each mapped to one of this library's forms
+    for form, path, launches in ((3, 2, 5), (7, 2, 5), (8, 1, 4), (5, 4, 6), (6, 4, 6), (9, 0, 2)):
         lib.t3_config_default(C.byref(cfg))
         cfg.decode_form = form
         assert lib.t3_configure(C.byref(cfg)) == 0

@@ -72,8 +72,9 @@ int32_t t3_configure(const t3_config* cfg) {
                           (cfg->mcg_pair == 0 || cfg->mcg_pair == 1) && (cfg->mul1_defer == 0 || cfg->mul1_defer == 1) &&
                           cfg->dense_gemm_rows >= 0 && (cfg->dense_rows_alone == 0 || cfg->dense_rows_alone == 1) &&
                           (cfg->dense_gemm_fill == 0 || cfg->dense_gemm_fill == 1);
-    if ((cfg->decode_form != 3 && cfg->decode_form != 4 && cfg->decode_form != 6 && cfg->decode_form != 9) || !flags_ok)
-        return T3_InvalidTurboexl3Config;
+    // the reference's own set (src/core/config.zig:140): any other value is refused, as there
+    const int32_t f = cfg->decode_form;
+    if ((f != 3 && f != 5 && f != 6 && f != 7 && f != 8 && f != 9) || !flags_ok) return T3_InvalidTurboexl3Config;
     std::lock_guard<std::mutex> lock(g_config_write);
     const uint32_t next = g_config_at.load(std::memory_order_relaxed) + 1u;
     g_configs[next % kConfigSlots] = *cfg;

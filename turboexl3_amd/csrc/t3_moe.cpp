@@ -197,9 +197,12 @@ int32_t admit_prefill(const MoeCall& call) {
     return T3_OK;
 }
 
-// decode_form 3: the five-launch chain; 4: four launches; 6: the grouped six; 9: two launches while a counter a (row-slot,
-// 128-block) fits the workspace's counter area (else four) and the gate|up launch stays within kTwoLaunchGroups workgroups
-// (else the grouped six from two rows, the five at one).
+// decode_form takes the reference's values (src/core/config.zig:8-12), every one with form 3's bytes there and here, each
+// mapped to the form of this library that stands closest: 3 and 7 (the prepare a launch of its own): the five-launch
+// chain; 5 and 6 ("share one decode among the row-slots that chose an expert"): the grouped six; 8 (the prepare inside
+// the gate|up launch): four launches; 9: two launches while a counter a (row-slot, 128-block) fits the workspace's counter
+// area (else four) and the gate|up launch stays within kTwoLaunchGroups workgroups (else the grouped six from two rows,
+// the five at one).
 // The two launches save three launch boundaries (~12 us of the chain) and pay with every gate|up workgroup's own prepare
 // of its block (once a column workgroup instead of once) and the coherent hand-offs, ~8 % of the decode at eight tiles a
 // load and twice that at four: past eight rounds of the GPU's resident workgroups the five launches are faster. Measured
@@ -214,9 +217,10 @@ int decode_form_of(const MoeLaunch& l) {
     const uint64_t rkt = static_cast<uint64_t>(l.rows) * (l.topk + l.shared_slots);
     const size_t widest = (l.hidden > l.inter ? l.hidden : l.inter) / 128u;
     const size_t counters = rkt * widest;
-    if (config().decode_form == 3) return kMoeFiveLaunches;
-    if (config().decode_form == 6) return kMoeGrouped;
-    if (config().decode_form == 4 || counters * 4u > kCounterBytes) return kMoeFourLaunches;
+    const int32_t want = config().decode_form;
+    if (want == 3 || want == 7) return kMoeFiveLaunches;
+    if (want == 5 || want == 6) return kMoeGrouped;
+    if (want == 8 || counters * 4u > kCounterBytes) return kMoeFourLaunches;
     const uint64_t gu_groups = static_cast<uint64_t>(l.inter / 16u / l.bt_gu) * rkt * 2u * l.ks_gu;
     if (gu_groups <= kTwoLaunchGroups) return kMoeTwoLaunches;
     // where the decode dominates, the row-slots that read one expert are served together (a grouping launch in front):
