@@ -310,7 +310,7 @@ def shapes_section(torch, api) -> dict:
         d = Dense(torch, api, in_f, out_f, n, MCG_CB, rows, torch.bfloat16, seed=78, copies=2, outliers=False)
         took = {}
         for name, cfg in (("served", {}), ("trellis_gemm", {"dense_gemm_rows": 0}),
-                          ("w_hat_form", {"dense_gemm_rows": 1, "dense_gemm_fill": 0})):
+                          ("w_hat_form", {"dense_gemm_rows": 1})):
             api.configure(**cfg)
             try:
                 d.bind(rows)

@@ -117,18 +117,15 @@ typedef struct t3_config {
     int32_t mcg_pair;      /* 1 (default): MCG's GEMV feeds the hashed pair to the matrix core unrounded; 0: the f16 weight */
     int32_t mul1_defer;    /* 1 (default): MUL1's affine map applied once an output (src/core/dense.zig deferFor); 0: per weight */
     int32_t dense_gemm_rows; /* dense calls of this many rows or more decode W_hat once into the workspace and run this
-                              * library's plain f16 GEMM, which ends with the finish (where dense_gemm_fill allows).
-                              * Default 512; 0: never */
+                              * library's plain f16 GEMM (K shared out over the grid where its tiles are few), which
+                              * ends with the finish. Default 513: up to four 128-row items the trellis GEMM is the faster,
+                              * from five on this form (measured over ten shapes); 0: never */
     int32_t dense_rows_alone; /* 0 (default): rows 17..32 run the GEMV and above 32 rows a dense call's launch shape follows
                                * its rows (K parts at few rows, the W_hat form at many), so a row's bytes can differ between
                                * calls of different row counts (each within the bars). 1: every call above 16 rows takes the
                                * trellis GEMM with one K part, and a row's bytes ignore the call's other rows, as the
                                * reference's own GEMM holds them for 17, 40, 129 and 200 rows (src/hip_tests.zig:866-880);
                                * few-row calls then run up to twice as long */
-    int32_t dense_gemm_fill;  /* 1 (default): the W_hat form serves only where its GEMM's grid fills the GPU: tiles =
-                               * ceil(rows / 256) * ceil(out / 256) (a 256 x 256 tile a workgroup, no K split) at least 120
-                               * and at least in / 56 (below that the trellis GEMM's K parts are faster, measured); 0: from
-                               * dense_gemm_rows rows whatever the shape */
 } t3_config;
 
 /* The served configuration. */
@@ -195,8 +192,7 @@ enum {
     T3_DENSE_ARRIVE = 1,       /* prepare launch, then the GEMV whose last workgroup a block runs the finish */
     T3_DENSE_CHAIN = 2,        /* prepare, GEMV, finish */
     T3_DENSE_TRELLIS_GEMM = 3, /* above 32 rows: prepare, the GEMM that decodes in registers, finish */
-    T3_DENSE_W_HAT_GEMM = 4    /* from dense_gemm_rows rows, where the GEMM's grid fills the GPU (dense_gemm_fill): W_hat
-                                * decode, prepare, plain f16 GEMM, finish */
+    T3_DENSE_W_HAT_GEMM = 4    /* from dense_gemm_rows rows: W_hat decode, prepare, plain f16 GEMM, finish */
 };
 typedef struct t3_linear_plan {
     int32_t path;            /* T3_DENSE_* */
@@ -219,11 +215,11 @@ int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_
  * t3_config.dense_gemm_rows rows decodes the whole trellis to W_hat on every call; a host that keeps the W_hat of
  * `t3_dequant` calls this instead: prepare, then one plain f16 GEMM that ends with the finish, the same launches on the
  * same operands, so y is `t3_linear`'s W_hat form byte for byte. w_hat F16 [in, out]. Up to 32 rows it refuses with
- * T3_Exl3EngineNotImplemented: decode and verify rows never read a W_hat (dense.zig:1309). The plain GEMM takes a
- * 256 x 256 tile a workgroup over the whole K, so this pays where ceil(rows / 256) * ceil(out / 256) reaches about a
- * hundred tiles; a call of few rows is faster through `t3_linear`'s trellis GEMM, which shares K out (measured at
- * 4096 -> 14336, us: 64 rows 87 against 42, 512 rows 97 against 123; at 7168 -> 2048: 64 rows 136 against 27,
- * 2048 rows 153 against 164). The same holds for `t3_linear_unrot`. */
+ * T3_Exl3EngineNotImplemented: decode and verify rows never read a W_hat (dense.zig:1309). Where the GEMM's 256 x 256
+ * tiles are few it shares K out over the grid (planes in the workspace, the finish a launch of its own), so a kept W_hat
+ * pays at every row count above 32 (measured against `t3_linear` at 4096 -> 14336, us: 64 rows 36 against 41, 512 rows
+ * 77 against 103, 2048 rows 235 against 276). `t3_linear_unrot` takes no workspace and so has no K parts: a W_std call
+ * of few rows leaves most of the GPU idle (64 rows: 78 us) and is faster through `t3_linear`. */
 int32_t t3_linear_resident_workspace_bytes(const t3_array* x, const t3_array* w_hat, size_t* bytes);
 int32_t t3_linear_resident(t3_stream stream, const t3_array* x, const t3_array* w_hat, const t3_array* suh,
                            const t3_array* svh, t3_array* y, void* workspace, size_t workspace_bytes);

@@ -55,7 +55,7 @@ def test_configure_refuses_unserved_values(lib):
     cfg = Config()
     lib.t3_config_default(C.byref(cfg))
     assert (cfg.decode_form, cfg.dec_one, cfg.prefill, cfg.mcg_pair, cfg.mul1_defer, cfg.dense_gemm_rows,
-            cfg.dense_rows_alone, cfg.dense_gemm_fill) == (9, 1, 1, 1, 1, 512, 0, 1)
+            cfg.dense_rows_alone) == (9, 1, 1, 1, 1, 513, 0)
     # src/core/config.zig:191-192,245: 3, 5, 6, 7, 8 and 9 are served, 0, 4 and 10 refused
     for form in (0, 4, 10):
         cfg.decode_form = form
@@ -65,7 +65,7 @@ def test_configure_refuses_unserved_values(lib):
         assert lib.t3_configure(C.byref(cfg)) == 0
     cfg.decode_form, cfg.dense_gemm_rows = 9, -1
     assert lib.t3_error_name(lib.t3_configure(C.byref(cfg))).decode() == "InvalidTurboexl3Config"
-    cfg.dense_gemm_rows = 512
+    cfg.dense_gemm_rows = 513
     cfg.decode_form = 3
     assert lib.t3_configure(C.byref(cfg)) == 0
     cfg.decode_form = 9

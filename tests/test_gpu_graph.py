@@ -18,16 +18,7 @@ def t3():
     return api
 
 
-@pytest.fixture
-def w_hat_form_at_any_shape(t3):
-    """The small shapes here would not fill the plain GEMM's grid, and the default configuration then keeps them on the
-    trellis GEMM: this test wants the W_hat form itself."""
-    t3.configure(dense_gemm_fill=0)
-    yield
-    t3.configure()
-
-
-def test_captured_calls_replay_to_the_eager_bytes(oracle, t3, w_hat_form_at_any_shape):
+def test_captured_calls_replay_to_the_eager_bytes(oracle, t3):
     rng = np.random.default_rng(0x64A9)
     in_f, out_f, n = 1024, 512, 64
     trellis, suh, svh = oracle.synth_linear(rng, in_f, out_f, n)

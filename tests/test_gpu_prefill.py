@@ -178,13 +178,8 @@ def test_dense_w_hat_form_from_512_rows(oracle, t3, in_f, out_f, n, codebook, dt
     x_dev, x_f32 = make_x(case.rng, rows, in_f, dtype, outliers=True)
     yref = case.ref(x_f32)
     bar = F32_BAR if dtype == torch.float32 else BF16_DENSE_BAR
-    t3.configure(dense_gemm_fill=0)  # these shapes would not fill the plain GEMM's grid: take the W_hat form all the same
-    try:
-        assert t3.linear_plan(x_dev, case.d_trellis, case.dec)["path"] == 4  # T3_DENSE_W_HAT_GEMM
-        got = to_f32(t3.linear(x_dev, case.d_trellis, case.d_suh, case.d_svh, case.dec))
-    finally:
-        t3.configure()
-    assert t3.linear_plan(x_dev, case.d_trellis, case.dec)["path"] == 3  # the default keeps them on the trellis GEMM
+    assert t3.linear_plan(x_dev, case.d_trellis, case.dec)["path"] == 4  # T3_DENSE_W_HAT_GEMM (few tiles: K parts)
+    got = to_f32(t3.linear(x_dev, case.d_trellis, case.d_suh, case.d_svh, case.dec))
     t3.configure(dense_gemm_rows=0)
     try:
         fused = to_f32(t3.linear(x_dev, case.d_trellis, case.d_suh, case.d_svh, case.dec))
@@ -213,7 +208,7 @@ def test_dense_over_a_resident_w_hat(oracle, t3, in_f, out_f, n, codebook, wbits
     w_hat = t3.dequant(case.d_trellis, case.dec)
     x_dev, x_f32 = make_x(case.rng, 530, in_f, dtype, outliers=True)
     bar = F32_BAR if dtype == torch.float32 else BF16_DENSE_BAR
-    t3.configure(dense_gemm_rows=33, dense_gemm_fill=0)
+    t3.configure(dense_gemm_rows=33)
     try:
         for rows in (40, 530):
             per_call = t3.linear(x_dev[:rows], case.d_trellis, case.d_suh, case.d_svh, case.dec)

@@ -224,7 +224,7 @@ def test_dense_draws_where_one_f16_step_passes_the_bar(oracle, t3, seed):
     rms = np.sqrt((ref.astype(np.float64) ** 2).mean(axis=1, keepdims=True))
     step = np.spacing(np.maximum(np.abs(ref), np.float32(2.0 ** -14)).astype(np.float16)).astype(np.float64)
     for rows in d["row_counts"]:
-        for form in ({}, {"mcg_pair": 0, "mul1_defer": 0}, {"dense_gemm_fill": 0}):
+        for form in ({}, {"mcg_pair": 0, "mul1_defer": 0}, {"dense_gemm_rows": 0}):
             t3.configure(**form)
             try:
                 got = to_f32(run_dense(t3, d, rows))

@@ -93,15 +93,14 @@ def test_few_rows_share_the_tile_rows_out(lib):
     assert p.workgroups == 56 * 16
     q = linear_plan(lib, 300, 4096, 14336, 64, BF16)   # three items: 168 workgroups a part, two parts fit the 512 resident
     assert (q.path, q.k_slices) == (3, 2)
-    # from dense_gemm_rows (512) rows the W_hat form serves: decode once, prepare, the f16 GEMM that ends with the finish
+    # from dense_gemm_rows (513) rows the W_hat form serves: decode once, prepare, the f16 GEMM that ends with the finish
+    # (or, over few tiles, shares K out and leaves the finish to a launch of its own): five 128-row items or more
     w = linear_plan(lib, 600, 4096, 14336, 64, BF16)
     assert (w.path, w.launches, w.k_slices) == (4, 3, 1)
-    # ... where its GEMM's 256 x 256 tiles fill the GPU (at least 120 of them, and in / 64): 512 rows of this shape are
-    # 2 x 56 = 112 tiles and stay on the trellis GEMM; a narrow out needs many rows; a long K more tiles (in / 56)
-    assert linear_plan(lib, 512, 4096, 14336, 64, BF16).path == 3
-    assert [linear_plan(lib, r, 7168, 2048, 48, BF16).path for r in (1024, 2048, 4096)] == [3, 3, 4]
-    assert [linear_plan(lib, r, 4096, 4096, 64, BF16).path for r in (1024, 1536, 2048)] == [3, 3, 4]
-    assert [linear_plan(lib, r, 14336, 4096, 64, BF16).path for r in (2048, 4096)] == [3, 4]
+    assert [linear_plan(lib, r, 4096, 14336, 64, BF16).path for r in (512, 513)] == [3, 4]
+    assert [linear_plan(lib, r, 7168, 2048, 48, BF16).path for r in (512, 1024, 4096)] == [3, 4, 4]
+    few = linear_plan(lib, 1024, 7168, 2048, 48, BF16)      # 4 x 8 tiles: eight K parts of 28 steps fill the 256 compute units
+    assert (few.k_slices, few.launches, few.workgroups) == (8, 4, 256)
     cfg = Config()
     lib.t3_config_default(C.byref(cfg))
     cfg.dense_gemm_rows = 0
@@ -209,7 +208,7 @@ def test_configure_publishes_whole_snapshots(lib):
     def writer(rows_alone):
         cfg = Config()
         lib.t3_config_default(C.byref(cfg))
-        cfg.dense_rows_alone, cfg.dense_gemm_rows = rows_alone, 512 if rows_alone == 0 else 0
+        cfg.dense_rows_alone, cfg.dense_gemm_rows = rows_alone, 513 if rows_alone == 0 else 0
         while not stop.is_set():
             assert lib.t3_configure(C.byref(cfg)) == 0
 

@@ -40,7 +40,7 @@ class Bank(C.Structure):
 class Config(C.Structure):
     _fields_ = [("decode_form", C.c_int32), ("dec_one", C.c_int32), ("prefill", C.c_int32),
                 ("mcg_pair", C.c_int32), ("mul1_defer", C.c_int32), ("dense_gemm_rows", C.c_int32),
-                ("dense_rows_alone", C.c_int32), ("dense_gemm_fill", C.c_int32)]
+                ("dense_rows_alone", C.c_int32)]
 
 
 class Block(C.Structure):

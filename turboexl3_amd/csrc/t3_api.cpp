@@ -18,7 +18,7 @@ namespace {
 // after 63 further t3_configure calls, by which time no call that started under it is still reading.)
 constexpr uint32_t kConfigSlots = 64;
 // what a process that never configures runs with, and what t3_config_default hands out
-constexpr t3_config kDefaultConfig = {9, 1, 1, 1, 1, 512, 0, 1};
+constexpr t3_config kDefaultConfig = {9, 1, 1, 1, 1, 513, 0};
 t3_config g_configs[kConfigSlots] = {kDefaultConfig};
 std::atomic<uint32_t> g_config_at{0};
 std::mutex g_config_write;
@@ -70,8 +70,7 @@ int32_t t3_configure(const t3_config* cfg) {
     if (!cfg) return T3_BadArgs;
     const bool flags_ok = (cfg->dec_one == 0 || cfg->dec_one == 1) && (cfg->prefill == 0 || cfg->prefill == 1) &&
                           (cfg->mcg_pair == 0 || cfg->mcg_pair == 1) && (cfg->mul1_defer == 0 || cfg->mul1_defer == 1) &&
-                          cfg->dense_gemm_rows >= 0 && (cfg->dense_rows_alone == 0 || cfg->dense_rows_alone == 1) &&
-                          (cfg->dense_gemm_fill == 0 || cfg->dense_gemm_fill == 1);
+                          cfg->dense_gemm_rows >= 0 && (cfg->dense_rows_alone == 0 || cfg->dense_rows_alone == 1);
     // the reference's own set (src/core/config.zig:140): any other value is refused, as there
     const int32_t f = cfg->decode_form;
     if ((f != 3 && f != 5 && f != 6 && f != 7 && f != 8 && f != 9) || !flags_ok) return T3_InvalidTurboexl3Config;

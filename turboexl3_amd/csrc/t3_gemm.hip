@@ -56,7 +56,14 @@ struct GemmArgs {
     int dt;               // FINISH: y's dtype (t3::Dtype); else y is in the operands' dtype
     uint32_t rows, in, cols, ldw, mt;
     uint32_t ntf, nth;    // column blocks of 256, then of 128
+    float* planes;        // PLANES: f32 [K parts][rows][cols], part blockIdx.z's sums
+    uint32_t part_steps;  // PLANES: K = 32 steps a part
 };
+
+// what a launch ends with: the product in the operands' dtype; format.finishOutput on z = f16(product); or the f32 sums of
+// one K part (a launch of few tiles shares K out over grid z so that the GPU fills; the planes are summed in part order
+// by the finish launch behind it)
+enum GemmEnd : int { kGemmPlain = 0, kGemmFinish = 1, kGemmPlanes = 2 };
 
 __device__ __forceinline__ uint4v gemm_rsrc(const void* p, uint64_t bytes) {
     const uint64_t addr = reinterpret_cast<uint64_t>(p);
@@ -85,8 +92,9 @@ __device__ __forceinline__ float4v gemm_mfma(uint4v a, uint4v b, float4v c) {
 // Grid (8 mt, ceil(ntf / 8) + ceil(nth / 8)), 512 threads: ntf column blocks of 256 first, then nth of 128 (launched
 // last, so they fill the launch's tail: a workgroup holds a compute unit alone, and a last round of full tiles on half
 // the compute units would take as long as a full one).
-template <bool BF16, bool FINISH>
+template <bool BF16, int END>
 __global__ void __launch_bounds__(512) gemm_half(const GemmArgs a) {
+    constexpr bool FINISH = END == kGemmFinish;
     __shared__ __attribute__((aligned(16))) unsigned char smem[kGLds];
     const uint32_t die = blockIdx.x & 7u, mi = blockIdx.x >> 3;
     const uint32_t yf = (a.ntf + 7u) >> 3;
@@ -116,13 +124,17 @@ __global__ void __launch_bounds__(512) gemm_half(const GemmArgs a) {
     }
     const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(smem));
     const uint32_t w_step_bytes = kGK * a.ldw * 2u;
+    // the K steps this workgroup walks: all of them, or K part blockIdx.z's
+    const uint32_t steps_all = a.in / kGK;
+    const uint32_t step0 = END == kGemmPlanes ? blockIdx.z * a.part_steps : 0u;
+    const uint32_t steps = END == kGemmPlanes ? (steps_all - step0 < a.part_steps ? steps_all - step0 : a.part_steps) : steps_all;
     auto issue = [&](uint32_t step, uint32_t slot) {
-        const uint32_t base = lds0 + slot * kGStep;
+        const uint32_t base = lds0 + slot * kGStep, at = step0 + step;
 #pragma unroll
-        for (uint32_t i = 0; i < 2u; ++i) gemm_load_to_lds(xdesc, base + (2u * wave + i) * 1024u, x_voff[i], step * (kGK * 2u));
+        for (uint32_t i = 0; i < 2u; ++i) gemm_load_to_lds(xdesc, base + (2u * wave + i) * 1024u, x_voff[i], at * (kGK * 2u));
 #pragma unroll
         for (uint32_t i = 0; i < 2u; ++i)
-            gemm_load_to_lds(wdesc, base + kGXBytes + (2u * wave + i) * 1024u, w_voff[i], step * w_step_bytes);
+            gemm_load_to_lds(wdesc, base + kGXBytes + (2u * wave + i) * 1024u, w_voff[i], at * w_step_bytes);
     };
 
     // where a lane's fragments sit inside a step's 32 KB
@@ -147,7 +159,6 @@ __global__ void __launch_bounds__(512) gemm_half(const GemmArgs a) {
 #pragma unroll
             for (int rb = 0; rb < 8; ++rb) acc[cb][rb] = float4v{0.f, 0.f, 0.f, 0.f};
 
-        const uint32_t steps = a.in / kGK;
 #pragma unroll
         for (uint32_t t = 0; t + 1u < kGD; ++t) issue(t, t);   // loads past the last step bring zeros or unused bytes
         gemm_wait_loads<static_cast<int>(kGD - 2u) * kGLoadsAStep>();
@@ -178,6 +189,20 @@ __global__ void __launch_bounds__(512) gemm_half(const GemmArgs a) {
             slot = slot + 1u == kGD ? 0u : slot + 1u;
         }
         gemm_wait_loads<0>();
+        if constexpr (END == kGemmPlanes) {
+            // the part's f32 sums as they lie in the accumulators: four adjacent columns of one row a lane and block
+            float* plane = a.planes + static_cast<size_t>(blockIdx.z) * a.rows * a.cols;
+#pragma unroll
+            for (int rb = 0; rb < 8; ++rb)
+#pragma unroll
+                for (int cb = 0; cb < CBN; ++cb) {
+                    const uint32_t row = row0 + 128u * wm + static_cast<uint32_t>(rb) * 16u + (lane & 15u);
+                    const uint32_t col = col0 + 16u * CBN * wn + static_cast<uint32_t>(cb) * 16u + 4u * (lane >> 4);
+                    if (row < a.rows && col < a.cols)
+                        *reinterpret_cast<float4v*>(plane + static_cast<size_t>(row) * a.cols + col) = acc[cb][rb];
+                }
+            return;
+        }
         // every wave is past its last fragment reads (the loop's last barrier) and no load is in flight: the ring's
         // memory takes the output tile. lane: row 16 rb + lane % 16, columns 16 cb + 4 (lane / 16) .. + 3 of the wave's part
         __syncthreads();
@@ -273,8 +298,8 @@ hipError_t launch_gemm_half(const void* x, const void* w, void* y, uint32_t rows
                             bool bf16, hipStream_t s) {
     const GemmArgs a = gemm_args(x, w, y, rows, in, cols, ldw);
     const dim3 grid = gemm_grid(a), block(512);
-    if (bf16) hipLaunchKernelGGL((gemm_half<true, false>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((gemm_half<false, false>), grid, block, 0, s, a);
+    if (bf16) hipLaunchKernelGGL((gemm_half<true, kGemmPlain>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((gemm_half<false, kGemmPlain>), grid, block, 0, s, a);
     return hipGetLastError();
 }
 
@@ -286,7 +311,21 @@ hipError_t launch_gemm_finish(const uint16_t* xp, const uint16_t* w_hat, const u
     a.svh = svh;
     a.dt = dtype;
     const dim3 grid = gemm_grid(a), block(512);
-    hipLaunchKernelGGL((gemm_half<false, true>), grid, block, 0, s, a);
+    hipLaunchKernelGGL((gemm_half<false, kGemmFinish>), grid, block, 0, s, a);
+    return hipGetLastError();
+}
+
+// planes f32 [kparts][rows][out]: part p = the sums over K steps [p part_steps, (p + 1) part_steps) of xp W_hat (cols a
+// multiple of 4, planes 16-byte aligned); kparts from gemm_kparts
+hipError_t launch_gemm_planes(const uint16_t* xp, const uint16_t* w_hat, float* planes, uint32_t rows, uint32_t in,
+                              uint32_t out, uint32_t kparts, hipStream_t s) {
+    GemmArgs a = gemm_args(xp, w_hat, nullptr, rows, in, out, out);
+    if (a.nth != 0u || kparts == 0u || (in / kGK) % kparts != 0u) return hipErrorInvalidValue;
+    a.planes = planes;
+    a.part_steps = (in / kGK) / kparts;
+    dim3 grid = gemm_grid(a);
+    grid.z = kparts;
+    hipLaunchKernelGGL((gemm_half<false, kGemmPlanes>), grid, dim3(512), 0, s, a);
     return hipGetLastError();
 }
 

@@ -177,6 +177,22 @@ hipError_t launch_gemm_half(const void* x, const void* w, void* y, uint32_t rows
 // the same product over a W_hat with format.finishOutput at its end: y [rows][out] in `dtype` from the prepared rows
 hipError_t launch_gemm_finish(const uint16_t* xp, const uint16_t* w_hat, const uint16_t* svh, void* y, uint32_t rows,
                               uint32_t in, uint32_t out, int dtype, hipStream_t s);
+// The W_hat form over few tiles: the product's f32 sums a K part (planes f32 [kparts][rows][out]), then the finish over the
+// planes summed in part order (the trellis GEMM's finish launch). A 256 x 256 tile a workgroup over the whole K leaves a
+// call of few rows on a handful of compute units; K parts fill them.
+hipError_t launch_gemm_planes(const uint16_t* xp, const uint16_t* w_hat, float* planes, uint32_t rows, uint32_t in,
+                              uint32_t out, uint32_t kparts, hipStream_t s);
+hipError_t launch_dense_planes_finish(const DenseLaunch& d, const float* planes, uint32_t kparts, hipStream_t s);
+// K parts of that GEMM: the most (a power of two, at most 16, each part at least 16 steps of K = 32) that keep the launch
+// within one workgroup a compute unit; 1: the launch that ends with the finish itself. (Fewer parts where the planes are
+// large, priced at 8 bytes an output a part through HBM, measured slower: the planes of such calls live in the Infinity
+// Cache. 2048 x 7168 at 512 rows 50 -> 68 us, 2560 x 5120 at 1024 rows 63 -> 78.)
+inline uint32_t gemm_kparts(uint32_t rows, uint32_t in, uint32_t out) {
+    const uint32_t tiles = ((rows + 255u) / 256u) * ((out + 255u) / 256u), steps = in / 32u;
+    uint32_t k = 1;
+    while (k < 16u && tiles * 2u * k <= 256u && steps % (2u * k) == 0u && steps / (2u * k) >= 16u) k *= 2u;
+    return k;
+}
 inline bool gemm_half_ok(uint64_t in, uint64_t ldw) {
     return in % 32u == 0u && ldw % 8u == 0u && in * ldw * 2u < (1ull << 32);
 }

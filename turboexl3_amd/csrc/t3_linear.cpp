@@ -100,28 +100,29 @@ constexpr uint32_t kGemvRowsMax = 32;
 uint32_t gemv_rows_max() { return config().dense_rows_alone ? 16u : kGemvRowsMax; }
 
 // From dense_gemm_rows rows up a dense call decodes W_hat once and multiplies plainly (src/core/dense.zig:909-922,
-// 1290-1302): the decode is paid once a call, not once a 128-row item. The plain GEMM takes a 256 x 256 tile a workgroup
-// over the whole K, so it only pays where its grid fills the GPU: with few tiles (a narrow out, or rows in the hundreds)
-// a handful of workgroups walk K while the trellis GEMM shares the tile rows out into K parts. Measured (trellis GEMM
-// against W_hat form, us): 7168 x 2048 at 1024 / 4096 rows 66 / 156 and 173 / 170, 14336 x 4096 at 512 / 2048 / 4096 rows
-// 97 / 290, 297 / 322 and 570 / 459, 4096 x 4096 at 1024 / 2048 / 4096 rows 67 / 104, 105 / 106 and 182 / 140, 8192 x 8192 at
-// 1024 / 1536 rows 177 / 194 and 320 / 226, 5120 x 5120 at 1024 / 1536 rows 105 / 126 and 161 / 127, 4096 x 14336 at 512 / 640 /
-// 2048 rows 111 / 116, 170 / 123 and 316 / 244, 2048 x 7168 at 1024 rows 80 / 70. Across ten shapes and eight row counts
-// from 256 to 4096 the W_hat form wins from about 120 tiles (half the compute units), a long K asking for more (tiles x 56
-// >= in: 8192 x 8192 at 1024 rows, 128 tiles, 172 / 195); the rule below is within 10 % of the better form in every cell
-// measured.
+// 1290-1302): the decode is paid once a call, not once a 128-row item, and the plain GEMM shares K out where its tiles are
+// few (gemm_kparts), so it fills the GPU at any shape. Measured over ten model shapes x eight row counts from 256 to 4096
+// (trellis GEMM against W_hat form, us): up to 512 rows (four items) the trellis GEMM wins or ties everywhere (4096 x 4096
+// 47 / 63, 4096 x 14336 98 / 109); from five items on the W_hat form does (640 rows: 4096 x 4096 64 / 56, 4096 x 14336
+// 158 / 130, 14336 x 4096 159 / 133, 7168 x 2048 60 / 55; 2048 rows: 2560 x 5120 109 / 84, 8192 x 8192 321 / 270), with
+// ties at 1024 rows and two cells the other way (2048 x 2048 at 2048 rows 49 / 57, 7168 x 2048 at 1024 rows 65 / 75).
+// Hence the default of 513.
 bool takes_w_hat(const DenseLaunch& l) {
     const int32_t from = config().dense_gemm_rows;
-    if (config().dense_rows_alone || from <= 0 || l.rows < static_cast<uint32_t>(from) || !gemm_half_ok(l.in, l.out))
-        return false;
-    const uint64_t tiles = static_cast<uint64_t>((l.rows + 255u) / 256u) * ((l.out + 255u) / 256u);
-    return !config().dense_gemm_fill || (tiles >= 120u && tiles * 56u >= l.in);
+    return !config().dense_rows_alone && from > 0 && l.rows >= static_cast<uint32_t>(from) && gemm_half_ok(l.in, l.out);
 }
 
 struct WhatScratch {
     uint16_t* w_hat;  // f16 [in][out]
     uint16_t* xp;     // f16 [rows][in], natural order
+    float* planes;    // f32 [K parts][rows][out] where the GEMM shares K out (gemm_kparts > 1), else null
 };
+
+// the planes of the W_hat form's GEMM over few tiles
+float* carve_gemm_planes(Carver& c, const DenseLaunch& l) {
+    const uint32_t k = gemm_kparts(l.rows, l.in, l.out);
+    return k > 1u ? c.take<float>(static_cast<size_t>(k) * l.rows * l.out * 4u) : nullptr;
+}
 
 WhatScratch carve_dense_w_hat(DenseCall* call, void* workspace) {
     DenseLaunch& l = call->launch;
@@ -130,14 +131,21 @@ WhatScratch carve_dense_w_hat(DenseCall* call, void* workspace) {
     WhatScratch w;
     w.w_hat = c.take<uint16_t>(static_cast<size_t>(l.in) * l.out * 2u);
     w.xp = c.take<uint16_t>(static_cast<size_t>(l.rows) * l.in * 2u);
+    w.planes = carve_gemm_planes(c, l);
     call->workspace = c.used;
     return w;
 }
 
-// prepare (natural order) -> finish(z = f16(xp W_hat)): the product and the finish are one launch, z stays in LDS
-int32_t run_over_w_hat(const DenseLaunch& l, const uint16_t* w_hat, uint16_t* xp, hipStream_t s) {
+// prepare (natural order) -> finish(z = f16(xp W_hat)): the product and the finish are one launch, z stays in LDS; over
+// few tiles the product's K is shared out into parts (planes) and the finish is a launch of its own
+int32_t run_over_w_hat(const DenseLaunch& l, const uint16_t* w_hat, uint16_t* xp, float* planes, hipStream_t s) {
     if (const int32_t st = hip_status(launch_dense_prep_natural(l, xp, s)); st != T3_OK) return st;
-    return hip_status(launch_gemm_finish(xp, w_hat, l.svh, l.y, l.rows, l.in, l.out, l.dtype, s));
+    const uint32_t k = gemm_kparts(l.rows, l.in, l.out);
+    if (k == 1u) return hip_status(launch_gemm_finish(xp, w_hat, l.svh, l.y, l.rows, l.in, l.out, l.dtype, s));
+    if (!planes) return T3_BadArgs;
+    if (const int32_t st = hip_status(launch_gemm_planes(xp, w_hat, planes, l.rows, l.in, l.out, k, s)); st != T3_OK)
+        return st;
+    return hip_status(launch_dense_planes_finish(l, planes, k, s));
 }
 
 int32_t run_w_hat(const DenseCall& call, const WhatScratch& w, int codebook, hipStream_t s) {
@@ -145,7 +153,7 @@ int32_t run_w_hat(const DenseCall& call, const WhatScratch& w, int codebook, hip
     if (const int32_t st = hip_status(launch_dequant(l.trellis, w.w_hat, l.in, l.out, l.n, l.wbits, codebook, s));
         st != T3_OK)
         return st;
-    return run_over_w_hat(l, w.w_hat, w.xp, s);
+    return run_over_w_hat(l, w.w_hat, w.xp, w.planes, s);
 }
 
 // The operand checks of a call over a kept W_hat f16 [in, out]: `check_dense`'s, with the W_hat in the trellis's place.
@@ -195,11 +203,12 @@ int32_t check_resident(const t3_array* x, const t3_array* w_hat, const t3_array*
 
 // arrival counters (untouched here: a workspace's head stays zero whoever is called with it), xp f16 [rows][in]
 // (natural order)
-void carve_resident(DenseCall* call, void* workspace, uint16_t** xp) {
+void carve_resident(DenseCall* call, void* workspace, uint16_t** xp, float** planes) {
     DenseLaunch& l = call->launch;
     Carver c(workspace);
     l.arrive = c.take<uint32_t>(kCounterBytes);
     *xp = c.take<uint16_t>(static_cast<size_t>(l.rows) * l.in * 2u);
+    *planes = carve_gemm_planes(c, l);
     call->workspace = c.used;
 }
 
@@ -282,8 +291,10 @@ int32_t t3_linear_plan_of(const t3_array* x, const t3_array* trellis, t3_decode 
         const uint32_t item_rows = l.rows <= 64u ? 64u : 128u, items = (l.rows + item_rows - 1u) / item_rows;
         p.workgroups = t3::dense_prefill_workgroups(l.out, items) * l.ks;
     } else {
-        p.launches = 3;  // W_hat decode, prepare, the GEMM that finishes
-        p.k_slices = 1;
+        // W_hat decode, prepare, the GEMM that finishes; over few tiles the GEMM's K parts and the finish by itself
+        p.k_slices = t3::gemm_kparts(l.rows, l.in, l.out);
+        p.launches = p.k_slices == 1u ? 3 : 4;
+        p.workgroups = ((l.rows + 255u) / 256u) * ((l.out + 255u) / 256u) * p.k_slices;
     }
     *plan = p;
     return T3_OK;
@@ -371,7 +382,8 @@ int32_t t3_linear_resident_workspace_bytes(const t3_array* x, const t3_array* w_
     t3::DenseCall call;
     if (const int32_t st = t3::check_resident(x, w_hat, nullptr, nullptr, nullptr, &call); st != T3_OK) return st;
     uint16_t* xp;
-    t3::carve_resident(&call, nullptr, &xp);
+    float* planes;
+    t3::carve_resident(&call, nullptr, &xp, &planes);
     *bytes = call.workspace;
     return T3_OK;
 }
@@ -383,9 +395,11 @@ int32_t t3_linear_resident(t3_stream stream, const t3_array* x, const t3_array* 
     if (const int32_t st = t3::check_resident(x, w_hat, suh, svh, y, &call); st != T3_OK) return st;
     if (!t3::workspace_ok(workspace)) return T3_BadArgs;
     uint16_t* xp;
-    t3::carve_resident(&call, workspace, &xp);
+    float* planes;
+    t3::carve_resident(&call, workspace, &xp, &planes);
     if (workspace_bytes < call.workspace) return T3_WorkspaceTooSmall;
-    return t3::run_over_w_hat(call.launch, static_cast<const uint16_t*>(w_hat->data), xp, static_cast<hipStream_t>(stream));
+    return t3::run_over_w_hat(call.launch, static_cast<const uint16_t*>(w_hat->data), xp, planes,
+                              static_cast<hipStream_t>(stream));
 }
 
 int32_t t3_unrot_workspace_bytes(const t3_array* trellis, size_t* bytes) {

@@ -760,6 +760,13 @@ hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s) {
     return hipGetLastError();
 }
 
+hipError_t launch_dense_planes_finish(const DenseLaunch& d, const float* planes, uint32_t kparts, hipStream_t s) {
+    DenseLaunch f = d;
+    f.ks = kparts;
+    f.codebook = kMcg;  // finished weights went into the product: no deferred map
+    return launch_pf_dense_finish(f, planes, s);
+}
+
 hipError_t launch_dense_prep_natural(const DenseLaunch& d, uint16_t* xp, hipStream_t s) {
     return launch_pf_dense_prep<true>(d, xp, nullptr, s);
 }
