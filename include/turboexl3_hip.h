@@ -218,8 +218,8 @@ int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_
  * T3_Exl3EngineNotImplemented: decode and verify rows never read a W_hat (dense.zig:1309). Where the GEMM's 256 x 256
  * tiles are few it shares K out over the grid (planes in the workspace, the finish a launch of its own), so a kept W_hat
  * pays at every row count above 32 (measured against `t3_linear` at 4096 -> 14336, us: 64 rows 36 against 41, 512 rows
- * 77 against 103, 2048 rows 235 against 276). `t3_linear_unrot` takes no workspace and so has no K parts: a W_std call
- * of few rows leaves most of the GPU idle (64 rows: 78 us) and is faster through `t3_linear`. */
+ * 77 against 103, 2048 rows 235 against 276). `t3_linear_unrot` takes no workspace and so has no K parts:
+ * `t3_linear_unrot_parts` is its form for calls of few rows. */
 int32_t t3_linear_resident_workspace_bytes(const t3_array* x, const t3_array* w_hat, size_t* bytes);
 int32_t t3_linear_resident(t3_stream stream, const t3_array* x, const t3_array* w_hat, const t3_array* suh,
                            const t3_array* svh, t3_array* y, void* workspace, size_t workspace_bytes);
@@ -241,6 +241,15 @@ int32_t t3_unrot_weight(t3_stream stream, const t3_array* trellis, const t3_arra
  * the trellis paths byte for byte. */
 int32_t t3_linear_unrot(t3_stream stream, const t3_array* x, const t3_array* w_std, int64_t col0, int64_t cols,
                         t3_array* y);
+/* The same product for calls of few rows or a narrow member (no counterpart in the reference, whose W_std product is one
+ * MLX matmul whatever the shape): where the GEMM's 256 x 256 tiles are few it shares K out over the grid (f32 planes in
+ * the workspace, summed in part order and rounded once by a second launch), so the GPU fills: 4096 -> 14336 at 64 rows
+ * 78 -> 29 us. Where the tiles fill the GPU by themselves it is `t3_linear_unrot`'s launch and bytes; with K parts the
+ * sums are added in another order and a value can differ from `t3_linear_unrot`'s by a step of the dtype (held to the
+ * same bars). Checks and refusals as `t3_linear_unrot`. */
+int32_t t3_linear_unrot_workspace_bytes(const t3_array* x, const t3_array* w_std, int64_t col0, int64_t cols, size_t* bytes);
+int32_t t3_linear_unrot_parts(t3_stream stream, const t3_array* x, const t3_array* w_std, int64_t col0, int64_t cols,
+                              t3_array* y, void* workspace, size_t workspace_bytes);
 
 /* ---- routed experts (src/root.zig:822-904,976-1004) ------------------------------------------------------- */
 

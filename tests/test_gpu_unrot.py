@@ -109,11 +109,16 @@ def test_linear_unrot_against_the_rotated_chain(oracle, t3, in_f, out_f, n, code
     x_dev, x_f32 = make_x(case.rng, rows, in_f, dtype)
     want = case.ref(x_f32).astype(np.float64)
     for r in (33, 97):
-        got = to_f32(t3.linear_unrot(x_dev[:r], w)).astype(np.float64)
-        d = got - want[:r]
-        rel = math.sqrt((d * d).sum() / (want[:r] ** 2).sum())
-        assert rel <= UNROT_BAR_RMS, f"rows {r}: rel rms {rel:.3e} over {UNROT_BAR_RMS:.3e}"
-        assert np.abs(d).max() <= UNROT_BAR_STEPS * step_of(np.abs(want[:r]).max(), dtype)
+        # the plain launch, and the form that shares K out over the grid where the tiles are few (these shapes: all of them)
+        for product in (t3.linear_unrot, t3.linear_unrot_parts):
+            got = to_f32(product(x_dev[:r], w)).astype(np.float64)
+            d = got - want[:r]
+            rel = math.sqrt((d * d).sum() / (want[:r] ** 2).sum())
+            assert rel <= UNROT_BAR_RMS, f"{product.__name__} rows {r}: rel rms {rel:.3e} over {UNROT_BAR_RMS:.3e}"
+            assert np.abs(d).max() <= UNROT_BAR_STEPS * step_of(np.abs(want[:r]).max(), dtype)
+        # the two sum K in different orders: a value may differ by a step of the dtype, no more
+        a, b = to_f32(t3.linear_unrot(x_dev[:r], w)), to_f32(t3.linear_unrot_parts(x_dev[:r], w))
+        assert np.abs(a - b).max() <= 2 * step_of(np.abs(want[:r]).max(), dtype)
     # decode and verify rows keep the trellis paths: the plain product refuses them
     with pytest.raises(t3.T3Error) as e:
         t3.linear_unrot(x_dev[:32], w)

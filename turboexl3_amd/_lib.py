@@ -97,6 +97,8 @@ SYMBOLS = {
     "t3_unrot_weight": (C.c_int32, [C.c_void_p, _AP, _AP, _AP, Decode, _AP, C.c_int64, C.c_void_p, C.c_void_p,
                                     C.c_size_t]),
     "t3_linear_unrot": (C.c_int32, [C.c_void_p, _AP, _AP, C.c_int64, C.c_int64, _AP]),
+    "t3_linear_unrot_workspace_bytes": (C.c_int32, [_AP, _AP, C.c_int64, C.c_int64, C.POINTER(C.c_size_t)]),
+    "t3_linear_unrot_parts": (C.c_int32, [C.c_void_p, _AP, _AP, C.c_int64, C.c_int64, _AP, C.c_void_p, C.c_size_t]),
     "t3_moe": (C.c_int32, [C.c_void_p, _AP, _BP, _AP, _AP, Decode, C.c_int32, _AP, C.c_void_p, C.c_size_t]),
     "t3_moe_clamped": (C.c_int32, [C.c_void_p, _AP, _BP, _AP, _AP, Decode, C.c_int32, _AP, C.c_void_p, C.c_size_t]),
     "t3_moe_swiglu": (C.c_int32, [C.c_void_p, _AP, _BP, _AP, _AP, Decode, C.c_int32, C.c_int32, _AP, C.c_void_p,

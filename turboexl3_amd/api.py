@@ -233,6 +233,20 @@ def linear_unrot(x, w_std, col0: int = 0, cols=None, stream=None) -> torch.Tenso
     return y
 
 
+def linear_unrot_parts(x, w_std, col0: int = 0, cols=None, stream=None) -> torch.Tensor:
+    """`linear_unrot` with K shared out over the grid where the GEMM's tiles are few (calls of few rows)."""
+    L = _lib.lib()
+    cols = w_std.shape[1] - col0 if cols is None else cols
+    y = torch.empty(*x.shape[:-1], cols, dtype=x.dtype, device=x.device)
+    ax, aw, ay = _arr(x), _arr(w_std), _arr(y)
+    need = C.c_size_t(0)
+    _check(L.t3_linear_unrot_workspace_bytes(C.byref(ax), C.byref(aw), col0, cols, C.byref(need)))
+    ws = _workspace(x.device, need.value)
+    _check(L.t3_linear_unrot_parts(_stream_ptr(stream), C.byref(ax), C.byref(aw), col0, cols, C.byref(ay), ws.data_ptr(),
+                                   ws.numel()))
+    return y
+
+
 def _cbank(bank: Bank):
     keep = []
 

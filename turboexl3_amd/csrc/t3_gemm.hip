@@ -315,17 +315,44 @@ hipError_t launch_gemm_finish(const uint16_t* xp, const uint16_t* w_hat, const u
     return hipGetLastError();
 }
 
-// planes f32 [kparts][rows][out]: part p = the sums over K steps [p part_steps, (p + 1) part_steps) of xp W_hat (cols a
-// multiple of 4, planes 16-byte aligned); kparts from gemm_kparts
-hipError_t launch_gemm_planes(const uint16_t* xp, const uint16_t* w_hat, float* planes, uint32_t rows, uint32_t in,
-                              uint32_t out, uint32_t kparts, hipStream_t s) {
-    GemmArgs a = gemm_args(xp, w_hat, nullptr, rows, in, out, out);
-    if (a.nth != 0u || kparts == 0u || (in / kGK) % kparts != 0u) return hipErrorInvalidValue;
+// planes f32 [kparts][rows][cols]: part p = the sums over K steps [p part_steps, (p + 1) part_steps) of x w[:, 0:cols]
+// (cols a multiple of 4, planes 16-byte aligned); kparts from gemm_kparts
+hipError_t launch_gemm_planes(const void* x, const void* w, float* planes, uint32_t rows, uint32_t in, uint32_t cols,
+                              uint32_t ldw, bool bf16, uint32_t kparts, hipStream_t s) {
+    GemmArgs a = gemm_args(x, w, nullptr, rows, in, cols, ldw);
+    if (a.nth != 0u || kparts == 0u || (in / kGK) % kparts != 0u || cols % 4u != 0u) return hipErrorInvalidValue;
     a.planes = planes;
     a.part_steps = (in / kGK) / kparts;
     dim3 grid = gemm_grid(a);
     grid.z = kparts;
-    hipLaunchKernelGGL((gemm_half<false, kGemmPlanes>), grid, dim3(512), 0, s, a);
+    if (bf16) hipLaunchKernelGGL((gemm_half<true, kGemmPlanes>), grid, dim3(512), 0, s, a);
+    else hipLaunchKernelGGL((gemm_half<false, kGemmPlanes>), grid, dim3(512), 0, s, a);
+    return hipGetLastError();
+}
+
+namespace {
+// y [rows][cols] in f16 or bf16 = the planes summed in part order, one rounding: the plain product's end over K parts.
+// Four adjacent outputs a thread.
+template <bool BF16>
+__global__ void __launch_bounds__(256) gemm_planes_round(const float* planes, uint16_t* y, uint64_t count4, uint64_t plane,
+                                                         uint32_t kparts) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;
+    if (i >= count4) return;
+    float4v v = *reinterpret_cast<const float4v*>(planes + 4u * i);
+    for (uint32_t k = 1; k < kparts; ++k) v += *reinterpret_cast<const float4v*>(planes + k * plane + 4u * i);
+    uint32_t h[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) h[c] = BF16 ? bf16_bits(v[c]) : half_bits(v[c]);
+    *reinterpret_cast<uint2*>(y + 4u * i) = uint2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+}
+}  // namespace
+
+hipError_t launch_gemm_planes_round(const float* planes, void* y, uint32_t rows, uint32_t cols, uint32_t kparts, bool bf16,
+                                    hipStream_t s) {
+    const uint64_t plane = static_cast<uint64_t>(rows) * cols, count4 = plane / 4u;
+    const dim3 grid(static_cast<uint32_t>((count4 + 255u) / 256u)), block(256);
+    if (bf16) hipLaunchKernelGGL(gemm_planes_round<true>, grid, block, 0, s, planes, static_cast<uint16_t*>(y), count4, plane, kparts);
+    else hipLaunchKernelGGL(gemm_planes_round<false>, grid, block, 0, s, planes, static_cast<uint16_t*>(y), count4, plane, kparts);
     return hipGetLastError();
 }
 

@@ -180,8 +180,11 @@ hipError_t launch_gemm_finish(const uint16_t* xp, const uint16_t* w_hat, const u
 // The W_hat form over few tiles: the product's f32 sums a K part (planes f32 [kparts][rows][out]), then the finish over the
 // planes summed in part order (the trellis GEMM's finish launch). A 256 x 256 tile a workgroup over the whole K leaves a
 // call of few rows on a handful of compute units; K parts fill them.
-hipError_t launch_gemm_planes(const uint16_t* xp, const uint16_t* w_hat, float* planes, uint32_t rows, uint32_t in,
-                              uint32_t out, uint32_t kparts, hipStream_t s);
+hipError_t launch_gemm_planes(const void* x, const void* w, float* planes, uint32_t rows, uint32_t in, uint32_t cols,
+                              uint32_t ldw, bool bf16, uint32_t kparts, hipStream_t s);
+// the plain product's end over K parts: y [rows][cols] (f16 or bf16) = the planes summed in part order, one rounding
+hipError_t launch_gemm_planes_round(const float* planes, void* y, uint32_t rows, uint32_t cols, uint32_t kparts, bool bf16,
+                                    hipStream_t s);
 hipError_t launch_dense_planes_finish(const DenseLaunch& d, const float* planes, uint32_t kparts, hipStream_t s);
 // K parts of that GEMM: the most (a power of two, at most 16, each part at least 16 steps of K = 32) that keep the launch
 // within one workgroup a compute unit; 1: the launch that ends with the finish itself. (Fewer parts where the planes are

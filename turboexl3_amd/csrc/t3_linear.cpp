@@ -143,7 +143,8 @@ int32_t run_over_w_hat(const DenseLaunch& l, const uint16_t* w_hat, uint16_t* xp
     const uint32_t k = gemm_kparts(l.rows, l.in, l.out);
     if (k == 1u) return hip_status(launch_gemm_finish(xp, w_hat, l.svh, l.y, l.rows, l.in, l.out, l.dtype, s));
     if (!planes) return T3_BadArgs;
-    if (const int32_t st = hip_status(launch_gemm_planes(xp, w_hat, planes, l.rows, l.in, l.out, k, s)); st != T3_OK)
+    if (const int32_t st = hip_status(launch_gemm_planes(xp, w_hat, planes, l.rows, l.in, l.out, l.out, false, k, s));
+        st != T3_OK)
         return st;
     return hip_status(launch_dense_planes_finish(l, planes, k, s));
 }
@@ -456,30 +457,82 @@ int32_t t3_unrot_weight(t3_stream stream, const t3_array* trellis, const t3_arra
                                            w_std->dtype, nonfinite, s));  // T3_F16, T3_BF16 = the kernels' numbering
 }
 
-int32_t t3_linear_unrot(t3_stream stream, const t3_array* x, const t3_array* w_std, int64_t col0, int64_t cols,
-                        t3_array* y) {
-    if (!t3::array_ok(x) || !t3::array_ok(w_std) || !t3::array_ok(y)) return T3_BadArgs;
-    if (x->ndim < 1 || w_std->ndim != 2 || y->ndim != x->ndim) return T3_BadExl3Shape;
+namespace {
+// the operand checks of a product over W_std; rows and in out
+int32_t check_unrot(const t3_array* x, const t3_array* w_std, int64_t col0, int64_t cols, const t3_array* y, int64_t* rows_out,
+                    int64_t* in_out) {
+    if (!t3::array_ok(x) || !t3::array_ok(w_std) || (y && !t3::array_ok(y))) return T3_BadArgs;
+    if (x->ndim < 1 || w_std->ndim != 2 || (y && y->ndim != x->ndim)) return T3_BadExl3Shape;
     const int64_t in = w_std->shape[0];
     int64_t rows = 1;
     for (int i = 0; i + 1 < x->ndim; ++i) {
-        if (x->shape[i] != y->shape[i]) return T3_BadExl3Shape;
+        if (y && x->shape[i] != y->shape[i]) return T3_BadExl3Shape;
         rows *= x->shape[i];
     }
-    if (x->shape[x->ndim - 1] != in || y->shape[y->ndim - 1] != cols || col0 < 0 || cols <= 0 ||
+    if (x->shape[x->ndim - 1] != in || (y && y->shape[y->ndim - 1] != cols) || col0 < 0 || cols <= 0 ||
         col0 + cols > w_std->shape[1] || rows <= 0 || rows > (1ll << 30) || in > (1ll << 30) ||
         w_std->shape[1] > (1ll << 30))
         return T3_BadExl3Shape;
-    if ((w_std->dtype != T3_F16 && w_std->dtype != T3_BF16) || x->dtype != w_std->dtype || y->dtype != w_std->dtype)
+    if ((w_std->dtype != T3_F16 && w_std->dtype != T3_BF16) || x->dtype != w_std->dtype || (y && y->dtype != w_std->dtype))
         return T3_BadExl3Dtype;
-    if (!t3::aligned16(x) || !t3::aligned16(w_std) || !t3::aligned16(y) || col0 % 8 != 0) return T3_BadArgs;
+    if (!t3::aligned16(x) || !t3::aligned16(w_std) || (y && !t3::aligned16(y)) || col0 % 8 != 0) return T3_BadArgs;
     if (rows <= 32 || !t3::gemm_half_ok(static_cast<uint64_t>(in), static_cast<uint64_t>(w_std->shape[1])))
         return T3_Exl3EngineNotImplemented;
+    *rows_out = rows;
+    *in_out = in;
+    return T3_OK;
+}
+// K parts of the product over W_std: the W_hat form's, where the planes' four-column stores fit
+uint32_t unrot_kparts(int64_t rows, int64_t in, int64_t cols) {
+    if (cols % 4 != 0 || rows * cols >= (1ll << 31)) return 1u;
+    return t3::gemm_kparts(static_cast<uint32_t>(rows), static_cast<uint32_t>(in), static_cast<uint32_t>(cols));
+}
+}  // namespace
+
+int32_t t3_linear_unrot(t3_stream stream, const t3_array* x, const t3_array* w_std, int64_t col0, int64_t cols,
+                        t3_array* y) {
+    if (!y) return T3_BadArgs;
+    int64_t rows = 0, in = 0;
+    if (const int32_t st = check_unrot(x, w_std, col0, cols, y, &rows, &in); st != T3_OK) return st;
     const size_t esz = 2u;
     return t3::hip_status(t3::launch_gemm_half(
         x->data, static_cast<const unsigned char*>(w_std->data) + static_cast<size_t>(col0) * esz, y->data,
         static_cast<uint32_t>(rows), static_cast<uint32_t>(in), static_cast<uint32_t>(cols),
         static_cast<uint32_t>(w_std->shape[1]), w_std->dtype == T3_BF16, static_cast<hipStream_t>(stream)));
+}
+
+int32_t t3_linear_unrot_workspace_bytes(const t3_array* x, const t3_array* w_std, int64_t col0, int64_t cols, size_t* bytes) {
+    if (!bytes) return T3_BadArgs;
+    int64_t rows = 0, in = 0;
+    if (const int32_t st = check_unrot(x, w_std, col0, cols, nullptr, &rows, &in); st != T3_OK) return st;
+    t3::Carver c(nullptr);
+    c.take<uint32_t>(t3::kCounterBytes);
+    const uint32_t k = unrot_kparts(rows, in, cols);
+    if (k > 1u) c.take<float>(static_cast<size_t>(k) * rows * cols * 4u);
+    *bytes = c.used;
+    return T3_OK;
+}
+
+int32_t t3_linear_unrot_parts(t3_stream stream, const t3_array* x, const t3_array* w_std, int64_t col0, int64_t cols,
+                              t3_array* y, void* workspace, size_t workspace_bytes) {
+    if (!y) return T3_BadArgs;
+    int64_t rows = 0, in = 0;
+    if (const int32_t st = check_unrot(x, w_std, col0, cols, y, &rows, &in); st != T3_OK) return st;
+    if (!t3::workspace_ok(workspace)) return T3_BadArgs;
+    t3::Carver c(workspace);
+    c.take<uint32_t>(t3::kCounterBytes);  // the head stays as it is: the fused launches' counters
+    const uint32_t k = unrot_kparts(rows, in, cols);
+    float* planes = k > 1u ? c.take<float>(static_cast<size_t>(k) * rows * cols * 4u) : nullptr;
+    if (workspace_bytes < c.used) return T3_WorkspaceTooSmall;
+    const unsigned char* w = static_cast<const unsigned char*>(w_std->data) + static_cast<size_t>(col0) * 2u;
+    const bool bf16 = w_std->dtype == T3_BF16;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const uint32_t r = static_cast<uint32_t>(rows), i = static_cast<uint32_t>(in), n = static_cast<uint32_t>(cols);
+    const uint32_t ldw = static_cast<uint32_t>(w_std->shape[1]);
+    if (k == 1u) return t3::hip_status(t3::launch_gemm_half(x->data, w, y->data, r, i, n, ldw, bf16, s));
+    if (const int32_t st = t3::hip_status(t3::launch_gemm_planes(x->data, w, planes, r, i, n, ldw, bf16, k, s)); st != T3_OK)
+        return st;
+    return t3::hip_status(t3::launch_gemm_planes_round(planes, y->data, r, n, k, bf16, s));
 }
 
 }  // extern "C"
