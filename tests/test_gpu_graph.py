@@ -43,6 +43,7 @@ def test_captured_calls_replay_to_the_eager_bytes(oracle, t3):
             t3.linear(x_dense, d_t, d_suh, d_svh, dec),              # 530 rows: W_hat decoded, the f16 GEMM with its finish
             t3.linear_resident(x_dense[:100], w_hat, d_suh, d_svh),  # the same GEMM over a kept W_hat
             t3.linear_unrot(x_dense[:100], w_std),                   # the plain product over the un-rotated weight
+            t3.linear_unrot_parts(x_dense[:100], w_std),             # the same with K shared out: planes, then their sum
             t3.linear_static(x_dense[:3], d_t, d_suh, d_svh, dec),   # scratch in the library's own device array
             t3.moe_clamped(x_moe[:, :2], bank, slots[:, :2], scores[:, :2], dec, 7),   # two arriving launches
             t3.moe_clamped(x_moe, bank, slots, scores, dec, 7),      # 20 rows: route, GEMMs, combine
