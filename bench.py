@@ -322,6 +322,18 @@ def shapes_section(torch, api) -> dict:
         cells.append({"in": in_f, "out": out_f, "n": n, "rows": rows, **took})
         del d
     out["dense_above_32_rows"] = cells
+    # a call of few rows over a kept weight: the plain GEMM shares K out over the grid where its tiles are few
+    d = Dense(torch, api, 4096, 14336, 64, MCG_CB, 64, torch.bfloat16, seed=81, copies=1, outliers=False)
+    w_hat = api.dequant(d.trellis[0], d.dec)
+    w_std, _ = api.unrot_weight(d.trellis[0], d.suh, d.svh, d.dec, torch.bfloat16)
+    x = d.x[:64]
+    took = {name: graph_time(torch, fn, 8, 2, 3) * 1e6 for name, fn in (
+        ("linear_us", lambda i, st: api.linear(x, d.trellis[0], d.suh, d.svh, d.dec)),
+        ("resident_w_hat_us", lambda i, st: api.linear_resident(x, w_hat, d.suh, d.svh)),
+        ("w_std_us", lambda i, st: api.linear_unrot(x, w_std)),
+        ("w_std_k_parts_us", lambda i, st: api.linear_unrot_parts(x, w_std)))}
+    out["dense_64_rows_over_kept_weights"] = {"in": 4096, "out": 14336, "n": 64, "rows": 64, **took}
+    del d, w_hat, w_std, x
     # routed decode over large experts: two launches up to 8192 gate|up workgroups; past it the five launches behind a
     # grouping launch (the row-slots of one expert served together); GLM's profile
     cells = []
