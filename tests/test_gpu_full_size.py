@@ -129,8 +129,8 @@ def test_config5_dense_4096_rows_w_hat_form(oracle, t3):
 
 
 def test_config5_shape_few_rows_on_the_trellis_gemm(oracle, t3):
-    # few rows decode the matrix once: the launch shares the tile rows out into K parts (sixteen at 64 rows here, eight at
-    # 128, one at 600) and one item's column blocks go round all the dies; sampled blocks against the oracle either way
+    # few rows decode the matrix once: the launch shares the tile rows out into K parts (eight at 64 and at 128 rows here,
+    # one at 600) and one item's column blocks go round all the dies; sampled blocks against the oracle either way
     in_f, out_f, n = 4096, 14336, 64
     rng = np.random.default_rng(0xC56)
     trellis, suh, svh = oracle.synth_linear(rng, in_f, out_f, n)
@@ -151,7 +151,7 @@ def test_config5_shape_few_rows_on_the_trellis_gemm(oracle, t3):
 
 def test_config5_shape_rows_alone_configuration(oracle, t3):
     # The reference's own GEMM holds rows 0-16 of a 40-, 129- or 200-row call to the bytes of the 17-row call
-    # (src/hip_tests.zig:866-880). Here the served launch shape follows the rows (the GEMV up to 32, then sixteen K parts at
+    # (src/hip_tests.zig:866-880). Here the served launch shape follows the rows (the GEMV up to 32, then eight K parts at
     # 64 rows of this shape, two at 300, the W_hat form at 600), so those bytes may differ between row counts;
     # dense_rows_alone = 1 sends every call above 16 rows to the trellis GEMM with one K part and gives the reference's
     # invariant back, at its own row counts and beyond.
@@ -161,7 +161,7 @@ def test_config5_shape_rows_alone_configuration(oracle, t3):
     d_t, d_suh, d_svh = dev_u16(trellis), dev_f16_bits(suh), dev_f16_bits(svh)
     x_dev, x_f32 = make_x(rng, 600, in_f, torch.bfloat16)
     plans = {rows: t3.linear_plan(x_dev[:rows], d_t, t3.Decode.mcg) for rows in (17, 64, 300, 600)}
-    assert [plans[r]["k_slices"] for r in (64, 300, 600)] == [16, 2, 1] and plans[600]["path"] == 4
+    assert [plans[r]["k_slices"] for r in (64, 300, 600)] == [8, 2, 1] and plans[600]["path"] == 4
     assert plans[17]["path"] == 2  # the GEMV's chain
     t3.configure(dense_rows_alone=1)
     try:

@@ -87,10 +87,10 @@ def test_dense_path_by_rows(lib):
 
 
 def test_few_rows_share_the_tile_rows_out(lib):
-    # the trellis GEMM at 64 rows: one item, 56 workgroup columns spread over the dies, sixteen K parts of eight steps
+    # the trellis GEMM at 64 rows: one item, 56 workgroup columns spread over the dies, eight K parts of sixteen steps
     p = linear_plan(lib, 64, 4096, 14336, 64, BF16)
-    assert (p.path, p.launches, p.k_slices) == (3, 3, 16)
-    assert p.workgroups == 56 * 16
+    assert (p.path, p.launches, p.k_slices) == (3, 3, 8)
+    assert p.workgroups == 56 * 8
     q = linear_plan(lib, 300, 4096, 14336, 64, BF16)   # three items: 168 workgroups a part, two parts fit the 512 resident
     assert (q.path, q.k_slices) == (3, 2)
     # from dense_gemm_rows (513) rows the W_hat form serves: decode once, prepare, the f16 GEMM that ends with the finish

@@ -141,10 +141,11 @@ hipError_t launch_dense_prefill(const DenseLaunch& d, hipStream_t s);
 inline uint32_t dense_prefill_kparts(uint32_t rows, uint32_t in, uint32_t out) {
     const uint32_t item_rows = rows <= 64u ? 64u : 128u, items = (rows + item_rows - 1u) / item_rows;
     const uint32_t nblk = (out + 255u) / 256u, steps = in / 32u;
-    // the most parts that still fit one round of the workgroups the GPU holds at once (two a compute unit with a 128-row
-    // item's accumulators, four with a 64-row item's): a launch that spills into a second round takes that round's whole
-    // time for its few workgroups
-    const uint32_t slots = item_rows == 64u ? 1024u : 512u;
+    // the most parts that still fit one round of the 512 workgroups the GPU holds at once (two a compute unit): a launch
+    // that spills into a second round takes that round's whole time for its few workgroups. (The 64-row item's smaller
+    // accumulators would let four workgroups share a compute unit, but 1024 was measured slower than 512 for it as well:
+    // 4096 x 14336 at 64 rows 39.3 against 32.2 us.)
+    const uint32_t slots = 512u;
     uint32_t k = 1;
     while (k < 16u && steps % (4u * k) == 0u && steps / (2u * k) >= 8u && items * nblk * 2u * k <= slots) k *= 2u;
     return k;
