@@ -110,8 +110,9 @@ typedef struct t3_config {
                             * (the prepare inside gate|up); 9 (default): two
                             * launches (mid and combine run by the last workgroup to arrive) while the gate|up launch
                             * stays within 8192 workgroups; past that (large experts at several rows, where the decode
-                            * dominates) six: the five behind a grouping launch that serves the row-slots of one expert
-                            * together; the same bytes whichever runs; others refused */
+                            * dominates), or where a uniform routing is expected to leave few enough experts hit, six: the
+                            * five behind a grouping launch that serves the row-slots of one expert together; the same bytes
+                            * whichever runs; others refused */
     int32_t dec_one;       /* 1 (default): dense decode rows in one launch; 0: the three-launch chain */
     int32_t prefill;       /* 1 (default); 0: routed calls above 16 rows refuse Exl3EngineNotImplemented */
     int32_t mcg_pair;      /* 1 (default): MCG's GEMV feeds the hashed pair to the matrix core unrounded; 0: the f16 weight */

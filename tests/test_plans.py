@@ -152,17 +152,22 @@ def test_decode_forms_by_configuration(lib):
 
 
 def test_decode_form_by_the_gate_up_launch_size(lib):
-    # two launches while the gate|up launch stays within 8192 workgroups (column groups x row-slots x 2 x K slices), five
-    # past that: 4096 x 2048 K4 top-8 has 16 x 8 r x 2 x 8 = 2048 r of them
-    # (past it: the five launches behind a grouping launch, six in all)
-    for rows, launches in ((1, 2), (4, 2), (5, 6), (16, 6)):
+    # two launches while the gate|up launch stays within 8192 workgroups (column groups x row-slots x 2 x K slices); past
+    # that the five launches behind a grouping launch, six in all: 4096 x 2048 K4 top-8 has 16 x 8 r x 2 x 8 = 2048 r
+    for rows, launches in ((1, 2), (3, 2), (5, 6), (16, 6)):
         assert moe_plan(lib, rows, 64, 4096, 2048, 8, 64, 64).launches == launches
     # 7168 x 2048 K3 top-8: 16 x 8 r x 2 x 14 = 3584 r
     assert [moe_plan(lib, rows, 256, 7168, 2048, 8, 48, 48).launches for rows in (1, 2, 3)] == [2, 2, 6]
     # four tiles a load (K5) doubles the column groups: 4096 x 1024 has 16 x 8 r x 2 x 8 = 2048 r as well
-    assert [moe_plan(lib, rows, 64, 4096, 1024, 8, 80, 80).launches for rows in (4, 5)] == [2, 6]
+    assert [moe_plan(lib, rows, 64, 4096, 1024, 8, 80, 80).launches for rows in (3, 5)] == [2, 6]
     # one row of a top-k wide enough to pass the bound has nothing to group: the five launches
     assert moe_plan(lib, 1, 64, 8192, 4096, 32, 64, 64).launches == 5
+    # below the bound the grouped form serves where a uniform routing is expected to save more than ~1400 gate|up
+    # workgroups: 16 experts of 2048 x 1024, top-4, at 16 rows (4096 workgroups, 15.8 groups of 64 row-slots: 3084 saved),
+    # not at 8 (2048, 14.4 of 32: 1126); 64 experts of 4096 x 2048 top-8 at 4 rows (8192, 26.5 of 32: 1412)
+    assert [moe_plan(lib, rows, 16, 2048, 1024, 4, 64, 64).launches for rows in (4, 8, 16)] == [2, 2, 6]
+    assert moe_plan(lib, 4, 64, 4096, 2048, 8, 64, 64).launches == 6
+    assert moe_plan(lib, 16, 128, 2048, 768, 8, 64, 64).launches == 6      # 6144 workgroups, 82 groups of 128: 2200 saved
 
 
 def test_plan_refusals(lib):

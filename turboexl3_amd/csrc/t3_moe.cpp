@@ -222,10 +222,23 @@ int decode_form_of(const MoeLaunch& l) {
     if (want == 5 || want == 6) return kMoeGrouped;
     if (want == 8 || counters * 4u > kCounterBytes) return kMoeFourLaunches;
     const uint64_t gu_groups = static_cast<uint64_t>(l.inter / 16u / l.bt_gu) * rkt * 2u * l.ks_gu;
-    if (gu_groups <= kTwoLaunchGroups) return kMoeTwoLaunches;
     // where the decode dominates, the row-slots that read one expert are served together (a grouping launch in front):
     // every row-slot alone at worst, an expert's tiles decoded once for up to sixteen rows at best
-    return l.rows >= 2u ? kMoeGrouped : kMoeFiveLaunches;
+    if (gu_groups > kTwoLaunchGroups) return l.rows >= 2u ? kMoeGrouped : kMoeFiveLaunches;
+    // Below the bound the six launches cost ~20 us more of chain than the two, and win where grouping removes more decode
+    // than that: by the groups a uniform routing is expected to leave (E (1 - (1 - k / E)^rows) experts hit, one group a
+    // shared slot), gate|up workgroups saved = gu_groups (1 - groups / row-slots). Measured crossover ~1400 (two against
+    // grouped, us: 128 experts of 2048 x 768 top-8 at 16 rows, 2200 saved, 108 / 96; 16 experts of 2048 x 1024 top-4 at 16
+    // rows, 3100 saved, 68 / 49, at 8 rows, 1100 saved, 43 / 43; 512 of 2048 x 512 top-10 + shared at 16 rows, 1200 saved,
+    // 100 / 106). A skewed routing groups better than this estimate.
+    if (l.rows >= 2u) {
+        const double e = static_cast<double>(l.bank.experts), k = static_cast<double>(l.topk);
+        const double hit = e * (1.0 - __builtin_pow(1.0 - (k < e ? k / e : 1.0), static_cast<double>(l.rows)));
+        const double groups = hit + static_cast<double>(l.shared_slots);
+        const double saved = static_cast<double>(gu_groups) * (1.0 - groups / static_cast<double>(rkt));
+        if (saved > 1400.0) return kMoeGrouped;
+    }
+    return kMoeTwoLaunches;
 }
 
 int32_t run_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,

@@ -286,43 +286,90 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ?
 constexpr uint32_t kGroupRows = 16u, kMaxRowSlots = 1024u;  // 16 rows x (top-k + shared slots <= 64)
 
 // One workgroup, 256 threads. Members of a group in ascending row-slot order, groups in the order of their first member;
-// an expert read more than sixteen times starts a new group.
+// an expert read more than sixteen times starts a new group. Three passes over the call's keys in LDS, four keys a read
+// and the reads of a pass independent of one another (a first form with one dependent LDS read a step took 18 us at 128
+// row-slots; this one ~2): a slot's rank among the slots of its key, the leaders before every slot, then each slot's
+// leader and through it the group's index.
 __global__ void __launch_bounds__(256) moe_group(const MoeLaunch a) {
-    __shared__ uint32_t key[kMaxRowSlots], rank[kMaxRowSlots], leaders;
-    const uint32_t rkt = a.rows * (a.topk + a.shared_slots);
+    __shared__ __attribute__((aligned(16))) uint32_t key[kMaxRowSlots];
+    __shared__ __attribute__((aligned(16))) uint32_t aux[kMaxRowSlots];  // rank, bit 31: leads a group
+    __shared__ uint32_t pre[kMaxRowSlots];                               // leaders before the slot
+    constexpr uint32_t kDead = 0xFFFFFFFFu;
+    const uint32_t rkt = a.rows * (a.topk + a.shared_slots), n4 = (rkt + 3u) & ~3u;
     uint32_t* info = a.groups + 1;
     uint32_t* member = a.groups + 1u + 2u * rkt;
-    for (uint32_t rk = threadIdx.x; rk < rkt; rk += 256u) {
-        const SlotRef s = resolve_slot(a, rk);
-        key[rk] = !s.live ? 0xFFFFFFFFu : (s.shared ? 0x80000000u | s.e : s.e);
-    }
-    if (threadIdx.x == 0u) leaders = 0u;
-    __syncthreads();
-    for (uint32_t rk = threadIdx.x; rk < rkt; rk += 256u) {
-        uint32_t r = 0;
-        for (uint32_t j = 0; j < rk; ++j) r += key[j] == key[rk] ? 1u : 0u;
-        rank[rk] = r;
+    for (uint32_t rk = threadIdx.x; rk < n4; rk += 256u) {
+        uint32_t k = kDead;
+        if (rk < rkt) {
+            const SlotRef s = resolve_slot(a, rk);
+            if (s.live) k = s.shared ? 0x80000000u | s.e : s.e;
+        }
+        key[rk] = k;
+        aux[rk] = 0u;
     }
     __syncthreads();
-    for (uint32_t rk = threadIdx.x; rk < rkt; rk += 256u) {
-        if (key[rk] == 0xFFFFFFFFu) continue;
-        const uint32_t first = rank[rk] / kGroupRows * kGroupRows, pos = rank[rk] - first;
+    uint32_t total[4];  // rkt <= 1024: at most four slots a thread
+#pragma unroll
+    for (uint32_t it = 0; it < 4u; ++it) {
+        const uint32_t rk = threadIdx.x + 256u * it;
+        total[it] = 0u;
+        if (rk >= rkt || key[rk] == kDead) continue;
+        const uint32_t mine = key[rk];
+        uint32_t before = 0, all = 0;
+#pragma unroll 8
+        for (uint32_t j = 0; j < n4; j += 4u) {
+            const uint4v k4 = *reinterpret_cast<const uint4v*>(key + j);
+#pragma unroll
+            for (uint32_t c = 0; c < 4u; ++c) {
+                const uint32_t m = k4[c] == mine ? 1u : 0u;
+                all += m;
+                before += j + c < rk ? m : 0u;
+            }
+        }
+        total[it] = all;
+        aux[rk] = before | (before % kGroupRows == 0u ? 0x80000000u : 0u);
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t it = 0; it < 4u; ++it) {
+        const uint32_t rk = threadIdx.x + 256u * it;
+        if (rk >= rkt) continue;
+        uint32_t p = 0;
+#pragma unroll 8
+        for (uint32_t j = 0; j < n4; j += 4u) {
+            const uint4v a4 = *reinterpret_cast<const uint4v*>(aux + j);
+#pragma unroll
+            for (uint32_t c = 0; c < 4u; ++c) p += j + c < rk ? a4[c] >> 31 : 0u;
+        }
+        pre[rk] = p;
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t it = 0; it < 4u; ++it) {
+        const uint32_t rk = threadIdx.x + 256u * it;
+        if (rk >= rkt || key[rk] == kDead) continue;
+        const uint32_t mine = key[rk], rank = aux[rk] & 0x7FFFFFFFu;
+        const uint32_t first = rank / kGroupRows * kGroupRows, pos = rank - first;
         uint32_t leader = rk;
-        for (uint32_t j = 0; j < rk; ++j)
-            if (key[j] == key[rk] && rank[j] == first) leader = j;
-        uint32_t g = 0;
-        for (uint32_t j = 0; j < leader; ++j) g += key[j] != 0xFFFFFFFFu && rank[j] % kGroupRows == 0u ? 1u : 0u;
+        if (pos != 0u) {
+#pragma unroll 8
+            for (uint32_t j = 0; j < n4; j += 4u) {
+                const uint4v k4 = *reinterpret_cast<const uint4v*>(key + j);
+                const uint4v a4 = *reinterpret_cast<const uint4v*>(aux + j);
+#pragma unroll
+                for (uint32_t c = 0; c < 4u; ++c)  // rank `first` of this key leads (one slot of the call at most)
+                    leader = k4[c] == mine && a4[c] == (first | 0x80000000u) ? j + c : leader;
+            }
+        }
+        const uint32_t g = pre[leader];
         member[g * kGroupRows + pos] = rk;
         if (pos == 0u) {
-            uint32_t count = 0;
-            for (uint32_t j = rk; j < rkt; ++j) count += key[j] == key[rk] && rank[j] < first + kGroupRows ? 1u : 0u;
-            info[2u * g] = key[rk];
-            info[2u * g + 1u] = count;
-            atomicAdd(&leaders, 1u);
+            const uint32_t left = total[it] - first;
+            info[2u * g] = mine;
+            info[2u * g + 1u] = left < kGroupRows ? left : kGroupRows;
         }
     }
-    __syncthreads();
-    if (threadIdx.x == 0u) a.groups[0] = leaders;
+    if (threadIdx.x == 0u) a.groups[0] = rkt == 0u ? 0u : pre[rkt - 1u] + (aux[rkt - 1u] >> 31);
 }
 
 template <int BT>
