@@ -288,8 +288,8 @@ constexpr uint32_t kGroupRows = 16u, kMaxRowSlots = 1024u;  // 16 rows x (top-k 
 // One workgroup, 256 threads. Members of a group in ascending row-slot order, groups in the order of their first member;
 // an expert read more than sixteen times starts a new group. Three passes over the call's keys in LDS, four keys a read
 // and the reads of a pass independent of one another (a first form with one dependent LDS read a step took 18 us at 128
-// row-slots; this one 3 to 11 by the row-slots): a slot's rank among the slots of its key, the leaders before every slot, then each slot's
-// leader and through it the group's index.
+// row-slots; this one 3 to 11 by the row-slots): a slot's rank among the slots of its key, the leaders before every slot,
+// then each slot's leader and through it the group's index.
 __global__ void __launch_bounds__(256) moe_group(const MoeLaunch a) {
     __shared__ __attribute__((aligned(16))) uint32_t key[kMaxRowSlots];
     __shared__ __attribute__((aligned(16))) uint32_t aux[kMaxRowSlots];  // rank, bit 31: leads a group
