@@ -115,7 +115,10 @@ typedef struct t3_config {
                             * whichever runs; others refused */
     int32_t dec_one;       /* 1 (default): dense decode rows in one launch; 0: the three-launch chain */
     int32_t prefill;       /* 1 (default); 0: routed calls above 16 rows refuse Exl3EngineNotImplemented */
-    int32_t mcg_pair;      /* 1 (default): MCG's GEMV feeds the hashed pair to the matrix core unrounded; 0: the f16 weight */
+    int32_t mcg_pair;      /* 0 (default): MCG's GEMV multiplies by the format's f16 weight (format.decodeMcg's bits), which holds
+                            * the reference's bars at every shape; 1: it feeds the hashed pair to the matrix core unrounded
+                            * (x lo + x hi in f32: this library's own form, ~5 % faster, inside the bars at the benchmark
+                            * shapes and within 1.5 x of them on small random ones) */
     int32_t mul1_defer;    /* 1 (default): MUL1's affine map applied once an output (src/core/dense.zig deferFor); 0: per weight */
     int32_t dense_gemm_rows; /* dense calls of this many rows or more decode W_hat once into the workspace and run this
                               * library's plain f16 GEMM (K shared out over the grid where its tiles are few), which
@@ -170,14 +173,19 @@ int32_t t3_linear_stages(t3_stream stream, const t3_array* x, const t3_array* tr
  * own their scratch, src/hip/plan.zig:137-146). The scratch `t3_linear` takes as `workspace` lives in a device array of
  * the library itself, T3_STATIC_SCRATCH_BYTES on every GPU the library runs on, held until the process ends; the call
  * allocates nothing, frees nothing and calls no library routine that could. Same kernels, same launches, same bytes
- * as `t3_linear` for the same operands. Refusals before any launch: more than 32 rows: T3_Exl3EngineNotImplemented;
+ * as `t3_linear` for the same operands. Refusals before any launch: more than 32 rows (more than 16 under
+ * t3_config.dense_rows_alone = 1, which sends rows 17..32 to the trellis GEMM): T3_Exl3EngineNotImplemented;
  * a call whose scratch (`t3_linear_workspace_bytes`) exceeds T3_STATIC_SCRATCH_BYTES: T3_WorkspaceTooSmall; else as
  * `t3_linear`. All calls on one GPU share that GPU's array: calls that overlap on one GPU (two streams, two threads)
  * race on it; order them on one stream. The first call on a device looks up the array's address there
- * (hipGetSymbolAddress) and clears its counter head on `stream`: make that call outside graph capture. */
+ * (hipGetSymbolAddress) and clears its counter head on `stream`: make that call outside graph capture. A call that did
+ * not run to its end (a failed launch, a reset stream) may leave arrival counters nonzero in the array, which no caller
+ * can reach: `t3_linear_static_reset` zeroes the head again with one small fill launch on `stream` (it allocates
+ * nothing either), and `t3_linear_static` does the same by itself when one of its own launches reports an error. */
 #define T3_STATIC_SCRATCH_BYTES (16u << 20)
 int32_t t3_linear_static(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
                          const t3_array* svh, t3_decode dec, t3_array* y);
+int32_t t3_linear_static_reset(t3_stream stream);
 
 /* `t3_linear` plus a bias [out] in x's dtype: one add in x's dtype after the projection's own output rounding, so a
  * sum rounds twice (src/root.zig:358-376 `linearBias`). */
@@ -292,8 +300,8 @@ int32_t t3_moe_shared_expert(t3_stream stream, const t3_array* x, const t3_bank*
 /* `t3_moe_shared_expert` (shared_bank NULL: `t3_moe_swiglu` at gate_in; limit 0: no clamp) with a choice of its
  * launches, for profilers and benchmarks that time one stage at a time (the role `t3_linear_stages` has for the dense
  * chain; src/hip/plan.zig:294-364,436-476 publishes the same launches one by one). The workspace carries the stages'
- * results between calls. Up to 16 rows in the two-launch form: bit 0 gate|up + mid, bit 1 down + combine (one and two
- * rows: the mid stage runs inside the down launch; the four- and five-launch forms run whole). Above: bit 0 the route, 1 prepare, 2 gate|up GEMM, 3 mid, 4 down GEMM, 5 combine. */
+ * results between calls. Up to 16 rows in the two-launch form: bit 0 gate|up + mid, bit 1 down + combine (one to four
+ * rows: the mid stage runs inside the down launch, so bit 0 is gate|up alone; the four- and five-launch forms run whole). Above: bit 0 the route, 1 prepare, 2 gate|up GEMM, 3 mid, 4 down GEMM, 5 combine. */
 #define T3_MOE_STAGE_GATE_UP 1u
 #define T3_MOE_STAGE_DOWN 2u
 #define T3_PREFILL_STAGE_ROUTE 1u
@@ -369,7 +377,7 @@ int32_t t3_moe_plan_of(const t3_array* x, const t3_bank* bank, const t3_array* i
  * gate and up round to bf16 and are limited (limit 0: not), the SiLU rounds to bf16, the product rounds to bf16; y F32
  * [B, S, K, D]: each routed slot's own down finish, no score (the host combines a row's slots and its shared expert). A
  * slot whose id is outside [0, E) is skipped and its output left as it is. Any row count: the decode chain up to 16 rows
- * (the launch forms of t3_moe, the same bytes; the exact codebook forms and decode_form 8 take the five launches), the
+ * (the launch forms of t3_moe, the same bytes; MUL1 decoded weight by weight (mul1_defer = 0) and decode_form 8 take the five launches), the
  * prefill chain above. Workspace: t3_moe_workspace_bytes (shared_bank NULL). */
 int32_t t3_moe_glm(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds, t3_decode dec,
                    int32_t limit, t3_array* y, void* workspace, size_t workspace_bytes);
@@ -462,6 +470,11 @@ int32_t t3_test_lane(t3_stream stream, const uint16_t* trellis, int64_t n, int32
 int32_t t3_test_convert(t3_stream stream, const float* in, uint16_t* bf16, uint16_t* f16, float* back, int64_t count);
 /* a f16 [16, 32], b f16 [32, 16] (bits), d f32 [16, 16] = a b through the kernels' MFMA fragments. */
 int32_t t3_test_mfma(t3_stream stream, const uint16_t* a, const uint16_t* b, float* d);
+/* A measurement, not a test: a plain read of `bytes` device bytes (a multiple of 16, 16-byte aligned), 16 bytes a lane,
+ * by `workgroups` workgroups of 256 threads, folded into sink u32 [workgroups * 256]: the read rate the memory system gives
+ * a kernel that does nothing else, which the benchmark states beside the 8 TB/s figure (no counterpart in the reference,
+ * whose bench quotes the vendor's bandwidth, src/core/bench.zig:217). */
+int32_t t3_test_hbm_read(t3_stream stream, const void* src, uint64_t bytes, uint32_t* sink, int32_t workgroups);
 
 #ifdef __cplusplus
 }

@@ -55,7 +55,7 @@ def test_configure_refuses_unserved_values(lib):
     cfg = Config()
     lib.t3_config_default(C.byref(cfg))
     assert (cfg.decode_form, cfg.dec_one, cfg.prefill, cfg.mcg_pair, cfg.mul1_defer, cfg.dense_gemm_rows,
-            cfg.dense_rows_alone) == (9, 1, 1, 1, 1, 513, 0)
+            cfg.dense_rows_alone) == (9, 1, 1, 0, 1, 513, 0)
     # src/core/config.zig:191-192,245: 3, 5, 6, 7, 8 and 9 are served, 0, 4 and 10 refused
     for form in (0, 4, 10):
         cfg.decode_form = form

@@ -122,19 +122,21 @@ def test_dec_one_off_runs_the_chain(oracle, t3):
     assert bytes_of(got) == bytes_of(want)
 
 
-def test_dense_exact_codebook_forms_stay_within_bar(oracle, t3):
-    # the f16-weight forms (mcg_pair off, mul1_defer off) against the same reference
-    t3.configure(mcg_pair=0, mul1_defer=0)
-    try:
-        for codebook in (MCG, MUL1):
-            case = DenseCase(oracle, t3, 77 + codebook, 512, 256, 64, codebook)
-            x_dev, x_f32 = make_x(case.rng, 5, 512, torch.float32)
-            got = to_f32(t3.linear_chain(x_dev, case.d_trellis, case.d_suh, case.d_svh, case.dec))
-            yref = case.ref(x_f32)
-            for r in range(5):
-                assert oracle.compare(got[r], yref[r]) <= F32_BAR
-    finally:
-        t3.configure()
+def test_dense_other_codebook_forms_stay_within_bar(oracle, t3):
+    # the forms beside the served ones against the same reference: every weight the format's f16 value (mul1_defer off),
+    # and MCG's hashed pair fed unrounded (mcg_pair on, this library's opt-in form)
+    for cfg, books in (({"mcg_pair": 0, "mul1_defer": 0}, (MCG, MUL1)), ({"mcg_pair": 1}, (MCG,))):
+        t3.configure(**cfg)
+        try:
+            for codebook in books:
+                case = DenseCase(oracle, t3, 77 + codebook, 512, 256, 64, codebook)
+                x_dev, x_f32 = make_x(case.rng, 5, 512, torch.float32)
+                got = to_f32(t3.linear_chain(x_dev, case.d_trellis, case.d_suh, case.d_svh, case.dec))
+                yref = case.ref(x_f32)
+                for r in range(5):
+                    assert oracle.compare(got[r], yref[r]) <= F32_BAR, (cfg, codebook, r)
+        finally:
+            t3.configure()
 
 
 def test_dense_leading_dims_and_outliers(oracle, t3):

@@ -68,31 +68,37 @@ def test_config2_qkv_shape_rows_1_4_16_32(oracle, t3, k):
         assert bytes_of(y[0]) == bytes_of(alone[0]), "row 0 differs from the row alone"
 
 
-def test_config2_qkv_shape_exact_weight_forms(oracle, t3):
-    # The served GEMV feeds MCG's hashed pair unrounded (mcg_pair) and MUL1's affine map once an output (mul1_defer): both
-    # differ from format.project's f16-rounded weight in the last bits of a product, the second as the reference's own
-    # kernels do (src/kernels/hip/common.hpp:95-104), the first this library's own form. With both switched off every
-    # weight is the format's f16 value: the q|k|v shape at K4, rows 1 and 32, both codebooks, held to the same bar, and the
-    # one launch still equal to its chain.
+def test_config2_qkv_shape_codebook_forms(oracle, t3):
+    # The GEMV's other codebook forms at the q|k|v shape, K4, rows 1 and 32, held to the same bar, the one launch still
+    # equal to its chain. Served by default: MCG as the format's f16 weight, MUL1's affine map applied once an output
+    # (mul1_defer, the reference's own kernels' form, src/kernels/hip/common.hpp:95-104). Here: every weight the format's
+    # f16 value for both codebooks (mul1_defer off), and MCG's hashed pair fed unrounded (mcg_pair on: this library's own
+    # opt-in form, which differs from format.project's rounded weight in the last bits of a product).
     in_f, out_f, n = 4096, 12288, 64
     rng = np.random.default_rng(0xC2E)
     trellis, suh, svh = oracle.synth_linear(rng, in_f, out_f, n)
     d_t, d_suh, d_svh = dev_u16(trellis), dev_f16_bits(suh), dev_f16_bits(svh)
     x_dev, x_f32 = make_x(rng, 32, in_f, torch.float16, outliers=True)
-    t3.configure(mcg_pair=0, mul1_defer=0)
-    try:
-        for codebook, dec in ((MCG, t3.Decode.mcg), (MUL1, t3.Decode.mul1)):
-            w_hat = oracle.reconstruct_inner(trellis, in_f, out_f, n, codebook)
-            ref = oracle.project_rows(x_f32, trellis, suh, svh, in_f, out_f, n, codebook, 0xFFFF, threads=8, w_hat=w_hat)
-            for rows in (1, 32):
-                y = t3.linear(x_dev[:rows], d_t, d_suh, d_svh, dec)
-                got = to_f32(y)
-                worst = max(oracle.compare(got[r], ref[r], 2.0 ** -11) for r in range(rows))
-                assert worst <= F32_BAR, f"codebook {codebook} rows {rows}: {worst:.3e}"
-                if rows == 1:
-                    assert bytes_of(y) == bytes_of(t3.linear_chain(x_dev[:1], d_t, d_suh, d_svh, dec))
-    finally:
-        t3.configure()
+    refs = {}
+    for cfg, books in (({"mcg_pair": 0, "mul1_defer": 0}, ((MCG, t3.Decode.mcg), (MUL1, t3.Decode.mul1))),
+                       ({"mcg_pair": 1}, ((MCG, t3.Decode.mcg),))):
+        t3.configure(**cfg)
+        try:
+            for codebook, dec in books:
+                if codebook not in refs:
+                    w_hat = oracle.reconstruct_inner(trellis, in_f, out_f, n, codebook)
+                    refs[codebook] = oracle.project_rows(x_f32, trellis, suh, svh, in_f, out_f, n, codebook, 0xFFFF,
+                                                         threads=8, w_hat=w_hat)
+                ref = refs[codebook]
+                for rows in (1, 32):
+                    y = t3.linear(x_dev[:rows], d_t, d_suh, d_svh, dec)
+                    got = to_f32(y)
+                    worst = max(oracle.compare(got[r], ref[r], 2.0 ** -11) for r in range(rows))
+                    assert worst <= F32_BAR, f"{cfg} codebook {codebook} rows {rows}: {worst:.3e}"
+                    if rows == 1:
+                        assert bytes_of(y) == bytes_of(t3.linear_chain(x_dev[:1], d_t, d_suh, d_svh, dec))
+        finally:
+            t3.configure()
 
 
 def test_config5_lm_head_k6_rows_1_and_256(oracle, t3):
@@ -246,6 +252,55 @@ def test_config3_routed_decode_with_shared_expert(oracle, t3):
             first = bytes_of(y[0, 0])
         else:
             assert bytes_of(y[0, 0]) == first, "row 0 of 8 tokens differs from the row alone"
+
+
+def test_reference_workload_widths_2560_by_640(oracle, t3):
+    # The reference's own published workload (docs/models/qwen38/results.md:278-284): hidden 2560, expert width 640, top-10,
+    # bf16, MUL1: 160 and 40 input tile rows, a K partition none of the benchmark configurations has (twenty 128-blocks of
+    # the hidden width in five K slices, five of the expert width in two). On 24 of its 512 experts so the CPU side stays
+    # small: the decode chain at 1 and 4 rows and the prefill chain at 40 rows against ref.moeRow, a row's bytes those of
+    # the row alone, the launch forms equal; and one dense projection of the same widths.
+    experts, hidden, inter, n, topk = 24, 2560, 640, 64, 10
+    rng = np.random.default_rng(0x2560)
+    bank = oracle.synth_bank(rng, experts, hidden, inter, n)
+    dbank = dev_bank(t3, bank)
+    ref = RefBank(oracle, bank, MUL1, 0xFFFF)
+    x_dev, x_f32 = make_x(rng, 40, hidden, torch.bfloat16)
+    slots, scores = routing_softmax(rng, 40, topk, experts)
+    d_slots, d_scores = torch.from_numpy(slots).cuda(), torch.from_numpy(scores).cuda()
+    plan = t3.moe_plan(x_dev[:1].reshape(1, 1, hidden), dbank, d_slots[:1].reshape(1, 1, topk))
+    assert (plan["k_slices_gu"], plan["k_slices_dn"]) == (5, 2), plan
+    call = lambda rows: t3.moe(x_dev[:rows].reshape(1, rows, hidden), dbank, d_slots[:rows].reshape(1, rows, topk),
+                               d_scores[:rows].reshape(1, rows, topk), t3.Decode.mul1)
+    want = [ref.row(x_f32[r], slots[r], scores[r], 0.0) for r in (0, 1, 2, 3, 39)]
+    alone = call(1)
+    for rows in (1, 4, 40):
+        y = call(rows)
+        got = to_f32(y).reshape(rows, hidden)
+        for i, r in enumerate((0, 1, 2, 3, 39)):
+            if r < rows:
+                e = oracle.compare(got[r], want[i], 2.0 ** -8)
+                assert e <= BF16_MOE_BAR, f"{rows} rows row {r}: {e:.3e}"
+        if rows <= 16:
+            assert bytes_of(y[0, 0]) == bytes_of(alone[0, 0]), "row 0 differs from the row alone"
+            for form in (3, 8):
+                t3.configure(decode_form=form)
+                try:
+                    assert bytes_of(call(rows)) == bytes_of(y), f"form {form} differs at {rows} rows"
+                finally:
+                    t3.configure()
+    # dense, the same widths both ways (the partition of a small matrix: four tiles a load)
+    for in_f, out_f in ((2560, 640), (640, 2560)):
+        trellis, suh, svh = oracle.synth_linear(rng, in_f, out_f, n)
+        d_t, d_suh, d_svh = dev_u16(trellis), dev_f16_bits(suh), dev_f16_bits(svh)
+        xd_dev, xd_f32 = make_x(rng, 4, in_f, torch.bfloat16)
+        yref = oracle.project_rows(xd_f32, trellis, suh, svh, in_f, out_f, n, MUL1, 0xFFFF, threads=8)
+        for rows in (1, 4):
+            y = t3.linear(xd_dev[:rows], d_t, d_suh, d_svh, t3.Decode.mul1)
+            assert bytes_of(y) == bytes_of(t3.linear_chain(xd_dev[:rows], d_t, d_suh, d_svh, t3.Decode.mul1))
+            got = to_f32(y)
+            for r in range(rows):
+                assert oracle.compare(got[r], yref[r], 2.0 ** -8) <= BF16_DENSE_BAR, (in_f, rows, r)
 
 
 def test_config4_routed_prefill_widths_mixed_rates(oracle, t3):

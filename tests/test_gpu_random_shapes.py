@@ -170,49 +170,54 @@ class UnroundedBank(RefBank):
 
 
 # Draws of a wider walk (500 seeds of each kind) where some row of a call sat at or over the reference's bar against
-# format.project's chain: ten draws, each a few rows of one or two row counts, none above 1.4 x the bar. Two things
-# put a row there, and the tests below hold each draw to the statement that is true of it.
-#   The served weights. The GEMV feeds MUL1 as the deferred map A h + B and MCG as its hashed pair, both unrounded, where
-#   format.project rounds every weight to f16; the deferred map is the reference's own choice for its kernels
-#   (src/core/decode.zig:346, src/kernels/hip/common.hpp:95-104), held there to the same bars at its own shapes
-#   (src/hip_tests.zig:450-458,483), the pair form is this library's. Half an f16 step a weight moves z by ~1.4e-4 of its
-#   size, which flips the f16 rounding of a fifth of z's values, and those flips are what the measure sees. On every row:
-#   the exact forms (mcg_pair = 0, mul1_defer = 0) within the bars of format.project's chain; the served forms within the
+# format.project's chain while the GEMV fed both codebooks unrounded: ten draws, each a few rows of one or two row counts,
+# none above 1.4 x the bar. Two things put a row there, and the tests below hold each draw to the statement that is true
+# of it.
+#   Unrounded weights. The GEMV feeds MUL1 as the deferred map A h + B (served: the reference's own choice for its
+#   kernels, src/core/decode.zig:346, src/kernels/hip/common.hpp:95-104, held there to the same bars at its own shapes,
+#   src/hip_tests.zig:450-458,483) and, where t3_config.mcg_pair is set (not by default), MCG as its hashed pair, where
+#   format.project rounds every weight to f16. Half an f16 step a weight moves z by ~1.4e-4 of its size, which flips the
+#   f16 rounding of a fifth of z's values, and those flips are what the measure sees. On every row: the f16-weight forms
+#   (MCG as served; MUL1 with mul1_defer = 0) within the bars of format.project's chain; the unrounded forms within the
 #   bars of the same chain with unrounded weights (what the forms define), and within 1.5 x the bars of format.project's.
 #   The result's own resolution. y is an f16 value (format.project's last statement rounds it), one f16 step of an
 #   element above 5.1 x the row's rms is more than 5e-3 of that rms, and a chain with three f16 rounding points flips a
 #   step wherever a sum lands within an f32 rounding of a tie. The dense draws hold every element within the bar or one
-#   f16 step of the oracle's value, with the exact weights of the W_hat form as well as with the served ones.
+#   f16 step of the oracle's value, with the exact weights of the W_hat form as well as with the unrounded ones.
 DEFERRED_SLACK = 1.5
 ROUTED_AT_THE_BAR = [11, 59, 66, 83, 305, 335, 405]
 DENSE_AT_THE_BAR = [117, 122, 445]
 
 
 @pytest.mark.parametrize("seed", ROUTED_AT_THE_BAR)
-def test_routed_draws_where_the_served_weights_sit_at_the_bar(oracle, t3, seed):
+def test_routed_draws_where_unrounded_weights_sit_at_the_bar(oracle, t3, seed):
     d = routed_draw(oracle, t3, seed)
     mask = (1 << d["wbits"]) - 1
     exact, unrounded = RefBank(oracle, d["bank"], d["codebook"], mask), UnroundedBank(oracle, d["bank"], d["codebook"], mask)
     bar, half = MOE_BARS[d["dtype"]], HALF_ULP[d["dtype"]]
     most = d["row_counts"][-1]
+    mcg = d["codebook"] == 1
     want = [exact.row(d["x_f32"][r], d["slots"][r], d["scores"][r], float(d["limit"])) for r in range(most)]
     want_unr = [unrounded.row(d["x_f32"][r], d["slots"][r], d["scores"][r], float(d["limit"])) for r in range(most)]
     for rows in d["row_counts"]:
         served = run_routed(t3, d, rows)
-        t3.configure(mcg_pair=0, mul1_defer=0)
+        # the other form of the draw's codebook: MUL1 decoded weight by weight, MCG's pair fed unrounded
+        t3.configure(**({"mcg_pair": 1} if mcg else {"mul1_defer": 0}))
         try:
-            exact_form = run_routed(t3, d, rows)
+            other = run_routed(t3, d, rows)
         finally:
             t3.configure()
-        # above 16 rows the prefill chain decodes MCG to the format's f16 weights; MUL1 keeps the deferred map there
-        unrounded_served = d["codebook"] == 0 or rows <= 16
+        exact_form, loose_form = (served, other) if mcg else (other, served)
+        # above 16 rows the prefill chain decodes MCG to the format's f16 weights whatever mcg_pair says; MUL1 keeps
+        # the deferred map there
+        loose_is_unrounded = (not mcg) or rows <= 16
         for r in range(rows):
             e = oracle.compare(exact_form[r], want[r], half)
-            assert e <= bar, f"exact form, {d['what']} rows {rows} row {r}: {e:.3e}"
-            e = oracle.compare(served[r], (want_unr if unrounded_served else want)[r], half)
-            assert e <= bar, f"served form against the chain with its own weights, {d['what']} rows {rows} row {r}: {e:.3e}"
-            e = oracle.compare(served[r], want[r], half)
-            assert e <= DEFERRED_SLACK * bar, f"served form against format.project, {d['what']} rows {rows} row {r}: {e:.3e}"
+            assert e <= bar, f"f16 weights, {d['what']} rows {rows} row {r}: {e:.3e}"
+            e = oracle.compare(loose_form[r], (want_unr if loose_is_unrounded else want)[r], half)
+            assert e <= bar, f"unrounded form against the chain with its own weights, {d['what']} rows {rows} row {r}: {e:.3e}"
+            e = oracle.compare(loose_form[r], want[r], half)
+            assert e <= DEFERRED_SLACK * bar, f"unrounded form against format.project, {d['what']} rows {rows} row {r}: {e:.3e}"
 
 
 @pytest.mark.parametrize("seed", DENSE_AT_THE_BAR)
@@ -224,7 +229,7 @@ def test_dense_draws_where_one_f16_step_passes_the_bar(oracle, t3, seed):
     rms = np.sqrt((ref.astype(np.float64) ** 2).mean(axis=1, keepdims=True))
     step = np.spacing(np.maximum(np.abs(ref), np.float32(2.0 ** -14)).astype(np.float16)).astype(np.float64)
     for rows in d["row_counts"]:
-        for form in ({}, {"mcg_pair": 0, "mul1_defer": 0}, {"dense_gemm_rows": 0}):
+        for form in ({}, {"mcg_pair": 1}, {"mul1_defer": 0}, {"dense_gemm_rows": 0}):
             t3.configure(**form)
             try:
                 got = to_f32(run_dense(t3, d, rows))

@@ -54,6 +54,20 @@ def test_static_scratch_rows_and_forms(oracle, t3):
         for dec in (t3.Decode.mcg, t3.Decode.mul1):
             y = t3.linear_static(x_dev[:rows], *ops[3:], dec)
             assert bytes_of(y) == bytes_of(t3.linear(x_dev[:rows], *ops[3:], dec)), (rows, dec)
+    # the reset (what a caller runs after a call that did not reach its end) leaves a working array behind
+    t3.linear_static_reset()
+    y = t3.linear_static(x_dev[:3], *ops[3:], t3.Decode.mcg)
+    assert bytes_of(y) == bytes_of(t3.linear(x_dev[:3], *ops[3:], t3.Decode.mcg))
+    # rows 17..32 leave the GEMV under dense_rows_alone: the entry point refuses them then
+    t3.configure(dense_rows_alone=1)
+    try:
+        with pytest.raises(t3.T3Error) as err:
+            t3.linear_static(x_dev[:17], *ops[3:], t3.Decode.mcg)
+        assert err.value.name == "Exl3EngineNotImplemented"
+        y = t3.linear_static(x_dev[:16], *ops[3:], t3.Decode.mcg)
+        assert bytes_of(y) == bytes_of(t3.linear(x_dev[:16], *ops[3:], t3.Decode.mcg))
+    finally:
+        t3.configure()
 
 
 def test_static_scratch_refusals_and_no_allocation(oracle, t3):

@@ -84,6 +84,7 @@ SYMBOLS = {
     "t3_release_engines": (None, []),
     "t3_linear": (C.c_int32, [C.c_void_p, _AP, _AP, _AP, _AP, Decode, _AP, C.c_void_p, C.c_size_t]),
     "t3_linear_static": (C.c_int32, [C.c_void_p, _AP, _AP, _AP, _AP, Decode, _AP]),
+    "t3_linear_static_reset": (C.c_int32, [C.c_void_p]),
     "t3_linear_workspace_bytes": (C.c_int32, [_AP, _AP, Decode, C.POINTER(C.c_size_t)]),
     "t3_linear_plan_of": (C.c_int32, [_AP, _AP, Decode, C.POINTER(LinearPlan)]),
     "t3_moe_plan_of": (C.c_int32, [_AP, _BP, _AP, _BP, C.POINTER(MoePlan)]),
@@ -136,6 +137,7 @@ SYMBOLS = {
                                  C.c_void_p]),
     "t3_test_convert": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64]),
     "t3_test_mfma": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "t3_test_hbm_read": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_uint64, C.c_void_p, C.c_int32]),
 }
 
 _lib = None

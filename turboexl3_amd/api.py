@@ -174,6 +174,11 @@ def linear_static(x, trellis, suh, svh, dec: Decode = Decode.mul1, stream=None, 
     return y
 
 
+def linear_static_reset(stream=None) -> None:
+    """Zero the counter head of the library's own scratch array again (after a call that did not run to its end)."""
+    _check(_lib.lib().t3_linear_static_reset(_stream_ptr(stream)))
+
+
 def linear_chain(x, trellis, suh, svh, dec: Decode = Decode.mul1, stream=None) -> torch.Tensor:
     """The three-launch chain `linear`'s fused launch must equal byte for byte."""
     return _linear(_lib.lib().t3_linear_chain, x, trellis, suh, svh, dec, stream)

@@ -12,22 +12,37 @@
 
 namespace {
 
-// The configuration a call reads is one whole snapshot, also while another thread configures: t3_configure writes the
-// next slot of a small ring and then publishes its index; a reader takes whichever snapshot is published when it asks.
-// (The reference sets its configuration once before the first call, src/core/config.zig:175-178; a slot is reused only
-// after 63 further t3_configure calls, by which time no call that started under it is still reading.)
+// t3_configure writes the next slot of a small ring and then publishes its index, so a reader copies a whole snapshot
+// also while another thread configures (a slot is reused only after 63 further t3_configure calls). An entry point
+// copies the published snapshot ONCE, into its thread's own storage (ConfigScope), and everything it calls reads that
+// copy: a call's checks, workspace carving and launches all see the same settings whatever another thread configures
+// meanwhile. (The reference sets its configuration once before the first call, src/core/config.zig:175-178.)
 constexpr uint32_t kConfigSlots = 64;
 // what a process that never configures runs with, and what t3_config_default hands out
-constexpr t3_config kDefaultConfig = {9, 1, 1, 1, 1, 513, 0};
+constexpr t3_config kDefaultConfig = {9, 1, 1, 0, 1, 513, 0};
 t3_config g_configs[kConfigSlots] = {kDefaultConfig};
 std::atomic<uint32_t> g_config_at{0};
 std::mutex g_config_write;
+
+thread_local t3_config tl_config = kDefaultConfig;
+thread_local int tl_config_depth = 0;
+
+t3_config published_config() { return g_configs[g_config_at.load(std::memory_order_acquire) % kConfigSlots]; }
 
 }  // namespace
 
 namespace t3 {
 
-const t3_config& config() { return g_configs[g_config_at.load(std::memory_order_acquire) % kConfigSlots]; }
+// the calling entry point's snapshot; outside any entry point (a helper called on its own), what is published now
+const t3_config& config() {
+    if (tl_config_depth == 0) tl_config = published_config();
+    return tl_config;
+}
+
+ConfigScope::ConfigScope() {
+    if (tl_config_depth++ == 0) tl_config = published_config();
+}
+ConfigScope::~ConfigScope() { --tl_config_depth; }
 
 }  // namespace t3
 
@@ -118,6 +133,15 @@ int32_t t3_test_convert(t3_stream stream, const float* in, uint16_t* bf16, uint1
     if (count <= 0 || count > (1 << 28)) return T3_BadExl3Shape;
     return t3::hip_status(t3::launch_test_convert(in, bf16, f16, back, static_cast<uint32_t>(count),
                                                   static_cast<hipStream_t>(stream)));
+}
+
+int32_t t3_test_hbm_read(t3_stream stream, const void* src, uint64_t bytes, uint32_t* sink, int32_t workgroups) {
+    if (!src || !sink) return T3_BadArgs;
+    if (bytes == 0 || bytes % 16u != 0u || (reinterpret_cast<uintptr_t>(src) & 15u) != 0u || workgroups <= 0 ||
+        workgroups > (1 << 20))
+        return T3_BadExl3Shape;
+    return t3::hip_status(t3::launch_test_hbm_read(src, bytes, sink, static_cast<uint32_t>(workgroups),
+                                                   static_cast<hipStream_t>(stream)));
 }
 
 int32_t t3_test_mfma(t3_stream stream, const uint16_t* a, const uint16_t* b, float* d) {

@@ -149,4 +149,31 @@ hipError_t launch_test_mfma(const uint16_t* a, const uint16_t* b, float* d, hipS
     return hipGetLastError();
 }
 
+namespace {
+// A plain read of `pieces` 16-byte pieces, one a lane a step, the steps of a workgroup 256 pieces apart and the
+// workgroups interleaved (piece = (step * grid + workgroup) * 256 + thread): what the memory system gives a kernel that
+// does nothing with its bytes but fold them. Every lane's fold is stored, so no load can be dropped. Grid (wgs), 256
+// threads; eight loads in flight a lane.
+__global__ void __launch_bounds__(256) test_hbm_read_kernel(const uint4v* src, uint64_t pieces, uint32_t* sink) {
+    const uint64_t stride = static_cast<uint64_t>(gridDim.x) * 256u;
+    uint64_t i = static_cast<uint64_t>(blockIdx.x) * 256u + threadIdx.x;
+    uint4v acc = {0u, 0u, 0u, 0u};
+    for (; i + 7u * stride < pieces; i += 8u * stride) {
+        uint4v v[8];
+#pragma unroll
+        for (uint32_t j = 0; j < 8u; ++j) v[j] = src[i + j * stride];
+#pragma unroll
+        for (uint32_t j = 0; j < 8u; ++j) acc ^= v[j];
+    }
+    for (; i < pieces; i += stride) acc ^= src[i];
+    sink[blockIdx.x * 256u + threadIdx.x] = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+}
+}  // namespace
+
+hipError_t launch_test_hbm_read(const void* src, uint64_t bytes, uint32_t* sink, uint32_t workgroups, hipStream_t s) {
+    hipLaunchKernelGGL(test_hbm_read_kernel, dim3(workgroups), dim3(256), 0, s, static_cast<const uint4v*>(src), bytes / 16u,
+                       sink);
+    return hipGetLastError();
+}
+
 }  // namespace t3

@@ -55,6 +55,8 @@ struct GemmArgs {
     const uint16_t* svh;  // FINISH: the output scale vector f16 [cols]
     int dt;               // FINISH: y's dtype (t3::Dtype); else y is in the operands' dtype
     uint32_t rows, in, cols, ldw, mt;
+    uint32_t wcol0;       // w's first column inside its [in][ldw] array (a member of a joined weight): the array's end,
+                          // past which loads bring zeros, lies in * ldw - wcol0 elements from w
     uint32_t ntf, nth;    // column blocks of 256, then of 128
     float* planes;        // PLANES: f32 [K parts][rows][cols], part blockIdx.z's sums
     uint32_t part_steps;  // PLANES: K = 32 steps a part
@@ -70,12 +72,17 @@ __device__ __forceinline__ uint4v gemm_rsrc(const void* p, uint64_t bytes) {
     const uint32_t n = bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : static_cast<uint32_t>(bytes);
     return uint4v{static_cast<uint32_t>(addr), static_cast<uint32_t>(addr >> 32) & 0xFFFFu, n, 0x00020000u};
 }
+// (m0 is named as clobbered so the compiler keeps nothing of its own in it across the statement; clang warns about any
+// reserved register in a clobber list, which is the point here)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void gemm_load_to_lds(uint4v desc, uint32_t lds, uint32_t voff, uint32_t soff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :
                  : "s"(lds), "v"(voff), "s"(desc), "s"(soff)
-                 : "memory");
+                 : "memory", "m0");
 }
+#pragma clang diagnostic pop
 template <int N>
 __device__ __forceinline__ void gemm_wait_loads() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
@@ -110,7 +117,7 @@ __global__ void __launch_bounds__(512) gemm_half(const GemmArgs a) {
     const uint4v xdesc = gemm_rsrc(static_cast<const unsigned char*>(a.x) + static_cast<size_t>(row0) * a.in * 2u,
                                    static_cast<uint64_t>(rows_here) * a.in * 2u);
     const uint4v wdesc = gemm_rsrc(static_cast<const unsigned char*>(a.w) + static_cast<size_t>(col0) * 2u,
-                                   (static_cast<uint64_t>(a.in) * a.ldw - col0) * 2u);
+                                   (static_cast<uint64_t>(a.in) * a.ldw - a.wcol0 - col0) * 2u);
     // this wave's loads a step: x rows 32 wave .. + 31 (two loads of 16 rows), w rows k = 4 wave .. + 3 (two of 2 rows;
     // a 128-column tile loads 256 columns all the same and leaves the second half alone)
     uint32_t x_voff[2], w_voff[2];
@@ -266,10 +273,12 @@ __global__ void __launch_bounds__(512) gemm_half(const GemmArgs a) {
 namespace {
 // The launch's column blocks. Every block 256 wide, except that a launch whose last round of workgroups (one a compute
 // unit) would fill at most half the GPU cuts that round's column blocks in two: twice the workgroups, half as long.
-GemmArgs gemm_args(const void* x, const void* w, void* y, uint32_t rows, uint32_t in, uint32_t cols, uint32_t ldw) {
+GemmArgs gemm_args(const void* x, const void* w, void* y, uint32_t rows, uint32_t in, uint32_t cols, uint32_t ldw,
+                   uint32_t wcol0) {
     GemmArgs a{};
     a.x = x;
-    a.w = w;
+    a.w = static_cast<const unsigned char*>(w) + static_cast<size_t>(wcol0) * 2u;
+    a.wcol0 = wcol0;
     a.y = y;
     a.rows = rows;
     a.in = in;
@@ -292,11 +301,12 @@ GemmArgs gemm_args(const void* x, const void* w, void* y, uint32_t rows, uint32_
 dim3 gemm_grid(const GemmArgs& a) { return dim3(8u * a.mt, (a.ntf + 7u) / 8u + (a.nth + 7u) / 8u); }
 }  // namespace
 
-// y [rows][cols] = x [rows][in] w[:, 0:cols] for w [in][ldw] (all f16 or all bf16; y row-contiguous). The host has
-// checked: in a multiple of 32, ldw a multiple of 8, w and x 16-byte aligned, in ldw 2 bytes under 4 GiB.
+// y [rows][cols] = x [rows][in] w[:, wcol0 : wcol0 + cols] for w [in][ldw] (all f16 or all bf16; y row-contiguous). The
+// host has checked: in a multiple of 32, ldw and wcol0 multiples of 8, wcol0 + cols within ldw, w and x 16-byte aligned,
+// in ldw 2 bytes under 4 GiB. A tile loads 256 columns whatever `cols`: what lies past w's last element reads as zeros.
 hipError_t launch_gemm_half(const void* x, const void* w, void* y, uint32_t rows, uint32_t in, uint32_t cols, uint32_t ldw,
-                            bool bf16, hipStream_t s) {
-    const GemmArgs a = gemm_args(x, w, y, rows, in, cols, ldw);
+                            uint32_t wcol0, bool bf16, hipStream_t s) {
+    const GemmArgs a = gemm_args(x, w, y, rows, in, cols, ldw, wcol0);
     const dim3 grid = gemm_grid(a), block(512);
     if (bf16) hipLaunchKernelGGL((gemm_half<true, kGemmPlain>), grid, block, 0, s, a);
     else hipLaunchKernelGGL((gemm_half<false, kGemmPlain>), grid, block, 0, s, a);
@@ -307,7 +317,7 @@ hipError_t launch_gemm_half(const void* x, const void* w, void* y, uint32_t rows
 // launch (xp: the prepared rows, f16 in natural order; out a multiple of 128)
 hipError_t launch_gemm_finish(const uint16_t* xp, const uint16_t* w_hat, const uint16_t* svh, void* y, uint32_t rows,
                               uint32_t in, uint32_t out, int dtype, hipStream_t s) {
-    GemmArgs a = gemm_args(xp, w_hat, y, rows, in, out, out);
+    GemmArgs a = gemm_args(xp, w_hat, y, rows, in, out, out, 0u);
     a.svh = svh;
     a.dt = dtype;
     const dim3 grid = gemm_grid(a), block(512);
@@ -318,8 +328,8 @@ hipError_t launch_gemm_finish(const uint16_t* xp, const uint16_t* w_hat, const u
 // planes f32 [kparts][rows][cols]: part p = the sums over K steps [p part_steps, (p + 1) part_steps) of x w[:, 0:cols]
 // (cols a multiple of 4, planes 16-byte aligned); kparts from gemm_kparts
 hipError_t launch_gemm_planes(const void* x, const void* w, float* planes, uint32_t rows, uint32_t in, uint32_t cols,
-                              uint32_t ldw, bool bf16, uint32_t kparts, hipStream_t s) {
-    GemmArgs a = gemm_args(x, w, nullptr, rows, in, cols, ldw);
+                              uint32_t ldw, uint32_t wcol0, bool bf16, uint32_t kparts, hipStream_t s) {
+    GemmArgs a = gemm_args(x, w, nullptr, rows, in, cols, ldw, wcol0);
     if (a.nth != 0u || kparts == 0u || (in / kGK) % kparts != 0u || cols % 4u != 0u) return hipErrorInvalidValue;
     a.planes = planes;
     a.part_steps = (in / kGK) / kparts;

@@ -10,7 +10,15 @@
 
 namespace t3 {
 
+// The configuration the current call runs with. An entry point opens a ConfigScope first: the published configuration is
+// copied once into the thread's own storage and every config() below it, however deep, reads that one copy.
 const t3_config& config();
+struct ConfigScope {
+    ConfigScope();
+    ~ConfigScope();
+    ConfigScope(const ConfigScope&) = delete;
+    ConfigScope& operator=(const ConfigScope&) = delete;
+};
 
 inline bool rate_ok(int64_t n) { return n % 2 == 0 && n >= 16 && n <= 128; }
 

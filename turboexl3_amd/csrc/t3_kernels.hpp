@@ -170,11 +170,11 @@ inline uint32_t dense_prefill_workgroups(uint32_t out, uint32_t items) { return 
 // The W_hat form's own prepare: natural order (plain f16 [rows][in], what a plain GEMM multiplies).
 hipError_t launch_dense_prep_natural(const DenseLaunch& d, uint16_t* xp, hipStream_t s);
 
-// The plain half-precision GEMM on the matrix cores (t3_gemm.hip): y [rows][cols] = x [rows][in] w[:, 0:cols] for
-// w [in][ldw], all f16 or all bf16, f32 accumulation, y row-contiguous. in a multiple of 32, ldw of 8, x and w 16-byte
-// aligned, in * ldw * 2 under 4 GiB (gemm_half_ok).
+// The plain half-precision GEMM on the matrix cores (t3_gemm.hip): y [rows][cols] = x [rows][in] w[:, wcol0 : wcol0 + cols]
+// for w [in][ldw] (the whole array: the kernel bounds its loads by the array's end), all f16 or all bf16, f32 accumulation,
+// y row-contiguous. in a multiple of 32, ldw and wcol0 of 8, x and w 16-byte aligned, in * ldw * 2 under 4 GiB (gemm_half_ok).
 hipError_t launch_gemm_half(const void* x, const void* w, void* y, uint32_t rows, uint32_t in, uint32_t cols, uint32_t ldw,
-                            bool bf16, hipStream_t s);
+                            uint32_t wcol0, bool bf16, hipStream_t s);
 // the same product over a W_hat with format.finishOutput at its end: y [rows][out] in `dtype` from the prepared rows
 hipError_t launch_gemm_finish(const uint16_t* xp, const uint16_t* w_hat, const uint16_t* svh, void* y, uint32_t rows,
                               uint32_t in, uint32_t out, int dtype, hipStream_t s);
@@ -182,7 +182,7 @@ hipError_t launch_gemm_finish(const uint16_t* xp, const uint16_t* w_hat, const u
 // planes summed in part order (the trellis GEMM's finish launch). A 256 x 256 tile a workgroup over the whole K leaves a
 // call of few rows on a handful of compute units; K parts fill them.
 hipError_t launch_gemm_planes(const void* x, const void* w, float* planes, uint32_t rows, uint32_t in, uint32_t cols,
-                              uint32_t ldw, bool bf16, uint32_t kparts, hipStream_t s);
+                              uint32_t ldw, uint32_t wcol0, bool bf16, uint32_t kparts, hipStream_t s);
 // the plain product's end over K parts: y [rows][cols] (f16 or bf16) = the planes summed in part order, one rounding
 hipError_t launch_gemm_planes_round(const float* planes, void* y, uint32_t rows, uint32_t cols, uint32_t kparts, bool bf16,
                                     hipStream_t s);
@@ -221,5 +221,7 @@ hipError_t launch_test_lane(const uint32_t* trellis, uint32_t n, uint32_t wbits,
 hipError_t launch_test_convert(const float* in, uint16_t* bf16, uint16_t* f16, float* back, uint32_t count, hipStream_t s);
 // test kernel: D = A B through the GEMV's MFMA with the fragments the kernels assume
 hipError_t launch_test_mfma(const uint16_t* a, const uint16_t* b, float* d, hipStream_t s);
+// measurement kernel: a plain 16-byte-a-lane read of `bytes` bytes (a multiple of 16) folded into sink [workgroups * 256]
+hipError_t launch_test_hbm_read(const void* src, uint64_t bytes, uint32_t* sink, uint32_t workgroups, hipStream_t s);
 
 }  // namespace t3

@@ -143,7 +143,7 @@ int32_t run_over_w_hat(const DenseLaunch& l, const uint16_t* w_hat, uint16_t* xp
     const uint32_t k = gemm_kparts(l.rows, l.in, l.out);
     if (k == 1u) return hip_status(launch_gemm_finish(xp, w_hat, l.svh, l.y, l.rows, l.in, l.out, l.dtype, s));
     if (!planes) return T3_BadArgs;
-    if (const int32_t st = hip_status(launch_gemm_planes(xp, w_hat, planes, l.rows, l.in, l.out, l.out, false, k, s));
+    if (const int32_t st = hip_status(launch_gemm_planes(xp, w_hat, planes, l.rows, l.in, l.out, l.out, 0u, false, k, s));
         st != T3_OK)
         return st;
     return hip_status(launch_dense_planes_finish(l, planes, k, s));
@@ -252,6 +252,7 @@ int32_t run_fused(const DenseCall& call, hipStream_t s) {
 extern "C" {
 
 int32_t t3_linear_workspace_bytes(const t3_array* x, const t3_array* trellis, t3_decode dec, size_t* bytes) {
+    const t3::ConfigScope one_config;
     if (!bytes) return T3_BadArgs;
     t3::DenseCall call;
     if (const int32_t st = t3::check_dense(x, trellis, nullptr, nullptr, dec, nullptr, 0, &call); st != T3_OK) return st;
@@ -263,6 +264,7 @@ int32_t t3_linear_workspace_bytes(const t3_array* x, const t3_array* trellis, t3
 }
 
 int32_t t3_linear_plan_of(const t3_array* x, const t3_array* trellis, t3_decode dec, t3_linear_plan* plan) {
+    const t3::ConfigScope one_config;
     if (!plan) return T3_BadArgs;
     t3::DenseCall call;
     if (const int32_t st = t3::check_dense(x, trellis, nullptr, nullptr, dec, nullptr, 0, &call); st != T3_OK) return st;
@@ -303,6 +305,7 @@ int32_t t3_linear_plan_of(const t3_array* x, const t3_array* trellis, t3_decode 
 
 int32_t t3_linear_chain(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
                         const t3_array* svh, t3_decode dec, t3_array* y, void* workspace, size_t workspace_bytes) {
+    const t3::ConfigScope one_config;
     return t3_linear_stages(stream, x, trellis, suh, svh, dec, y, workspace, workspace_bytes,
                             T3_STAGE_PREPARE | T3_STAGE_GEMV | T3_STAGE_FINISH);
 }
@@ -310,6 +313,7 @@ int32_t t3_linear_chain(t3_stream stream, const t3_array* x, const t3_array* tre
 int32_t t3_linear_stages(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
                          const t3_array* svh, t3_decode dec, t3_array* y, void* workspace, size_t workspace_bytes,
                          uint32_t stages) {
+    const t3::ConfigScope one_config;
     if (!suh || !svh || !y) return T3_BadArgs;
     if (stages == 0u || stages > 7u) return T3_BadArgs;
     t3::DenseCall call;
@@ -322,6 +326,7 @@ int32_t t3_linear_stages(t3_stream stream, const t3_array* x, const t3_array* tr
 
 int32_t t3_linear(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
                   const t3_array* svh, t3_decode dec, t3_array* y, void* workspace, size_t workspace_bytes) {
+    const t3::ConfigScope one_config;
     if (!suh || !svh || !y) return T3_BadArgs;
     t3::DenseCall call;
     if (const int32_t st = t3::check_dense(x, trellis, suh, svh, dec, y, 0, &call); st != T3_OK) return st;
@@ -346,6 +351,7 @@ int32_t t3_linear(t3_stream stream, const t3_array* x, const t3_array* trellis, 
 int32_t t3_linear_bias(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
                        const t3_array* svh, const t3_array* bias, t3_decode dec, t3_array* y, void* workspace,
                        size_t workspace_bytes) {
+    const t3::ConfigScope one_config;
     // root.linearBias's own checks (src/root.zig:365-370), then `linear`, then one add in x's dtype
     if (!t3::array_ok(bias) || !t3::array_ok(trellis) || !t3::array_ok(x)) return T3_BadArgs;
     if (!t3::aligned16(bias)) return T3_BadArgs;
@@ -361,6 +367,7 @@ int32_t t3_linear_bias(t3_stream stream, const t3_array* x, const t3_array* trel
 }
 
 int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_array* w_hat) {
+    const t3::ConfigScope one_config;
     if (!t3::array_ok(trellis) || !t3::array_ok(w_hat)) return T3_BadArgs;
     if (!t3::aligned16(trellis) || !t3::aligned16(w_hat)) return T3_BadArgs;
     if (trellis->ndim != 3 || w_hat->ndim != 2) return T3_BadExl3Shape;
@@ -379,6 +386,7 @@ int32_t t3_dequant(t3_stream stream, const t3_array* trellis, t3_decode dec, t3_
 }
 
 int32_t t3_linear_resident_workspace_bytes(const t3_array* x, const t3_array* w_hat, size_t* bytes) {
+    const t3::ConfigScope one_config;
     if (!bytes) return T3_BadArgs;
     t3::DenseCall call;
     if (const int32_t st = t3::check_resident(x, w_hat, nullptr, nullptr, nullptr, &call); st != T3_OK) return st;
@@ -391,6 +399,7 @@ int32_t t3_linear_resident_workspace_bytes(const t3_array* x, const t3_array* w_
 
 int32_t t3_linear_resident(t3_stream stream, const t3_array* x, const t3_array* w_hat, const t3_array* suh,
                            const t3_array* svh, t3_array* y, void* workspace, size_t workspace_bytes) {
+    const t3::ConfigScope one_config;
     if (!suh || !svh || !y) return T3_BadArgs;
     t3::DenseCall call;
     if (const int32_t st = t3::check_resident(x, w_hat, suh, svh, y, &call); st != T3_OK) return st;
@@ -404,6 +413,7 @@ int32_t t3_linear_resident(t3_stream stream, const t3_array* x, const t3_array* 
 }
 
 int32_t t3_unrot_workspace_bytes(const t3_array* trellis, size_t* bytes) {
+    const t3::ConfigScope one_config;
     if (!bytes || !t3::array_ok(trellis)) return T3_BadArgs;
     if (trellis->ndim != 3) return T3_BadExl3Shape;
     const int64_t in = trellis->shape[0] * 16, out = trellis->shape[1] * 16;
@@ -419,6 +429,7 @@ int32_t t3_unrot_workspace_bytes(const t3_array* trellis, size_t* bytes) {
 int32_t t3_unrot_weight(t3_stream stream, const t3_array* trellis, const t3_array* suh, const t3_array* svh,
                         t3_decode dec, t3_array* w_std, int64_t col0, uint32_t* nonfinite, void* workspace,
                         size_t workspace_bytes) {
+    const t3::ConfigScope one_config;
     if (!t3::array_ok(trellis) || !t3::array_ok(suh) || !t3::array_ok(svh) || !t3::array_ok(w_std) || !t3::workspace_ok(workspace))
         return T3_BadArgs;
     if (trellis->ndim != 3 || w_std->ndim != 2 || suh->ndim != 1 || svh->ndim != 1) return T3_BadExl3Shape;
@@ -491,17 +502,18 @@ uint32_t unrot_kparts(int64_t rows, int64_t in, int64_t cols) {
 
 int32_t t3_linear_unrot(t3_stream stream, const t3_array* x, const t3_array* w_std, int64_t col0, int64_t cols,
                         t3_array* y) {
+    const t3::ConfigScope one_config;
     if (!y) return T3_BadArgs;
     int64_t rows = 0, in = 0;
     if (const int32_t st = check_unrot(x, w_std, col0, cols, y, &rows, &in); st != T3_OK) return st;
-    const size_t esz = 2u;
     return t3::hip_status(t3::launch_gemm_half(
-        x->data, static_cast<const unsigned char*>(w_std->data) + static_cast<size_t>(col0) * esz, y->data,
-        static_cast<uint32_t>(rows), static_cast<uint32_t>(in), static_cast<uint32_t>(cols),
-        static_cast<uint32_t>(w_std->shape[1]), w_std->dtype == T3_BF16, static_cast<hipStream_t>(stream)));
+        x->data, w_std->data, y->data, static_cast<uint32_t>(rows), static_cast<uint32_t>(in), static_cast<uint32_t>(cols),
+        static_cast<uint32_t>(w_std->shape[1]), static_cast<uint32_t>(col0), w_std->dtype == T3_BF16,
+        static_cast<hipStream_t>(stream)));
 }
 
 int32_t t3_linear_unrot_workspace_bytes(const t3_array* x, const t3_array* w_std, int64_t col0, int64_t cols, size_t* bytes) {
+    const t3::ConfigScope one_config;
     if (!bytes) return T3_BadArgs;
     int64_t rows = 0, in = 0;
     if (const int32_t st = check_unrot(x, w_std, col0, cols, nullptr, &rows, &in); st != T3_OK) return st;
@@ -515,6 +527,7 @@ int32_t t3_linear_unrot_workspace_bytes(const t3_array* x, const t3_array* w_std
 
 int32_t t3_linear_unrot_parts(t3_stream stream, const t3_array* x, const t3_array* w_std, int64_t col0, int64_t cols,
                               t3_array* y, void* workspace, size_t workspace_bytes) {
+    const t3::ConfigScope one_config;
     if (!y) return T3_BadArgs;
     int64_t rows = 0, in = 0;
     if (const int32_t st = check_unrot(x, w_std, col0, cols, y, &rows, &in); st != T3_OK) return st;
@@ -524,13 +537,14 @@ int32_t t3_linear_unrot_parts(t3_stream stream, const t3_array* x, const t3_arra
     const uint32_t k = unrot_kparts(rows, in, cols);
     float* planes = k > 1u ? c.take<float>(static_cast<size_t>(k) * rows * cols * 4u) : nullptr;
     if (workspace_bytes < c.used) return T3_WorkspaceTooSmall;
-    const unsigned char* w = static_cast<const unsigned char*>(w_std->data) + static_cast<size_t>(col0) * 2u;
+    const void* w = w_std->data;
+    const uint32_t c0 = static_cast<uint32_t>(col0);
     const bool bf16 = w_std->dtype == T3_BF16;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const uint32_t r = static_cast<uint32_t>(rows), i = static_cast<uint32_t>(in), n = static_cast<uint32_t>(cols);
     const uint32_t ldw = static_cast<uint32_t>(w_std->shape[1]);
-    if (k == 1u) return t3::hip_status(t3::launch_gemm_half(x->data, w, y->data, r, i, n, ldw, bf16, s));
-    if (const int32_t st = t3::hip_status(t3::launch_gemm_planes(x->data, w, planes, r, i, n, ldw, bf16, k, s)); st != T3_OK)
+    if (k == 1u) return t3::hip_status(t3::launch_gemm_half(x->data, w, y->data, r, i, n, ldw, c0, bf16, s));
+    if (const int32_t st = t3::hip_status(t3::launch_gemm_planes(x->data, w, planes, r, i, n, ldw, c0, bf16, k, s)); st != T3_OK)
         return st;
     return t3::hip_status(t3::launch_gemm_planes_round(planes, y->data, r, n, k, bf16, s));
 }
@@ -556,6 +570,13 @@ __global__ void __launch_bounds__(256) static_scratch_clear(uint32_t* p, uint32_
     if (i < words) p[i] = 0u;
 }
 
+int32_t static_scratch_clear_head(hipStream_t s, unsigned char* p) {
+    const uint32_t words = static_cast<uint32_t>(t3::kCounterBytes / 4u);
+    hipLaunchKernelGGL(static_scratch_clear, dim3((words + 255u) / 256u), dim3(256), 0, s, reinterpret_cast<uint32_t*>(p),
+                       words);
+    return hipGetLastError() == hipSuccess ? T3_OK : T3_HipFailed;
+}
+
 // The current device's copy of the array. The first call on a device looks its address up and clears the counter head
 // on `s` (the loader zero-fills the array too; the clear makes the contract explicit). Two threads racing through the
 // first call store the same address and both clear before their own launches on their own streams' order.
@@ -567,10 +588,7 @@ int32_t static_scratch_of(hipStream_t s, unsigned char** out) {
         void* sym = nullptr;
         if (hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)) != hipSuccess || !sym) return T3_HipFailed;
         p = static_cast<unsigned char*>(sym);
-        const uint32_t words = static_cast<uint32_t>(t3::kCounterBytes / 4u);
-        hipLaunchKernelGGL(static_scratch_clear, dim3((words + 255u) / 256u), dim3(256), 0, s,
-                           reinterpret_cast<uint32_t*>(p), words);
-        if (hipGetLastError() != hipSuccess) return T3_HipFailed;
+        if (static_scratch_clear_head(s, p) != T3_OK) return T3_HipFailed;
         static_scratch_ptr[dev].store(p, std::memory_order_release);
     }
     *out = p;
@@ -583,6 +601,7 @@ extern "C" {
 
 int32_t t3_linear_static(t3_stream stream, const t3_array* x, const t3_array* trellis, const t3_array* suh,
                          const t3_array* svh, t3_decode dec, t3_array* y) {
+    const t3::ConfigScope one_config;
     if (!suh || !svh || !y) return T3_BadArgs;
     t3::DenseCall call;
     if (const int32_t st = t3::check_dense(x, trellis, suh, svh, dec, y, 0, &call); st != T3_OK) return st;
@@ -594,7 +613,17 @@ int32_t t3_linear_static(t3_stream stream, const t3_array* x, const t3_array* tr
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (const int32_t st = static_scratch_of(s, &base); st != T3_OK) return st;
     t3::carve_dense(&call, base);
-    return t3::run_fused(call, s);
+    const int32_t st = t3::run_fused(call, s);
+    // a launch that reported an error may have left part of the chain's counters counted: no caller can reach them
+    if (st != T3_OK) static_scratch_clear_head(s, base);
+    return st;
+}
+
+int32_t t3_linear_static_reset(t3_stream stream) {
+    unsigned char* base = nullptr;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (const int32_t st = static_scratch_of(s, &base); st != T3_OK) return st;
+    return static_scratch_clear_head(s, base);
 }
 
 }  // extern "C"

@@ -271,6 +271,7 @@ extern "C" {
 
 int32_t t3_moe_workspace_bytes(const t3_array* x, const t3_bank* bank, const t3_array* inds,
                                const t3_bank* shared_bank, size_t* bytes) {
+    const t3::ConfigScope one_config;
     if (!bytes) return T3_BadArgs;
     t3::MoeCall call;
     const t3_decode dec = {0, 16};
@@ -289,6 +290,7 @@ int32_t t3_moe_workspace_bytes(const t3_array* x, const t3_bank* bank, const t3_
 
 int32_t t3_moe_plan_of(const t3_array* x, const t3_bank* bank, const t3_array* inds, const t3_bank* shared_bank,
                        t3_moe_plan* plan) {
+    const t3::ConfigScope one_config;
     if (!plan) return T3_BadArgs;
     t3::MoeCall call;
     const t3_decode dec = {0, 16};
@@ -337,6 +339,7 @@ int32_t t3_moe_plan_of(const t3_array* x, const t3_bank* bank, const t3_array* i
 int32_t t3_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
                const t3_array* scores, t3_decode dec, int32_t verify_rows, t3_array* y, void* workspace,
                size_t workspace_bytes) {
+    const t3::ConfigScope one_config;
     (void)verify_rows;
     return t3::run_moe(stream, x, bank, inds, scores, nullptr, nullptr, dec, 0, y, workspace, workspace_bytes);
 }
@@ -344,6 +347,7 @@ int32_t t3_moe(t3_stream stream, const t3_array* x, const t3_bank* bank, const t
 int32_t t3_moe_clamped(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
                        const t3_array* scores, t3_decode dec, int32_t limit, t3_array* y, void* workspace,
                        size_t workspace_bytes) {
+    const t3::ConfigScope one_config;
     if (limit <= 0 || limit > 128) return T3_InvalidExl3Clamp;
     return t3::run_moe(stream, x, bank, inds, scores, nullptr, nullptr, dec, limit, y, workspace, workspace_bytes);
 }
@@ -351,6 +355,7 @@ int32_t t3_moe_clamped(t3_stream stream, const t3_array* x, const t3_bank* bank,
 int32_t t3_moe_swiglu(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
                       const t3_array* scores, t3_decode dec, int32_t limit, int32_t clamp_at, t3_array* y,
                       void* workspace, size_t workspace_bytes) {
+    const t3::ConfigScope one_config;
     if (limit < 0 || limit > 128 || (clamp_at != T3_CLAMP_GATE_IN && clamp_at != T3_CLAMP_SILU_OUT)) return T3_InvalidExl3Clamp;
     return t3::run_moe(stream, x, bank, inds, scores, nullptr, nullptr, dec, limit, y, workspace, workspace_bytes, clamp_at);
 }
@@ -358,6 +363,7 @@ int32_t t3_moe_swiglu(t3_stream stream, const t3_array* x, const t3_bank* bank, 
 int32_t t3_moe_with_shared(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
                            const t3_array* scores, t3_decode dec, int32_t verify_rows, const t3_array* shared,
                            t3_array* y, void* workspace, size_t workspace_bytes) {
+    const t3::ConfigScope one_config;
     (void)verify_rows;
     if (!shared) return T3_BadArgs;
     return t3::run_moe(stream, x, bank, inds, scores, nullptr, shared, dec, 0, y, workspace, workspace_bytes);
@@ -366,6 +372,7 @@ int32_t t3_moe_with_shared(t3_stream stream, const t3_array* x, const t3_bank* b
 int32_t t3_moe_shared_expert(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
                              const t3_array* scores, t3_decode dec, int32_t limit, const t3_bank* shared_bank,
                              t3_array* y, void* workspace, size_t workspace_bytes) {
+    const t3::ConfigScope one_config;
     if (!shared_bank) return T3_BadArgs;
     return t3::run_moe(stream, x, bank, inds, scores, shared_bank, nullptr, dec, limit, y, workspace, workspace_bytes);
 }
@@ -373,6 +380,7 @@ int32_t t3_moe_shared_expert(t3_stream stream, const t3_array* x, const t3_bank*
 int32_t t3_moe_stages(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
                       const t3_array* scores, t3_decode dec, int32_t limit, const t3_bank* shared_bank, t3_array* y,
                       void* workspace, size_t workspace_bytes, uint32_t stages) {
+    const t3::ConfigScope one_config;
     if (limit < 0 || limit > 128) return T3_InvalidExl3Clamp;
     if (stages == 0u || stages > 63u) return T3_BadArgs;
     return t3::run_moe(stream, x, bank, inds, scores, shared_bank, nullptr, dec, limit, y, workspace, workspace_bytes, 0,
@@ -383,6 +391,7 @@ int32_t t3_moe_stages(t3_stream stream, const t3_array* x, const t3_bank* bank, 
  * f32 output, no scores; the slots of a row are the host's to combine. */
 int32_t t3_moe_glm(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds, t3_decode dec,
                    int32_t limit, t3_array* y, void* workspace, size_t workspace_bytes) {
+    const t3::ConfigScope one_config;
     if (!t3::array_ok(y)) return T3_BadArgs;
     if (limit < 0 || limit > 128) return T3_InvalidExl3Clamp;
     t3::MoeCall call;
@@ -504,6 +513,7 @@ int32_t fused_shared(t3_stream stream, const t3_array* x, const t3_bank* bank, c
 int32_t t3_moe_fused_shared(t3_stream stream, const t3_array* x, const t3_bank* bank, const t3_array* inds,
                             const t3_array* scores, t3_decode dec, const t3_bank* shared_bank, const t3_array* sigtab,
                             const t3_array* logit, t3_array* y, void* workspace, size_t workspace_bytes) {
+    const t3::ConfigScope one_config;
     if (!inds || !scores || !y) return T3_BadArgs;
     if (!logit) return T3_BadArgs;
     return fused_shared(stream, x, bank, inds, scores, nullptr, 0, dec, shared_bank, sigtab, logit, nullptr, y, workspace,
@@ -512,6 +522,7 @@ int32_t t3_moe_fused_shared(t3_stream stream, const t3_array* x, const t3_bank* 
 
 int32_t t3_moe_fused_shared_routed_workspace_bytes(const t3_array* x, const t3_bank* bank, const t3_array* logits,
                                                    int64_t k, const t3_bank* shared_bank, size_t* bytes) {
+    const t3::ConfigScope one_config;
     if (!bytes || !logits) return T3_BadArgs;
     const t3_decode dec = {0, 16};
     return fused_shared(nullptr, x, bank, nullptr, nullptr, logits, k, dec, shared_bank, nullptr, nullptr, nullptr, nullptr,
@@ -522,6 +533,7 @@ int32_t t3_moe_fused_shared_routed(t3_stream stream, const t3_array* x, const t3
                                    int64_t k, t3_decode dec, const t3_bank* shared_bank, const t3_array* sigtab,
                                    const t3_array* logit, const t3_array* gate_vec, t3_array* y, void* workspace,
                                    size_t workspace_bytes) {
+    const t3::ConfigScope one_config;
     if (!logits || !y) return T3_BadArgs;
     return fused_shared(stream, x, bank, nullptr, nullptr, logits, k, dec, shared_bank, sigtab, logit, gate_vec, y,
                         workspace, workspace_bytes, nullptr);

@@ -35,10 +35,12 @@ __global__ void __launch_bounds__(64) moe_prep(const MoeLaunch a) {
 // tiles). z[proj]: f32 [KS][RKT][out], the four waves' sums, wave 0 first. XLDS (gate|up only, per == 8): the wave
 // prepares its own 128-block of x in LDS.
 //
-// XLDS on the down launch (per == 4): the wave makes its input itself, running the mid stage of the 128-block its
-// tiles lie in over the gate|up launch's planes; measured faster than the arriving gate|up launch up to two rows
-// (one row 25.3 against 26.5 us, two 29.7 against 31.2; three 38.0 against 37.3), since the stage no longer waits for
-// a hand-off inside a launch but is run by all sixteen column workgroups of a slot.
+// XLDS on the down launch (per == 8: a wave's eight input tiles are one 128-block): the wave makes its input itself,
+// running the mid stage of that block over the gate|up launch's planes: the stage no longer waits for a hand-off inside
+// a launch but is run by all sixteen column workgroups of a slot. Measured against the arriving gate|up launch with
+// eight tiles a down wave (us a call): 3 rows 35.0 against 35.5, 4 rows 38.0 against 38.6, 8 rows 57.9 against 56.0,
+// 16 rows 98.6 against 94.7: served up to kMidInDownRows = 4 rows. (With four tiles a down wave, an earlier form, it won
+// up to two rows only: one row 25.3 against 26.5, two 29.7 against 31.2, three 38.0 against 37.3.)
 //
 // ARRIVE: the launch also runs the stage after it. The planes are stored device-coherently, every workgroup counts
 // itself in at its 128-column block, and the last to arrive runs that block's next stage on the complete planes:
@@ -465,7 +467,8 @@ hipError_t launch_gemv_bt(const MoeLaunch& a, hipStream_t s) {
     return hipGetLastError();
 }
 
-// PROF 1 (GLM's roundings in the stages a launch runs itself) exists for the served codebook forms only
+// PROF 1 (GLM's roundings in the stages a launch runs itself) exists for the codebook forms a default or opt-in
+// configuration serves: MCG's f16 weight, its pair form, and MUL1's deferred map
 template <int NPROJ, bool XLDS, bool ARRIVE, int PROF = 0>
 hipError_t launch_gemv_cb(const MoeLaunch& a, hipStream_t s) {
     return with_reader(NPROJ == 2 ? a.n_gu : a.n_dn, [&](auto reader) {
@@ -481,6 +484,7 @@ hipError_t launch_gemv_cb(const MoeLaunch& a, hipStream_t s) {
             switch (a.codebook) {
                 case kMul1Defer: return launch_gemv_bt<kMul1Defer, R, NPROJ, XLDS, ARRIVE, 1>(a, s);
                 case kMcgPair: return launch_gemv_bt<kMcgPair, R, NPROJ, XLDS, ARRIVE, 1>(a, s);
+                case kMcg: return launch_gemv_bt<kMcg, R, NPROJ, XLDS, ARRIVE, 1>(a, s);
                 default: return hipErrorInvalidValue;
             }
         }
@@ -533,7 +537,7 @@ hipError_t launch_moe_decode(const MoeLaunch& a, int form, hipStream_t s) {
         if (a.stages & 2u) return mid_in_down ? launch_gemv_cb<1, true, true>(a, s) : launch_gemv_cb<1, false, true>(a, s);
         return hipSuccess;
     }
-    if (form == kMoeTwoLaunches && (a.codebook == kMcgPair || a.codebook == kMul1Defer)) {
+    if (form == kMoeTwoLaunches && a.codebook != kMul1) {
         // GLM's profile in the same two launches (src/hip/plan.zig's form 9 under Profile.glm), its own roundings in the
         // stages the launches run themselves
         if ((e = mid_in_down ? launch_gemv_cb<2, true, false, 1>(a, s) : launch_gemv_cb<2, true, true, 1>(a, s)) != hipSuccess)
@@ -557,8 +561,8 @@ hipError_t launch_moe_decode(const MoeLaunch& a, int form, hipStream_t s) {
         return hipGetLastError();
     }
     if (a.glm) {
-        // GLM's profile on the five launches (the exact codebook forms, or a configured decode_form): its own roundings
-        // in the stages between the GEMVs
+        // GLM's profile on the five launches (MUL1 decoded weight by weight, or a configured decode_form): its own
+        // roundings in the stages between the GEMVs
         hipLaunchKernelGGL(moe_prep<1>, dim3(a.hidden / 128u, rkt), dim3(64), 0, s, a);
         if ((e = hipGetLastError()) != hipSuccess) return e;
         if ((e = launch_gemv_cb<2, false, false>(a, s)) != hipSuccess) return e;

@@ -80,12 +80,17 @@ __device__ __forceinline__ uint4v rsrc_words(const void* p, uint64_t bytes) {
     const uint32_t n = bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : static_cast<uint32_t>(bytes);
     return uint4v{static_cast<uint32_t>(addr), static_cast<uint32_t>(addr >> 32) & 0xFFFFu, n, 0x00020000u};
 }
+// (m0 is named as clobbered so the compiler keeps nothing of its own in it across the statement; clang warns about any
+// reserved register in a clobber list, which is the point here)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void load_to_lds(uint4v desc, uint32_t lds, uint32_t voff, uint32_t soff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :
                  : "s"(lds), "v"(voff), "s"(desc), "s"(soff)
-                 : "memory");
+                 : "memory", "m0");
 }
+#pragma clang diagnostic pop
 // at most N of the wave's loads are still in flight (they complete in order)
 template <int N>
 __device__ __forceinline__ void wait_loads() {

@@ -406,6 +406,7 @@ int32_t t3_table_load_bank(const t3_block* block, const t3_array* trellis, const
 
 int32_t t3_table_matmul(t3_stream stream, const t3_weight* w, const t3_array* x, t3_array* y, void* workspace,
                         size_t workspace_bytes, char* why, size_t why_bytes) {
+    const t3::ConfigScope one_config;
     t3_decode dec;
     if (!t3::decode_of(w, &dec)) return t3::refuse(T3_VERDICT_FAILED, why, why_bytes, "turboexl3: a weight without its decode");
     return t3::verdict_of(t3_linear(stream, x, &w->w, &w->scales, &w->biases, dec, y, workspace, workspace_bytes), why,
@@ -413,6 +414,7 @@ int32_t t3_table_matmul(t3_stream stream, const t3_weight* w, const t3_array* x,
 }
 
 int32_t t3_table_matmul_workspace_bytes(const t3_weight* w, const t3_array* x, size_t* bytes) {
+    const t3::ConfigScope one_config;
     t3_decode dec;
     if (!t3::decode_of(w, &dec)) return T3_BadArgs;
     return t3_linear_workspace_bytes(x, &w->w, dec, bytes);
@@ -427,6 +429,7 @@ int32_t t3_table_swiglu(t3_stream stream, const t3_weight* gate, const t3_weight
                         const t3_array* x, const t3_array* inds, const t3_array* scores, int32_t limit,
                         int32_t verify_rows, t3_array* y, void* workspace, size_t workspace_bytes, char* why,
                         size_t why_bytes) {
+    const t3::ConfigScope one_config;
     // table/table.zig:210-222
     t3_decode dec, du, dd;
     if (!t3::decode_of(gate, &dec)) return t3::refuse(T3_VERDICT_FAILED, why, why_bytes, "turboexl3: a bank without its decode");
@@ -441,6 +444,7 @@ int32_t t3_table_swiglu(t3_stream stream, const t3_weight* gate, const t3_weight
 
 int32_t t3_table_swiglu_workspace_bytes(const t3_weight* gate, const t3_weight* up, const t3_weight* down,
                                         const t3_array* x, const t3_array* inds, size_t* bytes) {
+    const t3::ConfigScope one_config;
     if (!gate || !up || !down) return T3_BadArgs;
     const t3_bank bank = {t3::proj_of(gate), t3::proj_of(up), t3::proj_of(down)};
     return t3_moe_workspace_bytes(x, &bank, inds, nullptr, bytes);
