@@ -134,13 +134,16 @@ struct GemvArgs {
 // Grid (out / 16 / BT, KS), 256 threads (4 waves). A workgroup owns BT adjacent output tiles and K slice blockIdx.y;
 // wave sg takes part sg of the slice, `per` = in_tiles / (4 KS) input tiles (the host divides: the GPU has no scalar
 // divide). RB = 16-row blocks of x (1 or 2). z f32 [KS][rows][out]: the four waves' sums, wave 0 first.
-template <int CB, int WIDE, int RB, int BT, int FUSE>
+// LDS: the tiles go from memory straight into an LDS ring (served where a wave's walk is long, dense_gemv_lds_ring);
+// else through the register ring.
+template <int CB, int WIDE, int RB, int BT, int FUSE, bool LDS>
 __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
-    constexpr int ST = 2;  // tile rows in flight a wave: occupancy hides more latency here than a deeper ring does
-    constexpr uint32_t kStage = gemv_stage_bytes<BT>();
+    typedef GemvStream<LDS, CB, WIDE, RB, BT, XLds> StreamL;
+    typedef GemvStream<LDS, CB, WIDE, RB, BT, XGlobal> StreamG;
+    constexpr uint32_t kStage = StreamG::kStageBytes;
     constexpr uint32_t kRed = 4u * RB * BT * 64u * 16u;
     constexpr uint32_t kMain = kRed > 4u * kStage ? kRed : 4u * kStage;
-    // the waves' LDS stages while they stream; the four waves' partial sums afterwards
+    // the waves' LDS rings while they stream; the four waves' partial sums afterwards
     __shared__ __attribute__((aligned(16))) unsigned char smem[kMain];
     __shared__ uint32_t last_flag;
     float4v(*red)[RB * BT * 64] = reinterpret_cast<float4v(*)[RB * BT * 64]>(smem);
@@ -160,7 +163,8 @@ __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
     const uint32_t wstep = static_cast<uint32_t>(wstride) * 4u;
 
     // x fragment: activation row (lane % 16) of block r, K slots 8g..8g+7 = quad g's four inputs, each doubled.
-    // Rows past the call's last alias row 0: their sums are computed and never stored.
+    // Rows past the call's last are zeros (the chain forms) or alias row 0 (the one-launch form): their sums are
+    // computed and never stored.
     uint32_t xoff[RB];
     constexpr uint32_t kShare = 8u / BT;  // workgroup columns a 128-column block
     const uint32_t b128 = blk / kShare;
@@ -171,8 +175,7 @@ __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
         unsigned char* xst = xdyn + sg * ((per + 1u) * (kXldsRows * 64u));
         const uint32_t row = lane & 15u;
         xoff[0] = (row < rows ? row : 0u) * 64u + (lane >> 4) * 16u;
-        GemvStream<CB, WIDE, RB, BT, ST, XLds> stream(wbase, wstep, per, a.n, a.wbits, XLds{xst}, xoff,
-                                                      smem + sg * kStage, lane);
+        StreamL stream(wbase, wstep, per, a.n, a.wbits, XLds{xst}, xoff, smem + sg * kStage, lane);
         stream.issue();
         // While the codes fly, the wave prepares its own K part: per / 8 whole 128-blocks a row, the statements of
         // dense_prep, into its LDS x stage [per + 1][4][64 bytes] (the last tile row zeros). The block sums go to the
@@ -225,15 +228,15 @@ __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
 #pragma unroll
         for (int r = 0; r < RB; ++r) {
             const uint32_t row = static_cast<uint32_t>(r) * 16u + (lane & 15u);
-            xoff[r] = ((row < rows ? row : 0u) * 16u + 4u * (lane >> 4)) * 4u;
+            xoff[r] = x_frag_offset(lane, row < rows, row * 64u);
         }
-        GemvStream<CB, WIDE, RB, BT, ST, XGlobal> stream(
-            wbase, wstep, per, a.n, a.wbits, XGlobal{a.xq, static_cast<uint64_t>(rows) * a.in * 4u, tk0 * rows * 64u, rows * 64u}, xoff,
-            smem + sg * kStage, lane);
+        StreamG stream(wbase, wstep, per, a.n, a.wbits,
+                       XGlobal{a.xq, static_cast<uint64_t>(rows) * a.in * 4u, tk0 * rows * 64u, rows * 64u}, xoff,
+                       smem + sg * kStage, lane);
         stream.issue();
         stream.run(acc);
     }
-    __syncthreads();  // every wave is done with its stage before the sums take the memory
+    __syncthreads();  // every wave is done with its rings (no load in flight) before the sums take the memory
 
     // lane holds, for activation row (lane % 16) of block r, output columns 4g..4g+3 of tile t
 #pragma unroll
@@ -303,17 +306,21 @@ hipError_t launch_gemv_fuse(const DenseLaunch& d, int fuse, hipStream_t s) {
     a.dt = d.dtype;
     a.defer = d.codebook == kMul1Defer;
     const dim3 grid((d.out / 16u) / BT, d.ks), block(256);
+    const bool lds = dense_gemv_lds_ring(a.per);
     if (fuse == kOne) {
         if constexpr (RB == 1) {
+            // the one-launch form serves waves of 8 or 16 tile rows: below the LDS ring's bound
             const size_t dyn = 4u * (a.per + 1u) * (kXldsRows * 64u);
-            hipLaunchKernelGGL((dense_gemv<CB, WIDE, 1, BT, kOne>), grid, block, dyn, s, a);
+            hipLaunchKernelGGL((dense_gemv<CB, WIDE, 1, BT, kOne, false>), grid, block, dyn, s, a);
         } else {
             return hipErrorInvalidValue;
         }
     } else if (fuse == kArrive) {
-        hipLaunchKernelGGL((dense_gemv<CB, WIDE, RB, BT, kArrive>), grid, block, 0, s, a);
+        if (lds) hipLaunchKernelGGL((dense_gemv<CB, WIDE, RB, BT, kArrive, true>), grid, block, 0, s, a);
+        else hipLaunchKernelGGL((dense_gemv<CB, WIDE, RB, BT, kArrive, false>), grid, block, 0, s, a);
     } else {
-        hipLaunchKernelGGL((dense_gemv<CB, WIDE, RB, BT, kChain>), grid, block, 0, s, a);
+        if (lds) hipLaunchKernelGGL((dense_gemv<CB, WIDE, RB, BT, kChain, true>), grid, block, 0, s, a);
+        else hipLaunchKernelGGL((dense_gemv<CB, WIDE, RB, BT, kChain, false>), grid, block, 0, s, a);
     }
     return hipGetLastError();
 }

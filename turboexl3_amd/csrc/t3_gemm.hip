@@ -33,6 +33,7 @@
 
 #include "t3_common.hpp"
 #include "t3_kernels.hpp"
+#include "t3_lds_loads.hpp"
 #include "t3_stages.hpp"
 
 namespace t3 {
@@ -67,27 +68,6 @@ struct GemmArgs {
 // by the finish launch behind it)
 enum GemmEnd : int { kGemmPlain = 0, kGemmFinish = 1, kGemmPlanes = 2 };
 
-__device__ __forceinline__ uint4v gemm_rsrc(const void* p, uint64_t bytes) {
-    const uint64_t addr = reinterpret_cast<uint64_t>(p);
-    const uint32_t n = bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : static_cast<uint32_t>(bytes);
-    return uint4v{static_cast<uint32_t>(addr), static_cast<uint32_t>(addr >> 32) & 0xFFFFu, n, 0x00020000u};
-}
-// (m0 is named as clobbered so the compiler keeps nothing of its own in it across the statement; clang warns about any
-// reserved register in a clobber list, which is the point here)
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Winline-asm"
-__device__ __forceinline__ void gemm_load_to_lds(uint4v desc, uint32_t lds, uint32_t voff, uint32_t soff) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                 :
-                 : "s"(lds), "v"(voff), "s"(desc), "s"(soff)
-                 : "memory", "m0");
-}
-#pragma clang diagnostic pop
-template <int N>
-__device__ __forceinline__ void gemm_wait_loads() {
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
-}
-
 template <bool BF16>
 __device__ __forceinline__ float4v gemm_mfma(uint4v a, uint4v b, float4v c) {
     if constexpr (BF16)
@@ -114,9 +94,9 @@ __global__ void __launch_bounds__(512) gemm_half(const GemmArgs a) {
 
     // the tile's windows of x and w: rows past the last one, and the bytes past w's end, read as zeros
     const uint32_t rows_here = a.rows - row0 < kGM ? a.rows - row0 : kGM;
-    const uint4v xdesc = gemm_rsrc(static_cast<const unsigned char*>(a.x) + static_cast<size_t>(row0) * a.in * 2u,
+    const uint4v xdesc = rsrc_words(static_cast<const unsigned char*>(a.x) + static_cast<size_t>(row0) * a.in * 2u,
                                    static_cast<uint64_t>(rows_here) * a.in * 2u);
-    const uint4v wdesc = gemm_rsrc(static_cast<const unsigned char*>(a.w) + static_cast<size_t>(col0) * 2u,
+    const uint4v wdesc = rsrc_words(static_cast<const unsigned char*>(a.w) + static_cast<size_t>(col0) * 2u,
                                    (static_cast<uint64_t>(a.in) * a.ldw - a.wcol0 - col0) * 2u);
     // this wave's loads a step: x rows 32 wave .. + 31 (two loads of 16 rows), w rows k = 4 wave .. + 3 (two of 2 rows;
     // a 128-column tile loads 256 columns all the same and leaves the second half alone)
@@ -138,10 +118,10 @@ __global__ void __launch_bounds__(512) gemm_half(const GemmArgs a) {
     auto issue = [&](uint32_t step, uint32_t slot) {
         const uint32_t base = lds0 + slot * kGStep, at = step0 + step;
 #pragma unroll
-        for (uint32_t i = 0; i < 2u; ++i) gemm_load_to_lds(xdesc, base + (2u * wave + i) * 1024u, x_voff[i], at * (kGK * 2u));
+        for (uint32_t i = 0; i < 2u; ++i) load_to_lds(xdesc, base + (2u * wave + i) * 1024u, x_voff[i], at * (kGK * 2u));
 #pragma unroll
         for (uint32_t i = 0; i < 2u; ++i)
-            gemm_load_to_lds(wdesc, base + kGXBytes + (2u * wave + i) * 1024u, w_voff[i], at * w_step_bytes);
+            load_to_lds(wdesc, base + kGXBytes + (2u * wave + i) * 1024u, w_voff[i], at * w_step_bytes);
     };
 
     // where a lane's fragments sit inside a step's 32 KB
@@ -168,7 +148,7 @@ __global__ void __launch_bounds__(512) gemm_half(const GemmArgs a) {
 
 #pragma unroll
         for (uint32_t t = 0; t + 1u < kGD; ++t) issue(t, t);   // loads past the last step bring zeros or unused bytes
-        gemm_wait_loads<static_cast<int>(kGD - 2u) * kGLoadsAStep>();
+        wait_loads<static_cast<int>(kGD - 2u) * kGLoadsAStep>();
         __syncthreads();
         uint32_t slot = 0;
         for (uint32_t s = 0; s < steps; ++s) {
@@ -191,11 +171,11 @@ __global__ void __launch_bounds__(512) gemm_half(const GemmArgs a) {
                 for (int rb = 0; rb < 8; ++rb) acc[cb][rb] = gemm_mfma<BF16>(wf[cb], xf[rb], acc[cb][rb]);
             // step s + 1's loads of this wave have landed once at most kGD - 2 steps' are in flight; the barrier then
             // publishes every wave's part of it
-            gemm_wait_loads<static_cast<int>(kGD - 2u) * kGLoadsAStep>();
+            wait_loads<static_cast<int>(kGD - 2u) * kGLoadsAStep>();
             __syncthreads();
             slot = slot + 1u == kGD ? 0u : slot + 1u;
         }
-        gemm_wait_loads<0>();
+        wait_loads<0>();
         if constexpr (END == kGemmPlanes) {
             // the part's f32 sums as they lie in the accumulators: four adjacent columns of one row a lane and block
             float* plane = a.planes + static_cast<size_t>(blockIdx.z) * a.rows * a.cols;

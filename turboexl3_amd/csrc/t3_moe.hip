@@ -48,20 +48,20 @@ __global__ void __launch_bounds__(64) moe_prep(const MoeLaunch a) {
 // (row, block of hidden); skipped slots count themselves in too). The statements are the chain's, so are the bytes.
 constexpr uint32_t kMidInDownRows = 4u;
 
-// a workgroup's static LDS: the four waves' stages while they stream, their partial sums afterwards
+// a workgroup's static LDS: the four waves' rings while they stream, their partial sums afterwards
 template <int BT>
 constexpr uint32_t role_lds_bytes() {
-    constexpr uint32_t stage = 4u * gemv_stage_bytes<BT>(), red = 4u * BT * 4u * 16u;
+    constexpr uint32_t stage = 4u * GemvStreamRegs<kMcg, kNarrow, 1, BT, XLds>::kStageBytes, red = 4u * BT * 4u * 16u;
     return stage > red ? stage : red;
 }
 
 template <int CB, int WIDE, int BT, int NPROJ, bool XLDS, bool ARRIVE, int PROF>
 __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint32_t yidx, uint32_t ksl,
                                           unsigned char* smem, uint32_t& last_flag, uint32_t* cinfo, float* cscore) {
-    // Two tile rows in flight a wave (measured: all 8 in flight is no faster; a call's time is its chain of dependent
-    // round trips, not the depth of one wave's ring)
-    constexpr int ST = 2;
-    constexpr uint32_t kStage = gemv_stage_bytes<BT>();
+    // the register ring: a row-slot's waves walk eight tile rows (the LDS ring pays from about 32 a wave)
+    typedef GemvStreamRegs<CB, WIDE, 1, BT, XLds> StreamL;
+    typedef GemvStreamRegs<CB, WIDE, 1, BT, XGlobal> StreamG;
+    constexpr uint32_t kStage = StreamG::kStageBytes;
     float4v(*red)[BT * 4] = reinterpret_cast<float4v(*)[BT * 4]>(smem);  // the one live row: four lanes a tile a wave
     const uint32_t rk = yidx / NPROJ, proj = yidx % NPROJ;
     const uint32_t sg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
@@ -106,8 +106,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
             extern __shared__ __attribute__((aligned(16))) unsigned char xdyn[];
             unsigned char* xst = xdyn + sg * ((per + 1u) * (kXldsRows * 64u));
             xoff[0] = (lane >> 4) * 16u;
-            GemvStream<CB, WIDE, 1, BT, ST, XLds> stream(wbase, wstep, per, n, a.wbits, XLds{xst}, xoff,
-                                                         smem + sg * kStage, lane);
+            StreamL stream(wbase, wstep, per, n, a.wbits, XLds{xst}, xoff, smem + sg * kStage, lane);
             stream.issue();
             uint32_t hh[2];
             float sum;
@@ -126,8 +125,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
             extern __shared__ __attribute__((aligned(16))) unsigned char xdyn[];
             unsigned char* xst = xdyn + sg * ((per + 1u) * (kXldsRows * 64u));
             xoff[0] = (lane >> 4) * 16u;  // every activation row of the fragment is the slot's one row
-            GemvStream<CB, WIDE, 1, BT, ST, XLds> stream(wbase, wstep, per, n, a.wbits, XLds{xst}, xoff,
-                                                         smem + sg * kStage, lane);
+            StreamL stream(wbase, wstep, per, n, a.wbits, XLds{xst}, xoff, smem + sg * kStage, lane);
             stream.issue();
             const uint16_t* suh = (proj ? bank.up_suh : bank.gate_suh) + static_cast<size_t>(s.e) * a.hidden;
             const uint32_t blocks = per >> 3;
@@ -154,10 +152,10 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
             stream.run(acc);
         } else {
             const uint32_t* xq = NPROJ == 1 ? a.hd : (proj ? a.xu : a.xg);
-            xoff[0] = (rk * in + 4u * (lane >> 4)) * 4u;
-            GemvStream<CB, WIDE, 1, BT, ST, XGlobal> stream(
-                wbase, wstep, per, n, a.wbits, XGlobal{xq, static_cast<uint64_t>(rkt) * in * 4u, tk0 * 64u, 64u}, xoff,
-                smem + sg * kStage, lane);
+            // the fragment's row 0 is the slot's row; the other fifteen stay zero
+            xoff[0] = x_frag_offset(lane, (lane & 15u) == 0u, rk * in * 4u);
+            StreamG stream(wbase, wstep, per, n, a.wbits, XGlobal{xq, static_cast<uint64_t>(rkt) * in * 4u, tk0 * 64u, 64u},
+                           xoff, smem + sg * kStage, lane);
             stream.issue();
             stream.run(acc);
         }
@@ -376,7 +374,7 @@ __global__ void __launch_bounds__(256) moe_group(const MoeLaunch a) {
 
 template <int BT>
 constexpr uint32_t group_lds_bytes() {
-    constexpr uint32_t stage = 4u * gemv_stage_bytes<BT>(), red = 4u * kGroupRows * BT * 4u * 16u;
+    constexpr uint32_t stage = 4u * GemvStreamRegs<kMcg, kNarrow, 1, BT, XGlobal>::kStageBytes, red = 4u * kGroupRows * BT * 4u * 16u;
     return stage > red ? stage : red;
 }
 
@@ -385,8 +383,8 @@ constexpr uint32_t group_lds_bytes() {
 template <int CB, int WIDE, int BT, int NPROJ>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ? 2 : 4))) moe_gemv_grouped(const MoeLaunch a) {
     __shared__ __attribute__((aligned(16))) unsigned char smem[group_lds_bytes<BT>()];
-    constexpr int ST = 2;
-    constexpr uint32_t kStage = gemv_stage_bytes<BT>();
+    typedef GemvStreamRegs<CB, WIDE, 1, BT, XGlobal> StreamG;
+    constexpr uint32_t kStage = StreamG::kStageBytes;
     const uint32_t g = blockIdx.y / NPROJ, proj = blockIdx.y % NPROJ, blk = blockIdx.x, ksl = blockIdx.z;
     if (g >= a.groups[0]) return;  // uniform over the workgroup
     const uint32_t rkt = a.rows * (a.topk + a.shared_slots);
@@ -404,8 +402,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ?
     const uint32_t part = ksl * 4u + sg, tk0 = part * per;
     const uint64_t wstride = static_cast<uint64_t>(out_tiles) * nw;
     const uint32_t* wbase = wmat + static_cast<uint64_t>(blk) * BT * nw + tk0 * wstride;
-    // the lane's activation row: member lane % 16's (a lane past the members reads the first member's: valid memory, its
-    // sums are dropped)
+    // the lane's activation row: member lane % 16's (a row past the members stays zero, its sums are dropped)
     const uint32_t m = lane & 15u;
     const uint32_t rk = member[m < count ? m : 0u];
 
@@ -414,8 +411,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ?
     for (int t = 0; t < BT; ++t) acc[0][t] = float4v{0.f, 0.f, 0.f, 0.f};
     if (part < parts) {  // uniform over the wave; a wave past the last part adds zeros below
         const uint32_t* xq = NPROJ == 1 ? a.hd : (proj ? a.xu : a.xg);
-        uint32_t xoff[1] = {(rk * in + 4u * (lane >> 4)) * 4u};
-        GemvStream<CB, WIDE, 1, BT, ST, XGlobal> stream(
+        uint32_t xoff[1] = {x_frag_offset(lane, m < count, rk * in * 4u)};
+        StreamG stream(
             wbase, static_cast<uint32_t>(wstride) * 4u, per, n, a.wbits,
             XGlobal{xq, static_cast<uint64_t>(rkt) * in * 4u, tk0 * 64u, 64u}, xoff, smem + sg * kStage, lane);
         stream.issue();

@@ -15,6 +15,7 @@
 
 #include "t3_decode.hpp"
 #include "t3_kernels.hpp"
+#include "t3_lds_loads.hpp"
 #include "t3_routed.hpp"
 #include "t3_stages.hpp"
 
@@ -68,33 +69,6 @@ __device__ __forceinline__ uint32_t weight_halves(uint32_t cw_lo, uint32_t cw_hi
     } else {
         return weight_half<CB>(cw_lo) | (weight_half<CB>(cw_hi) << 16);
     }
-}
-
-// ---- loads that bypass the registers --------------------------------------------------------------------------
-// A raw buffer descriptor as four scalars, and a wave's load of 16 bytes a lane from it straight into LDS: lane L's
-// bytes land at lds + 16 L, from byte voff (the lane's) + soff (uniform) of the buffer; past the buffer's end they are
-// zeros. The compiler does not know these loads: the kernel counts them itself (wait_loads) and issues no other
-// vector memory load while they fly.
-__device__ __forceinline__ uint4v rsrc_words(const void* p, uint64_t bytes) {
-    const uint64_t addr = reinterpret_cast<uint64_t>(p);
-    const uint32_t n = bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : static_cast<uint32_t>(bytes);
-    return uint4v{static_cast<uint32_t>(addr), static_cast<uint32_t>(addr >> 32) & 0xFFFFu, n, 0x00020000u};
-}
-// (m0 is named as clobbered so the compiler keeps nothing of its own in it across the statement; clang warns about any
-// reserved register in a clobber list, which is the point here)
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Winline-asm"
-__device__ __forceinline__ void load_to_lds(uint4v desc, uint32_t lds, uint32_t voff, uint32_t soff) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                 :
-                 : "s"(lds), "v"(voff), "s"(desc), "s"(soff)
-                 : "memory", "m0");
-}
-#pragma clang diagnostic pop
-// at most N of the wave's loads are still in flight (they complete in order)
-template <int N>
-__device__ __forceinline__ void wait_loads() {
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
 // Grid (8 * ceil(nblk / spread) * ceil(max_items / (8 / spread)), projections, kparts), 256 threads. Consecutive
