@@ -80,6 +80,36 @@ __device__ __forceinline__ uint32_t weight_pair(uint32_t cw) {
     else return static_cast<uint32_t>(decode_exact<CB>(cw));
 }
 
+// The weight the matrix core takes as one f16 (the GEMMs, and the GEMV's two-tile-row steps): exact, or MUL1's h = 1024 + t when its map is deferred.
+template <int CB>
+__device__ __forceinline__ uint32_t weight_half(uint32_t cw) {
+    if constexpr (CB == kMul1Defer) return mul1_h(cw);
+    else return static_cast<uint32_t>(decode_exact<CB>(cw));
+}
+
+// Two weights as the two halves of one register. MCG: each weight is one f16 add of its hashed pair's halves, and the
+// sub-dword forms of v_add_f16 write the low half, then the high half of the same register (the plain form costs a
+// third instruction to merge them).
+template <int CB>
+__device__ __forceinline__ uint32_t weight_halves(uint32_t cw_lo, uint32_t cw_hi) {
+    if constexpr (CB == kMcg) {
+        const uint32_t pa = mcg_pair(cw_lo), pb = mcg_pair(cw_hi);
+        uint32_t d;
+        asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1"
+            : "=v"(d)
+            : "v"(pa));
+        // the two wait states a sub-dword write needs before a matrix instruction reads the register: the compiler
+        // adds them for its own SDWA instructions, not for this one
+        asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+            "s_nop 1"
+            : "+v"(d)
+            : "v"(pb));
+        return d;
+    } else {
+        return weight_half<CB>(cw_lo) | (weight_half<CB>(cw_hi) << 16);
+    }
+}
+
 // ---- the quad plan --------------------------------------------------------------------------------------------
 
 __device__ __forceinline__ uint32_t quad_first_position(uint32_t lane) {

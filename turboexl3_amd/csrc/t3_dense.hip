@@ -31,10 +31,13 @@ namespace {
 
 enum Fuse : int { kChain = 0, kArrive = 1, kOne = 2 };
 
-// Grid (in / 128, rows), 64 threads. xq: uint32 [in / 16][rows][16], word quad_slot(r) of (tile tk, row) = the f16 value of
-// input tk 16 + r in both halves: the rows of one input tile lie side by side, so the GEMV's fragment of a tile row (64 bytes
-// a row) is one contiguous piece of whole cache lines (with a row's tiles adjacent instead, a 16-row fragment touched 16
-// lines for half of each, and 32 rows cost the K5 GEMV a third of its time). xs: f32 [rows][in / 128].
+// Grid (in / 128, rows), 64 threads. xq: [steps][rows][64 bytes], a step R = 1 or 2 input tiles (the GEMV's codebook form
+// decides, gemv_step_rows): R 1: word quad_slot(r) of (tile, row) = the f16 value of input 16 tile + r in both halves; R 2:
+// the 32 inputs of the tile pair as plain f16 in pair-quad order. The rows of one step lie side by side, so the GEMV's
+// fragment of a step (64 bytes a row) is one contiguous piece of whole cache lines (with a row's tiles adjacent instead, a
+// 16-row fragment touched 16 lines for half of each, and 32 rows cost the K5 GEMV a third of its time).
+// xs: f32 [rows][in / 128].
+template <int R>
 __global__ void __launch_bounds__(64) dense_prep(const void* x, const uint16_t* suh, uint32_t* xq, float* xs,
                                                  uint32_t in, int dt) {
     const uint32_t b = blockIdx.x, row = blockIdx.y, lane = threadIdx.x;
@@ -43,8 +46,8 @@ __global__ void __launch_bounds__(64) dense_prep(const void* x, const uint16_t* 
     prep_values(dt, x, suh, in, row, b, lane, hv, sum);
 #pragma unroll
     for (uint32_t j = 0; j < 2u; ++j) {
-        const uint32_t i = b * 128u + lane + 64u * j;
-        xq[(static_cast<size_t>(i >> 4) * gridDim.y + row) * 16u + quad_slot(i & 15u)] = hv[j] | (hv[j] << 16);
+        const uint32_t i = b * 128u + lane + 64u * j, step = i / (16u * R), e = i % (16u * R);
+        x_step_store<R>(reinterpret_cast<unsigned char*>(xq) + (static_cast<size_t>(step) * gridDim.y + row) * 64u, e, hv[j]);
     }
     if (lane == 0u) xs[static_cast<size_t>(row) * (in / 128u) + b] = sum;
 }
@@ -141,6 +144,7 @@ __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
     typedef GemvStream<LDS, CB, WIDE, RB, BT, XLds> StreamL;
     typedef GemvStream<LDS, CB, WIDE, RB, BT, XGlobal> StreamG;
     constexpr uint32_t kStage = StreamG::kStageBytes;
+    constexpr int R = gemv_step_rows<CB>();   // tile rows a step
     constexpr uint32_t kRed = 4u * RB * BT * 64u * 16u;
     constexpr uint32_t kMain = kRed > 4u * kStage ? kRed : 4u * kStage;
     // the waves' LDS rings while they stream; the four waves' partial sums afterwards
@@ -172,13 +176,14 @@ __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
     if constexpr (FUSE == kOne) {
         static_assert(FUSE != kOne || RB == 1, "the one-launch form serves up to 4 rows");
         extern __shared__ __attribute__((aligned(16))) unsigned char xdyn[];
-        unsigned char* xst = xdyn + sg * ((per + 1u) * (kXldsRows * 64u));
+        const uint32_t steps = per / R;
+        unsigned char* xst = xdyn + sg * ((steps + 1u) * (kXldsRows * 64u));
         const uint32_t row = lane & 15u;
         xoff[0] = (row < rows ? row : 0u) * 64u + (lane >> 4) * 16u;
         StreamL stream(wbase, wstep, per, a.n, a.wbits, XLds{xst}, xoff, smem + sg * kStage, lane);
         stream.issue();
         // While the codes fly, the wave prepares its own K part: per / 8 whole 128-blocks a row, the statements of
-        // dense_prep, into its LDS x stage [per + 1][4][64 bytes] (the last tile row zeros). The block sums go to the
+        // dense_prep, into its LDS x stage [steps + 1][4][64 bytes] (the last step zeros). The block sums go to the
         // column block's own copy of xs (deferred MUL1 map only; the block's second workgroup column, if any, would
         // store the same values again).
         // Every row's loads go out together (rows and blocks past the call's alias the last real one, so there is no
@@ -213,16 +218,15 @@ __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
                 prep_core(v, lane, hv, sum, a.defer != 0);
 #pragma unroll
                 for (uint32_t j = 0; j < 2u; ++j) {
-                    const uint32_t i = lane + 64u * j;  // element of the block: tile row b 8 + i / 16
-                    const uint32_t at = ((b * 8u + (i >> 4)) * kXldsRows + r) * 64u + quad_slot(i & 15u) * 4u;
-                    *reinterpret_cast<uint32_t*>(xst + at) = hv[j] | (hv[j] << 16);
+                    const uint32_t i = b * 128u + lane + 64u * j;  // element of the wave's K part: step i / (16 R)
+                    x_step_store<R>(xst + ((i / (16u * R)) * kXldsRows + r) * 64u, i % (16u * R), hv[j]);
                 }
                 if (a.defer && lane == 0u && blk % kShare == 0u)
                     store_coherent(a.xs + (static_cast<size_t>(b128) * rows + r) * inblk + (tk0 >> 3) + b, sum);
             }
         }
         for (uint32_t i = lane; i < kXldsRows * 16u; i += 64u)
-            *reinterpret_cast<uint32_t*>(xst + per * (kXldsRows * 64u) + i * 4u) = 0u;
+            *reinterpret_cast<uint32_t*>(xst + steps * (kXldsRows * 64u) + i * 4u) = 0u;
         stream.run(acc);
     } else {
 #pragma unroll
@@ -231,8 +235,8 @@ __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
             xoff[r] = x_frag_offset(lane, row < rows, row * 64u);
         }
         StreamG stream(wbase, wstep, per, a.n, a.wbits,
-                       XGlobal{a.xq, static_cast<uint64_t>(rows) * a.in * 4u, tk0 * rows * 64u, rows * 64u}, xoff,
-                       smem + sg * kStage, lane);
+                       XGlobal{a.xq, static_cast<uint64_t>(rows) * (a.in / (16u * R)) * 64u, (tk0 / R) * rows * 64u, rows * 64u},
+                       xoff, smem + sg * kStage, lane);
         stream.issue();
         stream.run(acc);
     }
@@ -310,7 +314,7 @@ hipError_t launch_gemv_fuse(const DenseLaunch& d, int fuse, hipStream_t s) {
     if (fuse == kOne) {
         if constexpr (RB == 1) {
             // the one-launch form serves waves of 8 or 16 tile rows: below the LDS ring's bound
-            const size_t dyn = 4u * (a.per + 1u) * (kXldsRows * 64u);
+            const size_t dyn = 4u * (a.per / gemv_step_rows<CB>() + 1u) * (kXldsRows * 64u);
             hipLaunchKernelGGL((dense_gemv<CB, WIDE, 1, BT, kOne, false>), grid, block, dyn, s, a);
         } else {
             return hipErrorInvalidValue;
@@ -362,7 +366,12 @@ hipError_t launch_bias_add(void* y, const void* bias, uint32_t rows, uint32_t ou
 }
 
 hipError_t launch_dense_prep(const DenseLaunch& d, hipStream_t s) {
-    hipLaunchKernelGGL(dense_prep, dim3(d.in / 128u, d.rows), dim3(64), 0, s, d.x, d.suh, d.xq, d.xs, d.in, d.dtype);
+    // the layout the GEMV of this codebook form reads
+    const bool two = d.codebook == kMcg || d.codebook == kMul1;
+    static_assert(gemv_step_rows<kMcg>() == 2 && gemv_step_rows<kMul1>() == 2 && gemv_step_rows<kMcgPair>() == 1 &&
+                  gemv_step_rows<kMul1Defer>() == 1);
+    if (two) hipLaunchKernelGGL(dense_prep<2>, dim3(d.in / 128u, d.rows), dim3(64), 0, s, d.x, d.suh, d.xq, d.xs, d.in, d.dtype);
+    else hipLaunchKernelGGL(dense_prep<1>, dim3(d.in / 128u, d.rows), dim3(64), 0, s, d.x, d.suh, d.xq, d.xs, d.in, d.dtype);
     return hipGetLastError();
 }
 

@@ -91,6 +91,7 @@ constexpr uint32_t kGemvMinPer = 4;      // input tiles a wave at least
 // K slices of a GEMV over in_tiles input tiles and `groups` workgroup columns: the smallest divisor d of
 // in_tiles / 4 that reaches the target workgroup count while every wave keeps kGemvMinPer tiles. Splits that leave a
 // wave whole 128-blocks of the input (per % 8 == 0) are preferred: the one-launch form prepares its input by block.
+// Every split leaves a wave an even number of tiles: the f16-weight codebook forms walk two tile rows a step.
 inline uint32_t gemv_slices(uint32_t in_tiles, uint32_t groups) {
     const uint32_t q = in_tiles / 4u;
     for (int whole = 1; whole >= 0; --whole) {
@@ -99,6 +100,7 @@ inline uint32_t gemv_slices(uint32_t in_tiles, uint32_t groups) {
             if (q % d != 0) continue;
             const uint32_t per = q / d;
             if (per < kGemvMinPer && d > 1) break;
+            if (per % 2u != 0u) continue;
             if (whole && per % 8u != 0u) continue;
             best = d;
             if (static_cast<uint64_t>(groups) * d >= kGemvTargetWgs) break;

@@ -85,6 +85,8 @@ struct MoeLaunch {
     uint32_t n_gu = 0, n_dn = 0, wbits = 16;
     uint32_t per_gu = 8, per_dn = 8, parts_gu = 0, parts_dn = 0, ks_gu = 1, ks_dn = 1, bt_gu = 8, bt_dn = 8;
     int codebook = 0, dtype = 0, score_dt = 0, defer = 0;
+    int pair_order = 0;  // decode rows: the GEMVs take two tile rows a step (the f16-weight codebook forms) and read their
+                         // activations as plain f16 in pair-quad order; else one, doubled f16 in quad order
     float limit = 0.0f;
     int clamp_at = 0;  // format.ClampAt: 0 gate_in (the gate clamped before its SiLU), 1 silu_out (the SiLU's output)
     // prefill only (the route's roles, src/hip/plan.zig:40-45): row-slots sorted by expert. order [P] position ->

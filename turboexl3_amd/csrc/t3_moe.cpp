@@ -119,6 +119,7 @@ int32_t check_moe(const t3_array* x, const t3_bank* bank, const t3_array* inds, 
     l.wbits = d.wbits;
     l.codebook = d.gemv_form;
     l.defer = d.gemv_form == 2;
+    l.pair_order = d.gemv_form == 0 || d.gemv_form == 1;  // the f16-weight forms: two tile rows a GEMV step
     l.dtype = x->dtype;
     l.limit = static_cast<float>(limit);
     l.clamp_at = clamp_at;

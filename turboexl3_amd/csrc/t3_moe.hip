@@ -62,6 +62,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
     typedef GemvStreamRegs<CB, WIDE, 1, BT, XLds> StreamL;
     typedef GemvStreamRegs<CB, WIDE, 1, BT, XGlobal> StreamG;
     constexpr uint32_t kStage = StreamG::kStageBytes;
+    constexpr int R = gemv_step_rows<CB>();   // tile rows a step
     float4v(*red)[BT * 4] = reinterpret_cast<float4v(*)[BT * 4]>(smem);  // the one live row: four lanes a tile a wave
     const uint32_t rk = yidx / NPROJ, proj = yidx % NPROJ;
     const uint32_t sg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
@@ -104,26 +105,29 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
             // The down's input made here: the wave runs the mid stage of its own 128-block (its eight input tiles) over
             // the gate|up launch's planes and keeps the prepared block in LDS.
             extern __shared__ __attribute__((aligned(16))) unsigned char xdyn[];
-            unsigned char* xst = xdyn + sg * ((per + 1u) * (kXldsRows * 64u));
+            const uint32_t steps = per / R;
+            unsigned char* xst = xdyn + sg * ((steps + 1u) * (kXldsRows * 64u));
             xoff[0] = (lane >> 4) * 16u;
             StreamL stream(wbase, wstep, per, n, a.wbits, XLds{xst}, xoff, smem + sg * kStage, lane);
             stream.issue();
             uint32_t hh[2];
             float sum;
             routed_mid_values<false, false, PROF>(a, s, rk, tk0 >> 3, lane, hh, sum);
-            // element 64 j + lane of the block belongs to its tile row 4 j + lane / 16
+            // element i = 64 j + lane of the block belongs to step i / (16 R) of the wave's walk
 #pragma unroll
-            for (uint32_t j = 0; j < 2u; ++j)
-                *reinterpret_cast<uint32_t*>(xst + ((4u * j + (lane >> 4)) * kXldsRows) * 64u + quad_slot(lane & 15u) * 4u) =
-                    hh[j] | (hh[j] << 16);
+            for (uint32_t j = 0; j < 2u; ++j) {
+                const uint32_t i = 64u * j + lane;
+                x_step_store<R>(xst + ((i / (16u * R)) * kXldsRows) * 64u, i % (16u * R), hh[j]);
+            }
             // every column workgroup of the slot stores the same sum; the row's combine, later in this launch, reads it
             if (a.defer && lane == 0u) store_coherent(a.hs + static_cast<size_t>(rk) * (a.inter / 128u) + (tk0 >> 3), sum);
             for (uint32_t i = lane; i < kXldsRows * 16u; i += 64u)
-                *reinterpret_cast<uint32_t*>(xst + per * (kXldsRows * 64u) + i * 4u) = 0u;
+                *reinterpret_cast<uint32_t*>(xst + steps * (kXldsRows * 64u) + i * 4u) = 0u;
             stream.run(acc);
         } else if constexpr (XLDS) {
             extern __shared__ __attribute__((aligned(16))) unsigned char xdyn[];
-            unsigned char* xst = xdyn + sg * ((per + 1u) * (kXldsRows * 64u));
+            const uint32_t steps = per / R;
+            unsigned char* xst = xdyn + sg * ((steps + 1u) * (kXldsRows * 64u));
             xoff[0] = (lane >> 4) * 16u;  // every activation row of the fragment is the slot's one row
             StreamL stream(wbase, wstep, per, n, a.wbits, XLds{xst}, xoff, smem + sg * kStage, lane);
             stream.issue();
@@ -135,9 +139,8 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
                 prep_values(a.dtype, a.x, suh, a.hidden, s.row, (tk0 >> 3) + b, lane, hv, sum, PROF == 0);
 #pragma unroll
                 for (uint32_t j = 0; j < 2u; ++j) {
-                    const uint32_t i = lane + 64u * j;
-                    const uint32_t at = ((b * 8u + (i >> 4)) * kXldsRows) * 64u + quad_slot(i & 15u) * 4u;
-                    *reinterpret_cast<uint32_t*>(xst + at) = hv[j] | (hv[j] << 16);
+                    const uint32_t i = b * 128u + lane + 64u * j;  // element of the wave's K part
+                    x_step_store<R>(xst + ((i / (16u * R)) * kXldsRows) * 64u, i % (16u * R), hv[j]);
                 }
                 // every column workgroup of the slot stores the same sum: a handful of plain stores, read by the
                 // next launch
@@ -148,14 +151,17 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
                 }
             }
             for (uint32_t i = lane; i < kXldsRows * 16u; i += 64u)
-                *reinterpret_cast<uint32_t*>(xst + per * (kXldsRows * 64u) + i * 4u) = 0u;
+                *reinterpret_cast<uint32_t*>(xst + steps * (kXldsRows * 64u) + i * 4u) = 0u;
             stream.run(acc);
         } else {
             const uint32_t* xq = NPROJ == 1 ? a.hd : (proj ? a.xu : a.xg);
-            // the fragment's row 0 is the slot's row; the other fifteen stay zero
-            xoff[0] = x_frag_offset(lane, (lane & 15u) == 0u, rk * in * 4u);
-            StreamG stream(wbase, wstep, per, n, a.wbits, XGlobal{xq, static_cast<uint64_t>(rkt) * in * 4u, tk0 * 64u, 64u},
-                           xoff, smem + sg * kStage, lane);
+            // a row-slot's prepared inputs: 4 bytes an input (doubled f16) at one tile row a step, 2 (plain f16) at two:
+            // 64 bytes a step either way. The fragment's row 0 is the slot's row; the other fifteen stay zero.
+            constexpr uint32_t kIn = R == 1 ? 4u : 2u;
+            xoff[0] = x_frag_offset(lane, (lane & 15u) == 0u, rk * in * kIn);
+            StreamG stream(wbase, wstep, per, n, a.wbits,
+                           XGlobal{xq, static_cast<uint64_t>(rkt) * in * kIn, (tk0 / R) * 64u, 64u}, xoff, smem + sg * kStage,
+                           lane);
             stream.issue();
             stream.run(acc);
         }
@@ -270,7 +276,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
 }
 
 template <int CB, int WIDE, int BT, int NPROJ, bool XLDS, bool ARRIVE, int PROF>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ? 2 : 4))) moe_gemv(const MoeLaunch a) {
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ? 2 : (gemv_step_rows<CB>() == 2 ? 3 : 4)))) moe_gemv(const MoeLaunch a) {
     __shared__ __attribute__((aligned(16))) unsigned char smem[role_lds_bytes<BT>()];
     __shared__ uint32_t last_flag, cinfo[64];
     __shared__ float cscore[64];
@@ -381,7 +387,7 @@ constexpr uint32_t group_lds_bytes() {
 // Grid (out / 16 / BT, RKT * NPROJ, KS), 256 threads: workgroup row y serves group y / NPROJ (none past the table's count)
 // as moe_gemv serves a row-slot, from the prepared rows of the five-launch form, z [KS][RKT][out] by member.
 template <int CB, int WIDE, int BT, int NPROJ>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ? 2 : 4))) moe_gemv_grouped(const MoeLaunch a) {
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ? 2 : (gemv_step_rows<CB>() == 2 ? 3 : 4)))) moe_gemv_grouped(const MoeLaunch a) {
     __shared__ __attribute__((aligned(16))) unsigned char smem[group_lds_bytes<BT>()];
     typedef GemvStreamRegs<CB, WIDE, 1, BT, XGlobal> StreamG;
     constexpr uint32_t kStage = StreamG::kStageBytes;
@@ -411,10 +417,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ?
     for (int t = 0; t < BT; ++t) acc[0][t] = float4v{0.f, 0.f, 0.f, 0.f};
     if (part < parts) {  // uniform over the wave; a wave past the last part adds zeros below
         const uint32_t* xq = NPROJ == 1 ? a.hd : (proj ? a.xu : a.xg);
-        uint32_t xoff[1] = {x_frag_offset(lane, m < count, rk * in * 4u)};
+        constexpr int R = gemv_step_rows<CB>();
+        constexpr uint32_t kIn = R == 1 ? 4u : 2u;  // bytes a prepared input (moe_gemv's XGlobal form)
+        uint32_t xoff[1] = {x_frag_offset(lane, m < count, rk * in * kIn)};
         StreamG stream(
             wbase, static_cast<uint32_t>(wstride) * 4u, per, n, a.wbits,
-            XGlobal{xq, static_cast<uint64_t>(rkt) * in * 4u, tk0 * 64u, 64u}, xoff, smem + sg * kStage, lane);
+            XGlobal{xq, static_cast<uint64_t>(rkt) * in * kIn, (tk0 / R) * 64u, 64u}, xoff, smem + sg * kStage, lane);
         stream.issue();
         stream.run(acc);
     }
@@ -452,7 +460,7 @@ hipError_t launch_gemv_bt(const MoeLaunch& a, hipStream_t s) {
     const uint32_t bt = NPROJ == 2 ? a.bt_gu : a.bt_dn, ks = NPROJ == 2 ? a.ks_gu : a.ks_dn;
     const uint32_t rkt = a.rows * (a.topk + a.shared_slots);
     const dim3 grid((out / 16u) / bt, rkt * NPROJ, ks), block(256);
-    const size_t dyn = XLDS ? 4u * ((NPROJ == 2 ? a.per_gu : a.per_dn) + 1u) * (kXldsRows * 64u) : 0u;
+    const size_t dyn = XLDS ? 4u * ((NPROJ == 2 ? a.per_gu : a.per_dn) / gemv_step_rows<CB>() + 1u) * (kXldsRows * 64u) : 0u;
     if constexpr (WIDE == kNarrow) {
         if (bt == 8u) {
             hipLaunchKernelGGL((moe_gemv<CB, WIDE, 8, NPROJ, XLDS, ARRIVE, PROF>), grid, block, dyn, s, a);

@@ -41,36 +41,6 @@ struct PfGemm {
                       // a finish that starts by rounding them (no deferred map, not GLM's profile)
 };
 
-// The weight a GEMM feeds the matrix core as one f16: exact, or MUL1's h = 1024 + t when its map is deferred.
-template <int CB>
-__device__ __forceinline__ uint32_t weight_half(uint32_t cw) {
-    if constexpr (CB == kMul1Defer) return mul1_h(cw);
-    else return static_cast<uint32_t>(decode_exact<CB>(cw));
-}
-
-// Two weights as the two halves of one register. MCG: each weight is one f16 add of its hashed pair's halves, and the
-// sub-dword forms of v_add_f16 write the low half, then the high half of the same register (the plain form costs a
-// third instruction to merge them).
-template <int CB>
-__device__ __forceinline__ uint32_t weight_halves(uint32_t cw_lo, uint32_t cw_hi) {
-    if constexpr (CB == kMcg) {
-        const uint32_t pa = mcg_pair(cw_lo), pb = mcg_pair(cw_hi);
-        uint32_t d;
-        asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1"
-            : "=v"(d)
-            : "v"(pa));
-        // the two wait states a sub-dword write needs before a matrix instruction reads the register: the compiler
-        // adds them for its own SDWA instructions, not for this one
-        asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1\n\t"
-            "s_nop 1"
-            : "+v"(d)
-            : "v"(pb));
-        return d;
-    } else {
-        return weight_half<CB>(cw_lo) | (weight_half<CB>(cw_hi) << 16);
-    }
-}
-
 // Grid (8 * ceil(nblk / spread) * ceil(max_items / (8 / spread)), projections, kparts), 256 threads. Consecutive
 // workgroup ids go round the eight dies, so the workgroups that share an item's activations (its nblk column blocks)
 // are given ids 8 apart: one die's L2 serves them all. With fewer than eight items that would leave dies idle (one item:

@@ -133,11 +133,12 @@ __device__ __forceinline__ void plane_sums(const float* z, size_t planes_stride,
 // ---- the routed chain's per-block stages ----------------------------------------------------------------------
 // One wave a 128-block. rk: the row-slot; q: where its scratch lives (decode rows: q = rk; prefill: its position in
 // the expert-sorted order). PF = prefill: the prepared activations are plain f16 (the GEMM's B fragments), one plane a
-// projection; else u32 with the f16 in both halves (the GEMV's pairs of K slots) and ks planes.
+// projection; else ks planes, and the activations as the GEMV's codebook form reads them (a.pair_order: plain f16 in
+// pair-quad order as well, two tile rows a step; else u32 with the f16 in both halves, the pairs of K slots).
 
 template <bool PF>
-__device__ __forceinline__ void store_prepared(uint32_t* base, size_t row_at, uint32_t i, uint32_t hbits) {
-    if constexpr (PF) reinterpret_cast<uint16_t*>(base)[row_at + pair_quad_slot(i)] = static_cast<uint16_t>(hbits);
+__device__ __forceinline__ void store_prepared(const MoeLaunch& a, uint32_t* base, size_t row_at, uint32_t i, uint32_t hbits) {
+    if (PF || a.pair_order) reinterpret_cast<uint16_t*>(base)[row_at + pair_quad_slot(i)] = static_cast<uint16_t>(hbits);
     else base[row_at + (i & ~15u) + quad_slot(i & 15u)] = hbits | (hbits << 16);
 }
 
@@ -157,7 +158,7 @@ __device__ __forceinline__ void routed_prep_block(const MoeLaunch& a, uint32_t r
         prep_values(a.dtype, a.x, suh, a.hidden, s.row, b, lane, hv, sum, PROF == 0);
 #pragma unroll
         for (uint32_t j = 0; j < 2u; ++j)
-            store_prepared<PF>(proj ? a.xu : a.xg, static_cast<size_t>(q) * a.hidden, b * 128u + lane + 64u * j, hv[j]);
+            store_prepared<PF>(a, proj ? a.xu : a.xg, static_cast<size_t>(q) * a.hidden, b * 128u + lane + 64u * j, hv[j]);
         if (lane == 0u) (proj ? a.su : a.sg)[static_cast<size_t>(q) * nb + b] = sum;
     }
 }
@@ -229,7 +230,7 @@ __device__ __forceinline__ void routed_mid_block(const MoeLaunch& a, const SlotR
     routed_mid_values<PF, COH, PROF>(a, s, q, b, lane, hh, sum);
 #pragma unroll
     for (uint32_t j = 0; j < 2u; ++j)
-        store_prepared<PF>(a.hd, static_cast<size_t>(q) * a.inter, b * 128u + lane + 64u * j, hh[j]);
+        store_prepared<PF>(a, a.hd, static_cast<size_t>(q) * a.inter, b * 128u + lane + 64u * j, hh[j]);
     if (lane == 0u) a.hs[static_cast<size_t>(q) * (a.inter / 128u) + b] = sum;
 }
 
