@@ -110,6 +110,9 @@ struct MoeLaunch {
 // Or six: the five behind a grouping launch, the row-slots that read one expert served together (up to 16 a group), so
 // the expert's tiles are decoded once for all of them. The same bytes again: an output column of the matrix core depends
 // on its own activation row alone.
+// Rows up to which the two-launch form runs the mid stage inside the down launch (every down wave for its own
+// 128-block) and shapes both launches for few, long waves (t3_moe.hip)
+constexpr uint32_t kMoeFewRows = 4;
 enum MoeForm : int { kMoeFiveLaunches = 0, kMoeFourLaunches = 1, kMoeTwoLaunches = 2, kMoeGrouped = 3 };
 hipError_t launch_moe_decode(const MoeLaunch& a, int form, hipStream_t s);
 // a row's top-k experts by logit (ties to the lowest id) and their renormalised softmax weights in the logits' dtype

@@ -135,6 +135,14 @@ int32_t check_moe(const t3_array* x, const t3_bank* bank, const t3_array* inds, 
     l.per_dn = 8;
     l.parts_dn = (l.inter / 16u) / l.per_dn;
     l.ks_dn = (l.parts_dn + 3u) / 4u;
+    // Up to kMoeFewRows rows the launches' waves are few and long against the call's chain of round trips: the gate|up
+    // launch then takes four tiles a load (twice the workgroups of half the length; 512 experts of 2048 x 512 at one to
+    // four tokens, the launch alone: 9.6 / 11.9 / 16.8 / 19.5 -> 8.2 / 11.4 / 15.7 / 18.8 us). The down launch keeps eight: its
+    // workgroups count in at a counter a 128-column block, and twice the arrivals cost it more (one token 15.3 -> 15.8 us).
+    // A column's sums do not depend on the tiles a load, so a row's bytes stay those of the row alone. (Where the gate|up
+    // launch is small at eight tiles, within 2048 workgroups: large experts fill the GPU at one row already.)
+    const uint64_t gu_wgs = static_cast<uint64_t>(l.inter / 128u) * l.rows * (l.topk + l.shared_slots) * 2u * l.ks_gu;
+    if (l.rows <= kMoeFewRows && l.bt_gu == 8u && gu_wgs <= 2048u) l.bt_gu = 4u;
     return T3_OK;
 }
 
@@ -222,7 +230,8 @@ int decode_form_of(const MoeLaunch& l) {
     if (want == 3 || want == 7) return kMoeFiveLaunches;
     if (want == 5 || want == 6) return kMoeGrouped;
     if (want == 8 || counters * 4u > kCounterBytes) return kMoeFourLaunches;
-    const uint64_t gu_groups = static_cast<uint64_t>(l.inter / 16u / l.bt_gu) * rkt * 2u * l.ks_gu;
+    // (workgroups at the rate's own tiles a load: the few-row calls' four tiles do not move the bound)
+    const uint64_t gu_groups = static_cast<uint64_t>(l.inter / 16u / gemv_bt(l.n_gu)) * rkt * 2u * l.ks_gu;
     // where the decode dominates, the row-slots that read one expert are served together (a grouping launch in front):
     // every row-slot alone at worst, an expert's tiles decoded once for up to sixteen rows at best
     if (gu_groups > kTwoLaunchGroups) return l.rows >= 2u ? kMoeGrouped : kMoeFiveLaunches;

@@ -40,13 +40,16 @@ __global__ void __launch_bounds__(64) moe_prep(const MoeLaunch a) {
 // a launch but is run by all sixteen column workgroups of a slot. Measured against the arriving gate|up launch with
 // eight tiles a down wave (us a call): 3 rows 35.0 against 35.5, 4 rows 38.0 against 38.6, 8 rows 57.9 against 56.0,
 // 16 rows 98.6 against 94.7: served up to kMidInDownRows = 4 rows. (With four tiles a down wave, an earlier form, it won
-// up to two rows only: one row 25.3 against 26.5, two 29.7 against 31.2, three 38.0 against 37.3.)
+// up to two rows only: one row 25.3 against 26.5, two 29.7 against 31.2, three 38.0 against 37.3.) A workgroup of eight
+// waves over the same 128 columns (four tiles a load a wave, two column groups: the arrivals a counter unchanged, the
+// waves half as long) was measured for this launch as well: one row 15.3 -> 15.0 us, two 16.4 -> 17.5, three 18.3 ->
+// 21.4: every wave of a slot repeats the mid stage, and eight of them do it where four did. Taken out.
 //
 // ARRIVE: the launch also runs the stage after it. The planes are stored device-coherently, every workgroup counts
 // itself in at its 128-column block, and the last to arrive runs that block's next stage on the complete planes:
 // gate|up -> the slot's mid block (counter a (row-slot, block of inter)); down -> the row's combine block (counter a
 // (row, block of hidden); skipped slots count themselves in too). The statements are the chain's, so are the bytes.
-constexpr uint32_t kMidInDownRows = 4u;
+constexpr uint32_t kMidInDownRows = kMoeFewRows;
 
 // a workgroup's static LDS: the four waves' rings while they stream, their partial sums afterwards
 template <int BT>
@@ -153,6 +156,9 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
             for (uint32_t i = lane; i < kXldsRows * 16u; i += 64u)
                 *reinterpret_cast<uint32_t*>(xst + steps * (kXldsRows * 64u) + i * 4u) = 0u;
             stream.run(acc);
+            // (Touching the slot's down trellis from here, so that the down launch behind this one finds it in the
+            // memory-side cache, was measured: a piece a wave, the loads left to land by themselves. This launch 8.2 ->
+            // 8.9 us at one token, the down launch no shorter, the call 23.65 -> 23.97 us. Taken out.)
         } else {
             const uint32_t* xq = NPROJ == 1 ? a.hd : (proj ? a.xu : a.xg);
             // a row-slot's prepared inputs: 4 bytes an input (doubled f16) at one tile row a step, 2 (plain f16) at two:
