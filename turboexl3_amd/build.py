@@ -60,7 +60,9 @@ def _compile(src: str, force: bool) -> str:
     path = os.path.join(CSRC, src)
     if not force and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(path), _headers_mtime()):
         return obj
-    cmd = [hipcc(), "-x", "hip", *COMMON, *HIP_FLAGS, "-c", path, "-o", obj]
+    # T3_EXTRA_HIPCC_FLAGS: build-time switches of the measured variants (e.g. -DT3_GEMV_LDS_RING_FROM=0)
+    extra = os.environ.get("T3_EXTRA_HIPCC_FLAGS", "").split()
+    cmd = [hipcc(), "-x", "hip", *COMMON, *HIP_FLAGS, *extra, "-c", path, "-o", obj]
     cmd[-4:-4] = ["-Rpass-analysis=kernel-resource-usage", "-fno-caret-diagnostics"]  # remarks without source lines
     res = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in res.stderr.splitlines()

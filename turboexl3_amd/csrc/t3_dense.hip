@@ -139,6 +139,10 @@ struct GemvArgs {
 // divide). RB = 16-row blocks of x (1 or 2). z f32 [KS][rows][out]: the four waves' sums, wave 0 first.
 // LDS: the tiles go from memory straight into an LDS ring (served where a wave's walk is long, dense_gemv_lds_ring);
 // else through the register ring.
+// A persistent form of this grid (a workgroup looping over two or three column blocks, everything else unchanged) was
+// measured at 4096 x 12288 K4, one row: 14.9 us a call with 768 workgroups of one block each, 20.3 with 384 of two, 25.4
+// with 256 of three. Every workgroup of the launch is resident from its first cycle as it is; fewer, longer ones only
+// put the column blocks' chains of round trips (first bytes, hand-off, finish) one behind the other.
 template <int CB, int WIDE, int RB, int BT, int FUSE, bool LDS>
 __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
     typedef GemvStream<LDS, CB, WIDE, RB, BT, XLds> StreamL;
@@ -313,9 +317,10 @@ hipError_t launch_gemv_fuse(const DenseLaunch& d, int fuse, hipStream_t s) {
     const bool lds = dense_gemv_lds_ring(a.per);
     if (fuse == kOne) {
         if constexpr (RB == 1) {
-            // the one-launch form serves waves of 8 or 16 tile rows: below the LDS ring's bound
+            // (the one-launch form serves waves of 8 or 16 tile rows: below the LDS ring's served bound)
             const size_t dyn = 4u * (a.per / gemv_step_rows<CB>() + 1u) * (kXldsRows * 64u);
-            hipLaunchKernelGGL((dense_gemv<CB, WIDE, 1, BT, kOne, false>), grid, block, dyn, s, a);
+            if (lds) hipLaunchKernelGGL((dense_gemv<CB, WIDE, 1, BT, kOne, true>), grid, block, dyn, s, a);
+            else hipLaunchKernelGGL((dense_gemv<CB, WIDE, 1, BT, kOne, false>), grid, block, dyn, s, a);
         } else {
             return hipErrorInvalidValue;
         }

@@ -340,7 +340,10 @@ struct GemvStreamRegs {
 
 template <int CB, int WIDE, int RB, int BT, typename XSrc>
 struct GemvStreamLds {
-    static constexpr int ST = 4;                      // steps' slots in the LDS ring: ST - 1 steps in flight under a decode
+#ifndef T3_GEMV_LDS_RING_DEPTH
+#define T3_GEMV_LDS_RING_DEPTH 4
+#endif
+    static constexpr int ST = T3_GEMV_LDS_RING_DEPTH;  // steps' slots in the LDS ring: ST - 1 steps in flight under a decode
     static constexpr int R = gemv_step_rows<CB>();   // tile rows a step
     static constexpr bool kAhead = R == 1;            // as GemvStreamRegs: a second set of words, read a step ahead
     static constexpr uint32_t kSlotBytes = static_cast<uint32_t>(R) * kRowSlot;   // LDS bytes a step

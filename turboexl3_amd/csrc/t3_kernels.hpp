@@ -33,7 +33,12 @@ enum DenseFuse : int { kFuseChain = 0, kFuseArrive = 1, kFuseOne = 2 };
 // Whether a dense GEMV whose waves walk `per` tile rows each takes its tiles through the direct-to-LDS ring (four rows'
 // slots a wave) rather than the register ring: the LDS ring pays where a wave's walk is long (one row of 4096 x 151936,
 // 64 tile rows a wave: the GEMV launch 4-6 % shorter at K3..K6) and costs a launch of 8 or 16 tile rows a wave 1-3 %.
-inline bool dense_gemv_lds_ring(uint32_t per) { return per >= 32u; }
+// (T3_GEMV_LDS_RING_FROM: a build-time override for measuring one form everywhere; 0 also puts the routed GEMVs, whose
+// waves walk eight tile rows, on the LDS ring.)
+#ifndef T3_GEMV_LDS_RING_FROM
+#define T3_GEMV_LDS_RING_FROM 32
+#endif
+inline bool dense_gemv_lds_ring(uint32_t per) { return per >= static_cast<uint32_t>(T3_GEMV_LDS_RING_FROM); }
 
 hipError_t launch_dense_prep(const DenseLaunch& d, hipStream_t s);
 hipError_t launch_dense_gemv(const DenseLaunch& d, int fuse, hipStream_t s);

@@ -51,19 +51,21 @@ __global__ void __launch_bounds__(64) moe_prep(const MoeLaunch a) {
 // (row, block of hidden); skipped slots count themselves in too). The statements are the chain's, so are the bytes.
 constexpr uint32_t kMidInDownRows = kMoeFewRows;
 
+// the register ring: a row-slot's waves walk eight tile rows (the LDS ring pays from about 32 a wave)
+constexpr bool kMoeLdsRing = T3_GEMV_LDS_RING_FROM <= 8;
+
 // a workgroup's static LDS: the four waves' rings while they stream, their partial sums afterwards
 template <int BT>
 constexpr uint32_t role_lds_bytes() {
-    constexpr uint32_t stage = 4u * GemvStreamRegs<kMcg, kNarrow, 1, BT, XLds>::kStageBytes, red = 4u * BT * 4u * 16u;
+    constexpr uint32_t stage = 4u * GemvStream<kMoeLdsRing, kMcg, kNarrow, 1, BT, XLds>::kStageBytes, red = 4u * BT * 4u * 16u;
     return stage > red ? stage : red;
 }
 
 template <int CB, int WIDE, int BT, int NPROJ, bool XLDS, bool ARRIVE, int PROF>
 __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint32_t yidx, uint32_t ksl,
                                           unsigned char* smem, uint32_t& last_flag, uint32_t* cinfo, float* cscore) {
-    // the register ring: a row-slot's waves walk eight tile rows (the LDS ring pays from about 32 a wave)
-    typedef GemvStreamRegs<CB, WIDE, 1, BT, XLds> StreamL;
-    typedef GemvStreamRegs<CB, WIDE, 1, BT, XGlobal> StreamG;
+    typedef GemvStream<kMoeLdsRing, CB, WIDE, 1, BT, XLds> StreamL;
+    typedef GemvStream<kMoeLdsRing, CB, WIDE, 1, BT, XGlobal> StreamG;
     constexpr uint32_t kStage = StreamG::kStageBytes;
     constexpr int R = gemv_step_rows<CB>();   // tile rows a step
     float4v(*red)[BT * 4] = reinterpret_cast<float4v(*)[BT * 4]>(smem);  // the one live row: four lanes a tile a wave
@@ -386,7 +388,7 @@ __global__ void __launch_bounds__(256) moe_group(const MoeLaunch a) {
 
 template <int BT>
 constexpr uint32_t group_lds_bytes() {
-    constexpr uint32_t stage = 4u * GemvStreamRegs<kMcg, kNarrow, 1, BT, XGlobal>::kStageBytes, red = 4u * kGroupRows * BT * 4u * 16u;
+    constexpr uint32_t stage = 4u * GemvStream<kMoeLdsRing, kMcg, kNarrow, 1, BT, XGlobal>::kStageBytes, red = 4u * kGroupRows * BT * 4u * 16u;
     return stage > red ? stage : red;
 }
 
@@ -395,7 +397,7 @@ constexpr uint32_t group_lds_bytes() {
 template <int CB, int WIDE, int BT, int NPROJ>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ? 2 : (gemv_step_rows<CB>() == 2 ? 3 : 4)))) moe_gemv_grouped(const MoeLaunch a) {
     __shared__ __attribute__((aligned(16))) unsigned char smem[group_lds_bytes<BT>()];
-    typedef GemvStreamRegs<CB, WIDE, 1, BT, XGlobal> StreamG;
+    typedef GemvStream<kMoeLdsRing, CB, WIDE, 1, BT, XGlobal> StreamG;
     constexpr uint32_t kStage = StreamG::kStageBytes;
     const uint32_t g = blockIdx.y / NPROJ, proj = blockIdx.y % NPROJ, blk = blockIdx.x, ksl = blockIdx.z;
     if (g >= a.groups[0]) return;  // uniform over the workgroup
