@@ -52,8 +52,11 @@ READ_PEAK_GBPS = None  # measured at start-up (measured_hbm_read)
 # WRITE_SIZE counters scaled by a 256 MiB copy (profiles/dense_gemv_in4096_out12288_k4_rows1.txt): keyed by the sources
 # of the kernel the figure was measured on (`kernel_sources_key`), then by (in, out, n, rows). A kernel whose sources
 # have changed since reports null until it is measured again.
-MEASURED_TRAFFIC = {}
-GEMV_SOURCES = ("t3_dense.hip", "t3_gemv_core.hpp", "t3_decode.hpp", "t3_stages.hpp", "t3_common.hpp")
+MEASURED_TRAFFIC = {
+    # one launch: FETCH_SIZE 12646.11 x 1.99968 = 25288.2 KiB read + WRITE_SIZE 435.0 KiB = 1.047 x the code bytes
+    "268b24a0f6e0cb69": {(4096, 12288, 64, 1): 26340521},
+}
+GEMV_SOURCES = ("t3_dense.hip", "t3_gemv_core.hpp", "t3_lds_loads.hpp", "t3_decode.hpp", "t3_stages.hpp", "t3_common.hpp")
 
 
 def kernel_sources_key() -> str:
