@@ -103,7 +103,7 @@ def test_fused_launches_equal_the_chain_bytes(oracle, t3, in_f, out_f, n, codebo
     x_dev, _ = make_x(case.rng, 32, in_f, dtype)
     eight = n <= 64 and (out_f // 128) * t3.linear_plan(x_dev[:1], case.d_trellis, case.dec)["k_slices"] > 128
     assert t3.linear_plan(x_dev[:1], case.d_trellis, case.dec)["tiles_a_load"] == (8 if eight else 4)
-    for rows in (1, 2, 4, 5, 16, 17, 32):
+    for rows in (1, 2, 3, 4, 5, 16, 17, 32):
         chain = t3.linear_chain(x_dev[:rows], case.d_trellis, case.d_suh, case.d_svh, case.dec)
         for _ in range(2):
             fused = t3.linear(x_dev[:rows], case.d_trellis, case.d_suh, case.d_svh, case.dec)

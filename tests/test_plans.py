@@ -69,8 +69,8 @@ def test_the_k_split_never_depends_on_the_rows(lib):
 
 
 def test_dense_path_by_rows(lib):
-    paths = {rows: linear_plan(lib, rows, 4096, 12288, 64).path for rows in (1, 2, 3, 4, 32, 33, 511)}
-    assert paths == {1: 0, 2: 0, 3: 0, 4: 2, 32: 2, 33: 3, 511: 3}
+    paths = {rows: linear_plan(lib, rows, 4096, 12288, 64).path for rows in (1, 2, 3, 4, 5, 32, 33, 511)}
+    assert paths == {1: 0, 2: 0, 3: 0, 4: 0, 5: 2, 32: 2, 33: 3, 511: 3}
     assert linear_plan(lib, 2, 4096, 12288, 80).path == 0          # above four bits a weight: up to two rows
     assert linear_plan(lib, 3, 4096, 12288, 80).path == 2
     assert linear_plan(lib, 1, 4096, 151936, 96).path == 1         # 64 tiles a wave: prepare launch + arriving GEMV

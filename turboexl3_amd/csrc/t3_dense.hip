@@ -15,7 +15,7 @@
 //   chain   three launches: dense_prep, dense_gemv<kChain>, dense_finish;
 //   arrive  two launches: dense_prep, dense_gemv<kArrive>: the workgroup that completes a 128-column block's planes
 //           (an integer arrival counter over device-coherent stores, nothing spins) runs the block's finish;
-//   one     one launch, the fewest rows (the kernel serves up to 4, the host sends up to 3): dense_gemv<kOne> prepares
+//   one     one launch, the fewest rows (up to 4 at eight tiles a step, up to 2 at four): dense_gemv<kOne> prepares
 //           its own K part in LDS, then as arrive.
 // The role of each launch follows the reference's HIP plan (src/hip/plan.zig:161-204); the launch shapes, the lane
 // plan and the use of MFMA are this library's own.

@@ -222,18 +222,25 @@ int32_t run_chain(const DenseCall& call, hipStream_t s, uint32_t stages) {
     return T3_OK;
 }
 
-// The served form (src/core/dense.zig:1229-1242 takes DEC-ONE at its fewest rows the same way). Up to three rows where a
+// The served form (src/core/dense.zig:1229-1242 takes DEC-ONE at its fewest rows the same way). Up to four rows where a
 // wave takes eight tiles a step (up to four bits a weight), up to two otherwise: one launch where a wave's K part is whole
 // 128-blocks and small enough to prepare in LDS, else the prepare launch and the arriving GEMV. More rows: the chain.
-// Measured at 4096 x 12288 (us a call, one launch against the chain): K4 14.4 / 13.9 / 14.4 / 15.2 against 15.8 / 15.0 /
-// 15.1 / 15.2 at 1 / 2 / 3 / 4 rows, K5 14.8 / 15.7 / 16.7 / 17.7 against 16.7 / 16.7 / 16.9 / 16.8: every workgroup
-// prepares every row of its K part (all rows' loads in flight together, then a butterfly a row) and the last arriver
-// finishes a row a wave, which the chain's two small launches do once; with 16 and 32 rows the planes' coherent traffic
-// costs the arriving form more than the finish launch it saves. The forms give the same bytes.
+// Measured at 4096 x 12288 with the f16-weight codebook forms (us a call, one launch against the chain, four rows):
+// K3 15.9-16.4 against 17.1, K4 16.4-16.5 against 17.0-17.2, K5 (four tiles a step) 17.9-18.1 against 17.6-17.7: every
+// workgroup prepares every row of its K part (all rows' loads in flight together, then a butterfly a row) and the last
+// arriver finishes a row a wave, which the chain's two small launches do once; with 16 and 32 rows the planes' coherent
+// traffic costs the arriving form more than the finish launch it saves. The forms give the same bytes.
+// (T3_ONE_ROWS_BT8, T3_ONE_ROWS_BT4: build-time overrides of the two bounds, for measuring.)
+#ifndef T3_ONE_ROWS_BT8
+#define T3_ONE_ROWS_BT8 4u
+#endif
+#ifndef T3_ONE_ROWS_BT4
+#define T3_ONE_ROWS_BT4 2u
+#endif
 int dense_path(const DenseLaunch& l) {
     if (l.rows > gemv_rows_max()) return takes_w_hat(l) ? T3_DENSE_W_HAT_GEMM : T3_DENSE_TRELLIS_GEMM;
     const uint32_t per = (l.in / 16u) / (4u * l.ks);
-    if (!config().dec_one || l.rows > (l.bt == 8u ? 3u : 2u)) return T3_DENSE_CHAIN;
+    if (!config().dec_one || l.rows > (l.bt == 8u ? T3_ONE_ROWS_BT8 : T3_ONE_ROWS_BT4)) return T3_DENSE_CHAIN;
     return per % 8u == 0u && per <= 16u ? T3_DENSE_ONE_LAUNCH : T3_DENSE_ARRIVE;
 }
 
