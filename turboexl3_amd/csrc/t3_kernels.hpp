@@ -118,6 +118,9 @@ struct MoeLaunch {
 // Rows up to which the two-launch form runs the mid stage inside the down launch (every down wave for its own
 // 128-block) and shapes both launches for few, long waves (t3_moe.hip)
 constexpr uint32_t kMoeFewRows = 4;
+// floats from one row-slot's block sums to the next in the down launch's own copies of them: whole 128-byte lines, so
+// that the device-coherent stores of different slots never meet in a cache line
+__host__ __device__ inline uint32_t hs_copy_stride(uint32_t inter) { return (inter / 128u + 31u) & ~31u; }
 enum MoeForm : int { kMoeFiveLaunches = 0, kMoeFourLaunches = 1, kMoeTwoLaunches = 2, kMoeGrouped = 3 };
 hipError_t launch_moe_decode(const MoeLaunch& a, int form, hipStream_t s);
 // a row's top-k experts by logit (ties to the lowest id) and their renormalised softmax weights in the logits' dtype

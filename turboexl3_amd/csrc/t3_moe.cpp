@@ -156,7 +156,9 @@ void carve_moe(MoeCall* call, void* workspace) {
     l.hd = c.take<uint32_t>(rkt * l.inter * 4u);
     l.sg = c.take<float>(rkt * (l.hidden / 128u) * 4u);
     l.su = c.take<float>(rkt * (l.hidden / 128u) * 4u);
-    l.hs = c.take<float>(rkt * (l.inter / 128u) * 4u);
+    // up to kMoeFewRows rows the down launch makes the sums itself: a copy a 128-column block of its output
+    l.hs = c.take<float>(l.rows <= kMoeFewRows ? (l.hidden / 128u) * rkt * hs_copy_stride(l.inter) * 4u
+                                               : rkt * (l.inter / 128u) * 4u);
     l.zg = c.take<float>(static_cast<size_t>(l.ks_gu) * rkt * l.inter * 4u);
     l.zu = c.take<float>(static_cast<size_t>(l.ks_gu) * rkt * l.inter * 4u);
     l.zd = c.take<float>(static_cast<size_t>(l.ks_dn) * rkt * l.hidden * 4u);

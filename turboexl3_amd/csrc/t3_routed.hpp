@@ -108,14 +108,23 @@ __device__ __forceinline__ void ordered_sums(const float* const (&p)[N], size_t 
 }
 
 // 0 + p[0] + p[1] + ... in that order, the values fetched by one load across the wave's lanes (up to 64 of them)
+// In two steps, so that a caller can send the load out beside its other loads and add up once they are all back:
+// lane_sum_fetch is the load (a lane's own value), lane_sum_fold the additions.
 template <bool COH>
-__device__ __forceinline__ float lane_ordered_sum(const float* p, uint32_t count, uint32_t lane) {
+__device__ __forceinline__ float lane_sum_fetch(const float* p, uint32_t count, uint32_t lane) {
+    return lane < count ? (COH ? load_coherent(p + lane) : p[lane]) : 0.0f;
+}
+template <bool COH>
+__device__ __forceinline__ float lane_sum_fold(float mine, const float* p, uint32_t count) {
     if (count > 64u) return ordered_sum<COH>(p, 1u, count, false);
-    const float mine = lane < count ? (COH ? load_coherent(p + lane) : p[lane]) : 0.0f;
     float acc = 0.0f;
     for (uint32_t q = 0; q < count; ++q)
         acc += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), static_cast<int>(q)));
     return acc;
+}
+template <bool COH>
+__device__ __forceinline__ float lane_ordered_sum(const float* p, uint32_t count, uint32_t lane) {
+    return lane_sum_fold<COH>(lane_sum_fetch<COH>(p, count, lane), p, count);
 }
 
 template <bool COH>
@@ -184,11 +193,15 @@ __device__ __forceinline__ void routed_mid_values(const MoeLaunch& a, const Slot
     }
     const float* const planes[4] = {a.zg + at + lane, a.zg + at + lane + 64u, a.zu + at + lane, a.zu + at + lane + 64u};
     float sums[4];
+    const float* sgp = a.sg + static_cast<size_t>(q) * nb;
+    const float* sup = a.su + static_cast<size_t>(q) * nb;
+    const float mg = a.defer ? lane_sum_fetch<COH>(sgp, nb, lane) : 0.0f;  // out with the planes' loads
+    const float mu = a.defer ? lane_sum_fetch<COH>(sup, nb, lane) : 0.0f;
     ordered_sums<COH, 4>(planes, plane, ks, sums);
     float g[2] = {sums[0], sums[1]}, u[2] = {sums[2], sums[3]};
     if (a.defer) {
-        const float xg = lane_ordered_sum<COH>(a.sg + static_cast<size_t>(q) * nb, nb, lane);
-        const float xu = lane_ordered_sum<COH>(a.su + static_cast<size_t>(q) * nb, nb, lane);
+        const float xg = lane_sum_fold<COH>(mg, sgp, nb);
+        const float xu = lane_sum_fold<COH>(mu, sup, nb);
 #pragma unroll
         for (uint32_t j = 0; j < 2u; ++j) {
             g[j] = __builtin_fmaf(g[j], mul1_a(), mul1_b() * xg);
@@ -279,10 +292,19 @@ __device__ __forceinline__ void routed_down_finish_many(const MoeLaunch& a, cons
             planes[2 * r + j] = a.zd + static_cast<size_t>(q[r]) * a.hidden + b * 128u + lane + 64u * j;
         }
     }
+    // the block sums' loads go out with the planes' (HS_COH: the sums were made inside this launch, a copy a 128-column
+    // block of the output)
+    const float* hs[R];
+    float mine[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        hs[r] = a.hs + (HS_COH ? (static_cast<size_t>(b) * rkt + q[r]) * hs_copy_stride(a.inter) : static_cast<size_t>(q[r]) * nbi);
+        mine[r] = a.defer ? lane_sum_fetch<HS_COH>(hs[r], nbi, lane) : 0.0f;
+    }
     ordered_sums<COH, 2 * R>(planes, plane, ks, sums);
     if (a.defer)
 #pragma unroll
-        for (int r = 0; r < R; ++r) xsum[r] = lane_ordered_sum<HS_COH>(a.hs + static_cast<size_t>(q[r]) * nbi, nbi, lane);
+        for (int r = 0; r < R; ++r) xsum[r] = lane_sum_fold<HS_COH>(mine[r], hs[r], nbi);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         if (!s[r].live) continue;  // uniform over the wave
