@@ -83,6 +83,8 @@ struct MoeLaunch {
     float* sg = nullptr;         // f32 [RKT][hidden / 128]
     float* su = nullptr;
     float* hs = nullptr;         // f32 [RKT][inter / 128]
+    float* xt = nullptr;         // above the decode rows, the deferred map: f32 [3][positions], a position's totals of
+                                 // sg, su and hs for the GEMMs' ends
     float* zg = nullptr;         // f32 [ks_gu][RKT][inter]
     float* zu = nullptr;
     float* zd = nullptr;         // f32 [ks_dn][RKT][hidden]

@@ -182,6 +182,7 @@ void carve_moe_prefill(MoeCall* call, void* workspace) {
     l.sg = c.take<float>(p * (l.hidden / 128u) * 4u);
     l.su = c.take<float>(p * (l.hidden / 128u) * 4u);
     l.hs = c.take<float>(p * (l.inter / 128u) * 4u);
+    l.xt = c.take<float>(p * 3u * 4u);
     l.zg = c.take<float>(p * l.inter * 4u);
     l.zu = c.take<float>(p * l.inter * 4u);
     l.zd = c.take<float>(p * l.hidden * 4u);

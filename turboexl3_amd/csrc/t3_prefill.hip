@@ -38,7 +38,9 @@ struct PfGemm {
     uint32_t kparts;  // K parts (grid z): part k multiplies its share of the tile rows into plane k of z
     uint32_t plane;   // elements between z's planes
     uint32_t zhalf;   // z holds f16 [positions][out] (the sums rounded at the launch's end) instead of f32: one K part, and
-                      // a finish that starts by rounding them (no deferred map, not GLM's profile)
+                      // a finish that starts by rounding them (not GLM's profile)
+    const float* xtot[2];  // zhalf under MUL1's deferred map: a position's total of its input's block sums (pf_rowsums);
+                           // the launch's end applies the map before it rounds. Null: no map.
 };
 
 // Grid (8 * ceil(nblk / spread) * ceil(max_items / (8 / spread)), projections, kparts), 256 threads. Consecutive
@@ -221,9 +223,16 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(LBMAX 
             const size_t at = static_cast<size_t>(first + row) * a.out + col0 * 16u + 4u * (lane >> 4);
             if (a.zhalf) {  // uniform
                 uint16_t* zh = reinterpret_cast<uint16_t*>(z);
+                // the deferred map as the stages apply it to an f32 plane: fma(sum, A, B * total), then the rounding
+                const float* xt = a.xtot[proj];
+                const float bx = xt ? mul1_b() * xt[first + row] : 0.0f;
 #pragma unroll
                 for (uint32_t t = 0; t < kPfTiles; ++t) {
-                    const float4v v = acc[mb][t];
+                    float4v v = acc[mb][t];
+                    if (xt) {
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) v[c] = __builtin_fmaf(v[c], mul1_a(), bx);
+                    }
                     uint2v h;
                     h[0] = static_cast<uint32_t>(half_bits(v[0])) | (static_cast<uint32_t>(half_bits(v[1])) << 16);
                     h[1] = static_cast<uint32_t>(half_bits(v[2])) | (static_cast<uint32_t>(half_bits(v[3])) << 16);
@@ -415,13 +424,13 @@ __global__ void __launch_bounds__(256) pf_mid(const MoeLaunch a) {
     const size_t eo = static_cast<size_t>(s.e) * a.inter, qo = static_cast<size_t>(pos) * a.inter;
     const Row16 g16 = row16(lane);
     float gt[8], up[8], svg[8], svu[8], sdn[8];
-    const bool zhalf = PROF == 0 && !a.defer;
+    const bool zhalf = PROF == 0;  // the GEMM applied the deferred map, if any, before it rounded
     load8_plane(a.zg, qo + i, zhalf, gt);
     load8_plane(a.zu, qo + i, zhalf, up);
     load8_half(bank.gate_svh, eo + i, svg);
     load8_half(bank.up_svh, eo + i, svu);
     load8_half(bank.down_suh, eo + i, sdn);
-    if (a.defer) {
+    if (a.defer && !zhalf) {
         const float xg = wave_ordered_sum(a.sg + static_cast<size_t>(pos) * nbh, nbh, lane);
         const float xu = wave_ordered_sum(a.su + static_cast<size_t>(pos) * nbh, nbh, lane);
 #pragma unroll
@@ -474,9 +483,22 @@ __global__ void __launch_bounds__(256) pf_slots(const MoeLaunch a) {
     if (live) store8_act<kF32>(a.y, static_cast<size_t>(rk) * a.hidden + i, v);
 }
 
+// A position's total of its input's block sums, 0 + s[0] + s[1] + ... (wave_ordered_sum's order): what MUL1's deferred map
+// multiplies by B. Made once a position here so that the GEMM's end can apply the map to its sums and round them (f16
+// planes: the stages after it read half the bytes). A thread a position; up to two arrays a launch.
+__global__ void __launch_bounds__(256) pf_rowsums(const float* s0, const float* s1, float* t0, float* t1, uint32_t nb,
+                                                  uint32_t positions) {
+    const uint32_t pos = blockIdx.x * 256u + threadIdx.x;
+    if (pos >= positions) return;
+    const float* s = blockIdx.y ? s1 : s0;
+    float acc = 0.0f;
+    for (uint32_t b = 0; b < nb; ++b) acc += s[static_cast<size_t>(pos) * nb + b];
+    (blockIdx.y ? t1 : t0)[pos] = acc;
+}
+
 // every slot's down finish, then the score-weighted sum in slot order (routed_combine_block's statements)
 __global__ void __launch_bounds__(256) pf_combine(const MoeLaunch a) {
-    const uint32_t nb = a.hidden / 128u, nbi = a.inter / 128u, groups = (nb + kPfUnit - 1u) / kPfUnit;
+    const uint32_t nb = a.hidden / 128u, groups = (nb + kPfUnit - 1u) / kPfUnit;
     const uint32_t u0 = wave_unit(), row = u0 / groups, lane = threadIdx.x & 63u, q = lane & 15u;
     if (row >= a.rows) return;
     const uint32_t b1 = (u0 % groups) * kPfUnit + (lane >> 4);
@@ -494,13 +516,9 @@ __global__ void __launch_bounds__(256) pf_combine(const MoeLaunch a) {
         const uint32_t pos = a.inv[rk];
         const RoutedBank& bank = s.shared ? a.shared : a.bank;
         float v[8], sv[8];
-        load8_plane(a.zd, static_cast<size_t>(pos) * a.hidden + i, !a.defer, v);
+        // f16: the down GEMM applied the deferred map, if any, before it rounded
+        load8_plane(a.zd, static_cast<size_t>(pos) * a.hidden + i, true, v);
         load8_half(bank.down_svh, static_cast<size_t>(s.e) * a.hidden + i, sv);
-        if (a.defer) {
-            const float xsum = wave_ordered_sum(a.hs + static_cast<size_t>(pos) * nbi, nbi, lane);
-#pragma unroll
-            for (uint32_t r = 0; r < 8u; ++r) v[r] = __builtin_fmaf(v[r], mul1_a(), mul1_b() * xsum);
-        }
         const float w = s.shared ? 1.0f : score_of(a, row, k);
         finish_row16(v, sv, g16);
 #pragma unroll
@@ -680,9 +698,18 @@ hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s) {
     g.wbits = a.wbits;
     g.positions = p;
     g.experts = a.bank.experts;
-    g.zhalf = !a.defer && !a.glm;
-    if (a.stages & 4u)
+    g.zhalf = !a.glm;
+    const bool map = a.defer && !a.glm;  // the GEMMs' ends apply the deferred map (GLM's profile keeps f32 planes)
+    g.xtot[0] = map ? a.xt : nullptr;
+    g.xtot[1] = map ? a.xt + p : nullptr;
+    if (a.stages & 4u) {
+        if (map) {
+            hipLaunchKernelGGL(pf_rowsums, dim3((p + 255u) / 256u, 2u), dim3(256), 0, s, a.sg, a.su, a.xt, a.xt + p,
+                               a.hidden / 128u, p);
+            if ((e = hipGetLastError()) != hipSuccess) return e;
+        }
         if ((e = launch_gemm(g, a.codebook, a.max_items, 2u, a.item_rows, s)) != hipSuccess) return e;
+    }
 
     if (a.stages & 8u) {
         if (a.glm) hipLaunchKernelGGL(pf_mid<1>, unit_grid(p, a.inter), dim3(256), 0, s, a);
@@ -700,8 +727,16 @@ hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s) {
     g.in = a.inter;
     g.out = a.hidden;
     g.n = a.n_dn;
-    if (a.stages & 16u)
+    g.xtot[0] = map ? a.xt + 2u * static_cast<size_t>(p) : nullptr;
+    g.xtot[1] = nullptr;
+    if (a.stages & 16u) {
+        if (map) {
+            hipLaunchKernelGGL(pf_rowsums, dim3((p + 255u) / 256u, 1u), dim3(256), 0, s, a.hs, a.hs, a.xt + 2u * static_cast<size_t>(p),
+                               a.xt + 2u * static_cast<size_t>(p), a.inter / 128u, p);
+            if ((e = hipGetLastError()) != hipSuccess) return e;
+        }
         if ((e = launch_gemm(g, a.codebook, a.max_items, 1u, a.item_rows, s)) != hipSuccess) return e;
+    }
 
     if (!(a.stages & 32u)) return hipSuccess;
     if (a.glm) hipLaunchKernelGGL(pf_slots, unit_grid(p, a.hidden), dim3(256), 0, s, a);
