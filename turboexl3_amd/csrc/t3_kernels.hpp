@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cmath>
 #include <cstddef>
 #include <cstdint>
 
@@ -135,16 +136,27 @@ hipError_t launch_route_softmax_gate(const void* logits, int32_t* inds, void* sc
 
 // Rows a GEMM item of a routed call of `slots` row-slots over `experts` experts (the shared slots' among them). An item
 // pays its matrix's whole decode whatever its rows, so items are as tall as the experts' shares of the call: 32 rows
-// when the mean share is small, 64, then the 128-row shape once it passes 40 (most experts then stay one item). Between
-// the two, while the mean share plus three of its standard deviations (a routing's counts scatter like sqrt(mean))
-// stays within 96 rows, the route cuts items at 96 and the GEMM runs with accumulators for six row blocks instead of
-// eight: three waves a SIMD instead of two, and the rare expert past 96 rows becomes two items.
+// when the mean share is small, 64, then a shape of eight row blocks once it passes 40. That shape runs with
+// accumulators for all eight blocks (128-row items, two waves a SIMD) or for six (the route cuts items at 96 rows: three
+// waves a SIMD, an item's decode and MFMAs about an eighth faster; 512 experts of 2560 x 640, 160 rows an expert: the
+// call 2.11 -> 1.95 ms). The cut that costs fewer decodes wins: the items an expert becomes, 1 + P(rows > cut) +
+// P(rows > 2 cut) + ..., with an expert's rows scattering around the mean share like sqrt(mean) (a uniform routing's
+// counts), at 96 rows against 128, the 96-row count allowed the eighth its kernel is faster by. Mean 64: 96 (one item
+// either way); 100-150: 128 (most experts one item instead of two); 160: 96 (two either way); 200: 128.
 inline uint32_t moe_item_rows(size_t slots, size_t experts) {
+#ifdef T3_MOE_ITEM_ROWS  // a build-time override, for measuring one shape everywhere
+    return T3_MOE_ITEM_ROWS;
+#endif
     const size_t share = slots / experts;
     if (share <= 24u) return 32u;
     if (share <= 40u) return 64u;
-    const float mean = static_cast<float>(slots) / static_cast<float>(experts);
-    return mean + 3.0f * __builtin_sqrtf(mean) <= 96.0f ? 96u : 128u;
+    const float mean = static_cast<float>(slots) / static_cast<float>(experts), sd = std::sqrt(mean);
+    const auto items = [&](float cut) {
+        float n = 1.0f;
+        for (int j = 1; j <= 16; ++j) n += 0.5f * std::erfc((static_cast<float>(j) * cut - mean) / (sd * 1.41421356f));
+        return n;
+    };
+    return items(96.0f) <= 1.12f * items(128.0f) ? 96u : 128u;
 }
 
 // The same call above the decode rows: route, prepare, gate|up GEMM, mid, down GEMM, combine. xg, xu, hd hold plain f16
