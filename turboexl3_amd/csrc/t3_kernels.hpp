@@ -99,7 +99,8 @@ struct MoeLaunch {
     int clamp_at = 0;  // format.ClampAt: 0 gate_in (the gate clamped before its SiLU), 1 silu_out (the SiLU's output)
     // prefill only (the route's roles, src/hip/plan.zig:40-45): row-slots sorted by expert. order [P] position ->
     // row-slot, inv [P] row-slot -> position (~0: skipped), items [max_items] {expert, first position, rows, 0},
-    // counts [E + S + 4]: per-expert counts, then the item count and the placed total; cursor [E + S].
+    // counts [E + S + 4]: per-expert counts, then the item count and the placed total; cursor [E + S], a counter every
+    // 32 words (a cache line each).
     uint32_t* order = nullptr;
     uint32_t* inv = nullptr;
     uint32_t* items = nullptr;

@@ -194,7 +194,7 @@ void carve_moe_prefill(MoeCall* call, void* workspace) {
     l.items = c.take<uint32_t>(static_cast<size_t>(l.max_items) * 16u);
     call->counts_at = c.used;
     l.counts = c.take<uint32_t>((et + 4u) * 4u);
-    l.cursor = c.take<uint32_t>(et * 4u);
+    l.cursor = c.take<uint32_t>(et * 128u);  // a cache line a counter (t3_prefill.hip: kPfCounterStride)
     call->workspace = c.used;
 }
 
