@@ -417,13 +417,30 @@ __global__ void __launch_bounds__(256) pf_prep(const MoeLaunch a) {
 }
 
 // gate and up finishes, the (clamped) SwiGLU, the down's prepare (routed_mid_block's statements)
+// PROF 0: a wave's four blocks are four adjacent (position, block) pairs of all the call's, so that a width that is not
+// whole units (640 = five blocks: two units a position, the second a quarter full) wastes no lanes (8192 rows of 512
+// experts of 2560 x 640: 185 -> 125 us); a 16-lane group then has a position of its own. GLM's profile adds its block
+// sums up across the wave and keeps one position a wave.
 template <int PROF>
 __global__ void __launch_bounds__(256) pf_mid(const MoeLaunch a) {
     const uint32_t nb = a.inter / 128u, nbh = a.hidden / 128u, groups = (nb + kPfUnit - 1u) / kPfUnit;
-    const uint32_t u0 = wave_unit(), pos = u0 / groups, lane = threadIdx.x & 63u, q = lane & 15u;
-    if (pos >= a.counts[a.bank.experts + a.shared_slots + 1u]) return;
-    const uint32_t b1 = (u0 % groups) * kPfUnit + (lane >> 4);
-    const bool live = b1 < nb;
+    const uint32_t u0 = wave_unit(), lane = threadIdx.x & 63u, q = lane & 15u;
+    const uint32_t placed = a.counts[a.bank.experts + a.shared_slots + 1u];
+    uint32_t pos, b1;
+    bool live;
+    if constexpr (PROF == 0) {
+        const uint32_t total = placed * nb, f = u0 * kPfUnit + (lane >> 4);
+        if (u0 * kPfUnit >= total) return;  // uniform over the wave
+        live = f < total;
+        const uint32_t fc = live ? f : total - 1u;
+        pos = fc / nb;
+        b1 = fc - pos * nb;
+    } else {
+        pos = u0 / groups;
+        if (pos >= placed) return;
+        b1 = (u0 % groups) * kPfUnit + (lane >> 4);
+        live = b1 < nb;
+    }
     const uint32_t b = live ? b1 : nb - 1u, i = b * 128u + 8u * q;
     const SlotRef s = resolve_slot(a, a.order[pos]);
     const RoutedBank& bank = s.shared ? a.shared : a.bank;
@@ -719,7 +736,7 @@ hipError_t launch_moe_prefill(const MoeLaunch& a, hipStream_t s) {
 
     if (a.stages & 8u) {
         if (a.glm) hipLaunchKernelGGL(pf_mid<1>, unit_grid(p, a.inter), dim3(256), 0, s, a);
-        else hipLaunchKernelGGL(pf_mid<0>, unit_grid(p, a.inter), dim3(256), 0, s, a);
+        else hipLaunchKernelGGL(pf_mid<0>, dim3((p * (a.inter / 128u) + 4u * kPfUnit - 1u) / (4u * kPfUnit)), dim3(256), 0, s, a);
         if ((e = hipGetLastError()) != hipSuccess) return e;
     }
 
