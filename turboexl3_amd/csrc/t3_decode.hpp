@@ -28,6 +28,8 @@ enum Codebook : int {
     kMcg = 1,       // exact f16 weight, f16(lo + hi)
     kMul1Defer = 2, // h = 1024 + t as the weight; the affine map applied once an output (A acc + B sum x)
     kMcgPair = 3,   // the hashed pair (lo, hi) as two K slots: x lo + x hi, the weight never rounded to f16
+    kMcgTab = 4,    // kMcg's weights, some of a lane's looked up in an LDS table of all 65,536 (the measured two-pipe
+                    // form: t3_dense.hip, dense_gemv_tab)
 };
 
 constexpr uint32_t kMcgMult = 0xCBAC1FEDu;
@@ -68,7 +70,7 @@ __device__ __forceinline__ uint16_t decode_mul1(uint32_t cw) {
 }
 template <int CB>
 __device__ __forceinline__ uint16_t decode_exact(uint32_t cw) {
-    if constexpr (CB == kMcg || CB == kMcgPair) return decode_mcg(cw);
+    if constexpr (CB == kMcg || CB == kMcgPair || CB == kMcgTab) return decode_mcg(cw);
     else return decode_mul1(cw);
 }
 
@@ -108,6 +110,14 @@ __device__ __forceinline__ uint32_t weight_halves(uint32_t cw_lo, uint32_t cw_hi
     } else {
         return weight_half<CB>(cw_lo) | (weight_half<CB>(cw_hi) << 16);
     }
+}
+
+// The LDS table form: the f16 weight of every 16-bit codeword at byte 2 cw of the workgroup's dynamic LDS (the kernel
+// fills it and keeps no static LDS, so the table starts at LDS address 0). Two weights as one register's halves.
+extern __shared__ __attribute__((aligned(16))) unsigned char t3_table_lds[];
+__device__ __forceinline__ uint32_t table_halves(uint32_t cw_lo, uint32_t cw_hi) {
+    const uint16_t* tab = reinterpret_cast<const uint16_t*>(t3_table_lds);
+    return static_cast<uint32_t>(tab[cw_lo]) | (static_cast<uint32_t>(tab[cw_hi]) << 16);
 }
 
 // ---- the quad plan --------------------------------------------------------------------------------------------

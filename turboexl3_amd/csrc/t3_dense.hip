@@ -334,6 +334,103 @@ hipError_t launch_gemv_fuse(const DenseLaunch& d, int fuse, hipStream_t s) {
     return hipGetLastError();
 }
 
+// ---- the LDS-table decoder, measured (build with -DT3_GEMV_TABLE_FROM=<tile rows a wave> to route the chain's GEMV of a
+// matrix whose waves walk at least that many tile rows here; off in the served build) ---------------------------
+// One workgroup of twelve waves a compute unit holds the f16 weight of every 16-bit codeword in LDS (128 KB of the
+// 160) and runs three of dense_gemv's four-wave workgroups at a time beside it, persistently: virtual workgroup
+// (column block, K slice) v = (pass x grid + workgroup) x 3 + group. T3_GEMV_TABLE_PAIRS of a lane's four weight
+// registers a tile pair are looked up (two vector operations and a ds_read_u16 a weight), the others hashed (four
+// vector operations): the two pipes side by side. The K partition, the order of the waves' sums and so the planes' bytes
+// are dense_gemv's. Up to four rows, up to four bits a weight (a tile of whole 16-byte pieces within 128 bytes), MCG.
+#ifndef T3_GEMV_TABLE_FROM
+#define T3_GEMV_TABLE_FROM 0xFFFFFFFFu
+#endif
+constexpr uint32_t kTabTableBytes = 131072u, kTabWaves = 12u, kTabRows = 4u;
+
+template <int BT>
+__global__ void __launch_bounds__(768) dense_gemv_tab(const GemvArgs a, uint32_t nblk, uint32_t nvwg, uint32_t iters) {
+    typedef GemvStreamTab<BT, 2> Stream;
+    constexpr uint32_t kStage = Stream::kStageBytes;
+    static_assert(4u * kStage >= 4u * kTabRows * BT * 4u * 16u, "a group's sums fit its four stages");
+    unsigned char* stages = t3_table_lds + kTabTableBytes;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), g = wave >> 2, sg = wave & 3u;
+    const uint32_t lane = threadIdx.x & 63u, gtid = threadIdx.x & 255u;
+    uint32_t* tab32 = reinterpret_cast<uint32_t*>(t3_table_lds);
+    for (uint32_t i = threadIdx.x; i < 32768u; i += 768u)
+        tab32[i] = static_cast<uint32_t>(decode_mcg(2u * i)) | (static_cast<uint32_t>(decode_mcg(2u * i + 1u)) << 16);
+    __syncthreads();
+    const uint32_t out_tiles = a.out >> 4, nw = a.n >> 1, rows = a.rows, per = a.per;
+    const uint64_t wstride = static_cast<uint64_t>(out_tiles) * nw;
+    const uint32_t wstep = static_cast<uint32_t>(wstride) * 4u;
+    float4v* red = reinterpret_cast<float4v*>(stages + g * 4u * kStage);  // [wave][row][tile][lane / 16]
+    for (uint32_t it = 0; it < iters; ++it) {
+        const uint32_t v = (it * gridDim.x + blockIdx.x) * 3u + g;
+        const bool live = v < nvwg;  // uniform over the group's waves
+        const uint32_t vv = live ? v : 0u, ksl = vv / nblk, blk = vv - ksl * nblk;
+        float4v acc[1][BT];
+#pragma unroll
+        for (int t = 0; t < BT; ++t) acc[0][t] = float4v{0.f, 0.f, 0.f, 0.f};
+        if (live) {
+            const uint32_t tk0 = (ksl * 4u + sg) * per;
+            const uint32_t* wbase = a.w + static_cast<uint64_t>(blk) * BT * nw + tk0 * wstride;
+            const uint32_t xoff = x_frag_offset(lane, (lane & 15u) < rows, (lane & 15u) * 64u);
+            Stream stream(wbase, wstep, per, a.n, a.wbits,
+                          XGlobal{a.xq, static_cast<uint64_t>(rows) * (a.in / 32u) * 64u, (tk0 / 2u) * rows * 64u, rows * 64u},
+                          xoff, stages + wave * kStage, lane);
+            stream.issue();
+            stream.run(acc);
+        }
+        __syncthreads();  // every wave is done with its stage before the sums take the memory
+        if ((lane & 15u) < rows)
+#pragma unroll
+            for (int t = 0; t < BT; ++t)
+                red[((sg * kTabRows + (lane & 15u)) * BT + static_cast<uint32_t>(t)) * 4u + (lane >> 4)] = acc[0][t];
+        __syncthreads();
+        if (live && gtid < rows * BT * 4u) {
+            const uint32_t row = gtid / (BT * 4u), t = (gtid >> 2) % BT, q = gtid & 3u;
+            const uint32_t at = (row * BT + t) * 4u + q, wv = kTabRows * BT * 4u;
+            const float4v s = ((red[at] + red[wv + at]) + red[2u * wv + at]) + red[3u * wv + at];
+            *reinterpret_cast<float4v*>(a.z + (static_cast<size_t>(ksl) * rows + row) * a.out + (blk * BT + t) * 16u + 4u * q) = s;
+        }
+        __syncthreads();  // the sums are read before the next pass stages its first tile rows
+    }
+}
+
+inline bool gemv_table_serves(const DenseLaunch& d, int fuse) {
+    const uint32_t per = (d.in / 16u) / (4u * d.ks);
+    return fuse == kFuseChain && d.codebook == kMcg && per >= T3_GEMV_TABLE_FROM && d.rows <= kTabRows && d.n <= 64u &&
+           d.n % 8u == 0u && (d.out / 16u) % 4u == 0u;
+}
+
+hipError_t launch_gemv_tab(const DenseLaunch& d, hipStream_t s) {
+    constexpr int BT = 4;
+    GemvArgs a{};
+    a.w = d.trellis;
+    a.xq = d.xq;
+    a.z = d.z;
+    a.in = d.in;
+    a.out = d.out;
+    a.rows = d.rows;
+    a.n = d.n;
+    a.wbits = d.wbits;
+    a.per = (d.in / 16u) / (4u * d.ks);
+    a.ks = d.ks;
+    const uint32_t nblk = (d.out / 16u) / BT, nvwg = nblk * d.ks;
+    const uint32_t grid = (nvwg + 2u) / 3u < 256u ? (nvwg + 2u) / 3u : 256u;
+    const uint32_t iters = (nvwg + grid * 3u - 1u) / (grid * 3u);
+    const uint32_t dyn = kTabTableBytes + kTabWaves * GemvStreamTab<BT, 2>::kStageBytes;
+    static bool allowed = false;  // once a process: the launch may take more than 64 KB of dynamic LDS
+    if (!allowed) {
+        if (const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dense_gemv_tab<BT>),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(dyn));
+            e != hipSuccess)
+            return e;
+        allowed = true;
+    }
+    hipLaunchKernelGGL((dense_gemv_tab<BT>), dim3(grid), dim3(768), dyn, s, a, nblk, nvwg, iters);
+    return hipGetLastError();
+}
+
 template <int CB>
 hipError_t launch_gemv_cb(const DenseLaunch& d, int fuse, hipStream_t s) {
     const bool two = d.rows > 16u;
@@ -381,6 +478,7 @@ hipError_t launch_dense_prep(const DenseLaunch& d, hipStream_t s) {
 }
 
 hipError_t launch_dense_gemv(const DenseLaunch& d, int fuse, hipStream_t s) {
+    if (gemv_table_serves(d, fuse)) return launch_gemv_tab(d, s);
     switch (d.codebook) {
         case kMul1: return launch_gemv_cb<kMul1>(d, fuse, s);
         case kMcg: return launch_gemv_cb<kMcg>(d, fuse, s);

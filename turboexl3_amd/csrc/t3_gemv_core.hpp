@@ -58,7 +58,7 @@ constexpr uint32_t kNoBytes = 0x80000000u;  // a lane offset no buffer reaches: 
 // tile rows a step of codebook form CB
 template <int CB>
 constexpr int gemv_step_rows() {
-    return (CB == kMcg || CB == kMul1) ? 2 : 1;
+    return (CB == kMcg || CB == kMul1 || CB == kMcgTab) ? 2 : 1;
 }
 
 // Where a wave's prepared activations come from. A step's activations are 64 bytes a row either way: 16 inputs doubled
@@ -104,6 +104,10 @@ __device__ __forceinline__ uint32_t x_frag_offset(uint32_t lane, bool live, uint
 // run(): acc[r][t] += the 16 x 16 product of activation block r and tile t, summed over the wave's tile rows in order;
 // when it returns none of the wave's loads is in flight and the stage's memory is free.
 
+#ifndef T3_GEMV_TABLE_PAIRS
+#define T3_GEMV_TABLE_PAIRS 2
+#endif
+
 // What both forms share: a step's words out of its LDS slots, and its decode into the matrix core.
 template <int CB, int WIDE, int RB, int BT>
 struct GemvStep {
@@ -142,10 +146,19 @@ struct GemvStep {
                 uint32_t c0[4], c1[4];
                 quad_codewords<WIDE>(wd[0][t], plan, wbits, c0);
                 quad_codewords<WIDE>(wd[1][t], plan, wbits, c1);
-                a[0] = weight_halves<CB>(c0[0], c0[1]);
-                a[1] = weight_halves<CB>(c0[2], c0[3]);
-                a[2] = weight_halves<CB>(c1[0], c1[1]);
-                a[3] = weight_halves<CB>(c1[2], c1[3]);
+                if constexpr (CB == kMcgTab) {
+                    // T3_GEMV_TABLE_PAIRS of a lane's four registers a tile pair come out of the LDS table, the others
+                    // out of the ALU hash: both pipes at work
+                    a[0] = T3_GEMV_TABLE_PAIRS >= 1 ? table_halves(c0[0], c0[1]) : weight_halves<kMcg>(c0[0], c0[1]);
+                    a[1] = T3_GEMV_TABLE_PAIRS >= 3 ? table_halves(c0[2], c0[3]) : weight_halves<kMcg>(c0[2], c0[3]);
+                    a[2] = T3_GEMV_TABLE_PAIRS >= 2 ? table_halves(c1[0], c1[1]) : weight_halves<kMcg>(c1[0], c1[1]);
+                    a[3] = T3_GEMV_TABLE_PAIRS >= 4 ? table_halves(c1[2], c1[3]) : weight_halves<kMcg>(c1[2], c1[3]);
+                } else {
+                    a[0] = weight_halves<CB>(c0[0], c0[1]);
+                    a[1] = weight_halves<CB>(c0[2], c0[3]);
+                    a[2] = weight_halves<CB>(c1[0], c1[1]);
+                    a[3] = weight_halves<CB>(c1[2], c1[3]);
+                }
             }
 #pragma unroll
             for (int r = 0; r < RB; ++r)
@@ -475,6 +488,83 @@ struct GemvStreamLds {
 };
 
 // LDS: the direct-to-LDS ring; else the register ring
+// The stream of the measured LDS-table form (t3_dense.hip, dense_gemv_tab): GemvStreamRegs' register ring at two tile
+// rows a step, cut down to what fits beside a 128 KB table: the narrow reader, tiles of whole 16-byte pieces and at most
+// 128 bytes (up to four bits a weight), packed in the stage (R x BT x 128 bytes a wave), ST steps in flight.
+template <int BT, int ST>
+struct GemvStreamTab {
+    static constexpr int R = 2;
+    static constexpr uint32_t kRowBytes = static_cast<uint32_t>(BT) * 128u;
+    static constexpr uint32_t kStageBytes = static_cast<uint32_t>(R) * kRowBytes;
+    const uint32_t* wbase;
+    uint32_t wstep, steps, n, wbits, lane;
+    XGlobal xs;
+    uint32_t xoff;
+    unsigned char* stage;
+    uint32_t span_bytes, voff;
+    uint4v ring[ST][R];
+    uint4v xr[ST][1];
+
+    __device__ __forceinline__ GemvStreamTab(const uint32_t* wbase_, uint32_t wstep_, uint32_t per_, uint32_t n_,
+                                             uint32_t wbits_, const XGlobal& xs_, uint32_t xoff_, unsigned char* stage_,
+                                             uint32_t lane_)
+        : wbase(wbase_), wstep(wstep_), steps(per_ / 2u), n(n_), wbits(wbits_), lane(lane_), xs(xs_), xoff(xoff_),
+          stage(stage_) {
+        const uint32_t chunk_bytes = static_cast<uint32_t>(BT) * 2u * n;
+        span_bytes = (per_ - 1u) * wstep + chunk_bytes;
+        voff = lane * 16u < chunk_bytes ? lane * 16u : kNoBytes;
+    }
+    __device__ __forceinline__ void load_step(uint32_t step, uint4v (&dst)[R]) const {
+        const __amdgpu_buffer_rsrc_t res = make_rsrc(wbase, step < steps ? span_bytes : 0u);
+#pragma unroll
+        for (int j = 0; j < R; ++j) dst[j] = buf_load_u128(res, voff, (step * R + static_cast<uint32_t>(j)) * wstep);
+    }
+    __device__ __forceinline__ void load_x(uint32_t step, uint4v (&dst)[1]) const {
+        const __amdgpu_buffer_rsrc_t res = make_rsrc(xs.base, step < steps ? xs.bytes : 0u);
+        dst[0] = buf_load_u128(res, xoff, xs.first + step * xs.step);
+    }
+    __device__ __forceinline__ void issue() {
+#pragma unroll
+        for (int s = 0; s < ST; ++s) {
+            load_step(static_cast<uint32_t>(s), ring[s]);
+            load_x(static_cast<uint32_t>(s), xr[s]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    __device__ __forceinline__ void run(float4v (&acc)[1][BT]) {
+        const uint32_t tile_bytes = 2u * n;
+        const QuadPlan<kNarrow> plan = quad_plan<kNarrow>(n, lane);
+        const bool writer = lane * 16u < static_cast<uint32_t>(BT) * tile_bytes;
+        auto stage_step = [&](const uint4v (&v)[R]) {
+            if (writer) {
+#pragma unroll
+                for (int j = 0; j < R; ++j)
+                    *reinterpret_cast<uint4v*>(stage + static_cast<uint32_t>(j) * kRowBytes + lane * 16u) = v[j];
+            }
+        };
+        GemvStep<kMcgTab, kNarrow, 1, BT> words;
+        stage_step(ring[0]);
+        load_step(static_cast<uint32_t>(ST), ring[0]);
+        uint32_t i = 0;
+        do {
+#pragma unroll
+            for (int s = 0; s < ST; ++s) {
+                const uint32_t step = i + static_cast<uint32_t>(s);
+                const int sn = (s + 1) % ST;
+                __builtin_amdgcn_sched_barrier(0);
+                words.fetch(stage, kRowBytes, tile_bytes, plan);
+                stage_step(ring[sn]);
+                load_step(step + 1u + ST, ring[sn]);
+                __builtin_amdgcn_sched_barrier(0);
+                words.consume(plan, wbits, xr[s], acc);
+                __builtin_amdgcn_sched_barrier(0);
+                load_x(step + ST, xr[s]);
+            }
+            i += ST;
+        } while (i < steps);
+    }
+};
+
 template <bool LDS, int CB, int WIDE, int RB, int BT, typename XSrc>
 using GemvStream = std::conditional_t<LDS, GemvStreamLds<CB, WIDE, RB, BT, XSrc>, GemvStreamRegs<CB, WIDE, RB, BT, XSrc>>;
 
