@@ -68,6 +68,9 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
     typedef GemvStream<kMoeLdsRing, CB, WIDE, 1, BT, XGlobal> StreamG;
     constexpr uint32_t kStage = StreamG::kStageBytes;
     constexpr int R = gemv_step_rows<CB>();   // tile rows a step
+    // the codebook form says whether MUL1's map is deferred (a.defer repeats it): the other forms' kernels carry none of
+    // the map's loads, sums and stores
+    constexpr int kDefer = CB == kMul1Defer ? 1 : 0;
     float4v(*red)[BT * 4] = reinterpret_cast<float4v(*)[BT * 4]>(smem);  // the one live row: four lanes a tile a wave
     const uint32_t rk = yidx / NPROJ, proj = yidx % NPROJ;
     const uint32_t sg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
@@ -117,7 +120,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
             stream.issue();
             uint32_t hh[2];
             float sum;
-            routed_mid_values<false, false, PROF>(a, s, rk, tk0 >> 3, lane, hh, sum);
+            routed_mid_values<false, false, PROF, kDefer>(a, s, rk, tk0 >> 3, lane, hh, sum);
             // element i = 64 j + lane of the block belongs to step i / (16 R) of the wave's walk
 #pragma unroll
             for (uint32_t j = 0; j < 2u; ++j) {
@@ -130,7 +133,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
             // shared by every column workgroup of the slot takes hundreds of device-coherent stores to the same few
             // cache lines, which serialise: 512 experts of 2560 x 640 at one token, the deferred map, this launch
             // 30.5 us at K3 and 49.6 at K5 against 16.9 and 19.6 for the codebook without the map.)
-            if (a.defer && lane == 0u && blk % (8u / BT) == 0u)
+            if (kDefer && lane == 0u && blk % (8u / BT) == 0u)
                 store_coherent(a.hs + (static_cast<size_t>(blk / (8u / BT)) * rkt + rk) * hs_copy_stride(a.inter) + (tk0 >> 3), sum);
             for (uint32_t i = lane; i < kXldsRows * 16u; i += 64u)
                 *reinterpret_cast<uint32_t*>(xst + steps * (kXldsRows * 64u) + i * 4u) = 0u;
@@ -155,7 +158,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
                 }
                 // every column workgroup of the slot stores the same sum: a handful of plain stores, read by the
                 // next launch
-                if (a.defer && lane == 0u) {
+                if (kDefer && lane == 0u) {
                     float* at = (proj ? a.su : a.sg) + static_cast<size_t>(rk) * (a.hidden / 128u) + (tk0 >> 3) + b;
                     if constexpr (ARRIVE) store_coherent(at, sum);
                     else *at = sum;
@@ -216,7 +219,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
         if (threadIdx.x == 0u)  // zero again for the next call
             __hip_atomic_store(a.arrive + counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if constexpr (NPROJ == 2) {
-            if (sg == 0u) routed_mid_block<false, true, PROF>(a, s, rk, b128, lane);
+            if (sg == 0u) routed_mid_block<false, true, PROF, kDefer>(a, s, rk, b128, lane);
         } else if constexpr (PROF == 1) {
             // GLM's profile ends with each live slot's own finished output, f32 [row-slot][hidden]: four slots a wave,
             // every load of the four in flight together, nothing to add up
@@ -234,7 +237,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
                     sk[r].e = info & 0x7FFFFFFFu;
                     qk[r] = s.row * kt + (k < kt ? k : 0u);
                 }
-                routed_down_finish_many<true, XLDS, 4, 1>(a, sk, qk, b128, lane, v, ks);
+                routed_down_finish_many<true, XLDS, 4, 1, kDefer>(a, sk, qk, b128, lane, v, ks);
 #pragma unroll
                 for (uint32_t r = 0; r < 4u; ++r)
                     if (sk[r].live) {
@@ -262,7 +265,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
                     sk[r].e = info & 0x7FFFFFFFu;
                     qk[r] = s.row * kt + (k < kt ? k : 0u);
                 }
-                routed_down_finish_many<true, XLDS, 4, 0>(a, sk, qk, b128, lane, v, ks);
+                routed_down_finish_many<true, XLDS, 4, 0, kDefer>(a, sk, qk, b128, lane, v, ks);
 #pragma unroll
                 for (uint32_t r = 0; r < 4u; ++r)
                     if (sk[r].live) {

@@ -107,6 +107,14 @@ __device__ __forceinline__ void ordered_sums(const float* const (&p)[N], size_t 
     }
 }
 
+// Whether the launch's codebook form defers MUL1's map: known when the kernel is compiled (DEFER 0 or 1: the GEMV
+// kernels, whose codebook form is a template argument, carry no code of the other case) or read from the launch (-1).
+template <int DEFER>
+__device__ __forceinline__ bool defers(const MoeLaunch& a) {
+    if constexpr (DEFER < 0) return a.defer != 0;
+    else return DEFER != 0;
+}
+
 // 0 + p[0] + p[1] + ... in that order, the values fetched by one load across the wave's lanes (up to 64 of them)
 // In two steps, so that a caller can send the load out beside its other loads and add up once they are all back:
 // lane_sum_fetch is the load (a lane's own value), lane_sum_fold the additions.
@@ -175,7 +183,7 @@ __device__ __forceinline__ void routed_prep_block(const MoeLaunch& a, uint32_t r
 // gate and up finishes, the (clamped) SwiGLU in f32 on their f16 values, and the down's prepare: hd [.][inter],
 // hs f32 [.][inter / 128]
 // the values of it: hh[j], the prepared f16 of element lane + 64 j of the block, and the block's sum of them
-template <bool PF, bool COH = false, int PROF = 0>
+template <bool PF, bool COH = false, int PROF = 0, int DEFER = -1>
 __device__ __forceinline__ void routed_mid_values(const MoeLaunch& a, const SlotRef& s, uint32_t q, uint32_t b,
                                                   uint32_t lane, uint32_t (&hh)[2], float& sum) {
     const RoutedBank& bank = s.shared ? a.shared : a.bank;
@@ -195,11 +203,12 @@ __device__ __forceinline__ void routed_mid_values(const MoeLaunch& a, const Slot
     float sums[4];
     const float* sgp = a.sg + static_cast<size_t>(q) * nb;
     const float* sup = a.su + static_cast<size_t>(q) * nb;
-    const float mg = a.defer ? lane_sum_fetch<COH>(sgp, nb, lane) : 0.0f;  // out with the planes' loads
-    const float mu = a.defer ? lane_sum_fetch<COH>(sup, nb, lane) : 0.0f;
+    const bool defer = defers<DEFER>(a);
+    const float mg = defer ? lane_sum_fetch<COH>(sgp, nb, lane) : 0.0f;  // out with the planes' loads
+    const float mu = defer ? lane_sum_fetch<COH>(sup, nb, lane) : 0.0f;
     ordered_sums<COH, 4>(planes, plane, ks, sums);
     float g[2] = {sums[0], sums[1]}, u[2] = {sums[2], sums[3]};
-    if (a.defer) {
+    if (defer) {
         const float xg = lane_sum_fold<COH>(mg, sgp, nb);
         const float xu = lane_sum_fold<COH>(mu, sup, nb);
 #pragma unroll
@@ -234,17 +243,17 @@ __device__ __forceinline__ void routed_mid_values(const MoeLaunch& a, const Slot
     for (int m = 32; m > 0; m >>= 1) sum += __shfl_xor(sum, m, 64);
 }
 
-template <bool PF, bool COH = false, int PROF = 0>
+template <bool PF, bool COH = false, int PROF = 0, int DEFER = -1>
 __device__ __forceinline__ void routed_mid_block(const MoeLaunch& a, const SlotRef& s, uint32_t q, uint32_t b,
                                                  uint32_t lane) {
     if (!s.live) return;
     uint32_t hh[2];
     float sum;
-    routed_mid_values<PF, COH, PROF>(a, s, q, b, lane, hh, sum);
+    routed_mid_values<PF, COH, PROF, DEFER>(a, s, q, b, lane, hh, sum);
 #pragma unroll
     for (uint32_t j = 0; j < 2u; ++j)
         store_prepared<PF>(a, a.hd, static_cast<size_t>(q) * a.inter, b * 128u + lane + 64u * j, hh[j]);
-    if (lane == 0u) a.hs[static_cast<size_t>(q) * (a.inter / 128u) + b] = sum;
+    if (defers<DEFER>(a) && lane == 0u) a.hs[static_cast<size_t>(q) * (a.inter / 128u) + b] = sum;  // the map's alone
 }
 
 // One slot's finished down outputs of block b (f16-valued), false for a skipped slot. COH: only the planes cross
@@ -274,7 +283,7 @@ __device__ __forceinline__ bool routed_down_finish(const MoeLaunch& a, const Slo
 
 // R slots' finished down outputs of block b at once (a skipped slot's entry is left alone): all their planes, scales
 // and block sums are fetched together. q[r]: where slot r's scratch lives.
-template <bool COH, bool HS_COH, int R, int PROF = 0>
+template <bool COH, bool HS_COH, int R, int PROF = 0, int DEFER = -1>
 __device__ __forceinline__ void routed_down_finish_many(const MoeLaunch& a, const SlotRef (&s)[R], const uint32_t (&q)[R],
                                                         uint32_t b, uint32_t lane, float (&v)[R][2], uint32_t ks) {
     const uint32_t rkt = a.rows * (a.topk + a.shared_slots), nbi = a.inter / 128u;
@@ -294,15 +303,16 @@ __device__ __forceinline__ void routed_down_finish_many(const MoeLaunch& a, cons
     }
     // the block sums' loads go out with the planes' (HS_COH: the sums were made inside this launch, a copy a 128-column
     // block of the output)
+    const bool defer = defers<DEFER>(a);
     const float* hs[R];
     float mine[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         hs[r] = a.hs + (HS_COH ? (static_cast<size_t>(b) * rkt + q[r]) * hs_copy_stride(a.inter) : static_cast<size_t>(q[r]) * nbi);
-        mine[r] = a.defer ? lane_sum_fetch<HS_COH>(hs[r], nbi, lane) : 0.0f;
+        mine[r] = defer ? lane_sum_fetch<HS_COH>(hs[r], nbi, lane) : 0.0f;
     }
     ordered_sums<COH, 2 * R>(planes, plane, ks, sums);
-    if (a.defer)
+    if (defer)
 #pragma unroll
         for (int r = 0; r < R; ++r) xsum[r] = lane_sum_fold<HS_COH>(mine[r], hs[r], nbi);
 #pragma unroll
@@ -310,7 +320,7 @@ __device__ __forceinline__ void routed_down_finish_many(const MoeLaunch& a, cons
         if (!s[r].live) continue;  // uniform over the wave
         v[r][0] = sums[2 * r];
         v[r][1] = sums[2 * r + 1];
-        if (a.defer)
+        if (defer)
 #pragma unroll
             for (uint32_t j = 0; j < 2u; ++j) v[r][j] = __builtin_fmaf(v[r][j], mul1_a(), mul1_b() * xsum[r]);
         if constexpr (PROF == 0) finish_core(v[r], sv[r], lane);
