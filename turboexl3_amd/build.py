@@ -24,8 +24,12 @@ ARCH = "gfx950"
 COMMON = ["-O3", "-std=c++20", "-fPIC", "-ffp-contract=off", "-Wall", "-Wno-unused-function"]
 # -amdgpu-mfma-vgpr-form: MFMA accumulators stay in VGPRs (these kernels need no AGPRs; the default shuffles
 # accumulators through AGPR copies every loop iteration)
+# -fma-mix-insts: no v_fma_mixlo_f16. The compiler folds f16(fma(a, b, c)) into that instruction where the fma's result
+# has no other use, and the instruction rounds once where the two it replaces round twice (to f32, then to f16, as the
+# format's own arithmetic does): whether a value met the fold depended on the code around it, and the same statements
+# gave different bytes in different kernels (the routed chain's two-launch and five-launch forms, MUL1's map).
 HIP_FLAGS = [f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-             "-mllvm", "-amdgpu-mfma-vgpr-form"]
+             "-Xclang", "-target-feature", "-Xclang", "-fma-mix-insts", "-mllvm", "-amdgpu-mfma-vgpr-form"]
 
 
 def hipcc() -> str:
@@ -66,7 +70,7 @@ def _compile(src: str, force: bool) -> str:
     cmd[-4:-4] = ["-Rpass-analysis=kernel-resource-usage", "-fno-caret-diagnostics"]  # remarks without source lines
     res = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in res.stderr.splitlines()
-                    if "packed-fp32-ops" not in l and "kernel-resource-usage" not in l)
+                    if "packed-fp32-ops" not in l and "fma-mix-insts" not in l and "kernel-resource-usage" not in l)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{err}")
     _check_no_scratch(src, res.stderr)
