@@ -149,6 +149,9 @@ __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
     typedef GemvStream<LDS, CB, WIDE, RB, BT, XGlobal> StreamG;
     constexpr uint32_t kStage = StreamG::kStageBytes;
     constexpr int R = gemv_step_rows<CB>();   // tile rows a step
+    // MUL1's map is deferred exactly under that codebook form (a.defer repeats it): the other forms' kernels carry none
+    // of its block sums
+    constexpr bool kDefer = CB == kMul1Defer;
     constexpr uint32_t kRed = 4u * RB * BT * 64u * 16u;
     constexpr uint32_t kMain = kRed > 4u * kStage ? kRed : 4u * kStage;
     // the waves' LDS rings while they stream; the four waves' partial sums afterwards
@@ -219,13 +222,13 @@ __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
                 float v[2] = {round_half(raw[r][b][0]) * sc[b][0], round_half(raw[r][b][1]) * sc[b][1]};
                 uint32_t hv[2];
                 float sum;
-                prep_core(v, lane, hv, sum, a.defer != 0);
+                prep_core(v, lane, hv, sum, kDefer);
 #pragma unroll
                 for (uint32_t j = 0; j < 2u; ++j) {
                     const uint32_t i = b * 128u + lane + 64u * j;  // element of the wave's K part: step i / (16 R)
                     x_step_store<R>(xst + ((i / (16u * R)) * kXldsRows + r) * 64u, i % (16u * R), hv[j]);
                 }
-                if (a.defer && lane == 0u && blk % kShare == 0u)
+                if (kDefer && lane == 0u && blk % kShare == 0u)
                     store_coherent(a.xs + (static_cast<size_t>(b128) * rows + r) * inblk + (tk0 >> 3) + b, sum);
             }
         }
@@ -283,7 +286,7 @@ __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
                 const float* xs_row = a.xs + (FUSE == kOne ? (static_cast<size_t>(b128) * rows + row) * inblk
                                                            : static_cast<size_t>(row) * inblk);
                 // arrive form: the block sums came from the prepare launch, only the planes cross workgroups
-                finish_block<true, FUSE == kOne>(a.dt, a.z, xs_row, a.svh, a.y, a.out, rows, a.ks, inblk, a.defer, row,
+                finish_block<true, FUSE == kOne>(a.dt, a.z, xs_row, a.svh, a.y, a.out, rows, a.ks, inblk, kDefer ? 1 : 0, row,
                                                  b128, lane);
             }
             if (threadIdx.x == 0u)  // zero again for the next call
