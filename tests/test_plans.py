@@ -136,6 +136,9 @@ def test_config4_prefill_items(lib):
     assert q.item_rows == 128                      # 128 rows an expert: the full shape
     assert [moe_plan(lib, t, 256, 7168, 2048, 8, 32, 48).item_rows for t in (512, 1024, 1280, 1344)] == [32, 64, 64, 96]
     assert p.expert_code_bytes == 2 * 3670016 + 5505024
+    # the cut that leaves no more items an expert than the other (a uniform routing's counts scatter like sqrt(mean)), the
+    # 96-row kernel's speed allowed for: 512 experts of 2560 x 640, top-10, at 160 / 120 / 80 / 200 rows an expert
+    assert [moe_plan(lib, t, 512, 2560, 640, 10, 64, 64).item_rows for t in (8192, 6144, 4096, 10240)] == [96, 128, 96, 128]
 
 
 def test_decode_forms_by_configuration(lib):
