@@ -188,49 +188,73 @@ __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
         const uint32_t row = lane & 15u;
         xoff[0] = (row < rows ? row : 0u) * 64u + (lane >> 4) * 16u;
         StreamL stream(wbase, wstep, per, a.n, a.wbits, XLds{xst}, xoff, smem + sg * kStage, lane);
-        stream.issue();
+        // The register ring's loads are the compiler's own, and a wave's loads come back in the order they went out: the
+        // activations' go out first, so the prepare waits for nothing but them (behind the codes' first tile rows it
+        // began later: the call 14.8 -> 14.6 us at one row, 16.2 -> 15.7 at four). The LDS ring's loads are issued from
+        // asm and not counted by the compiler, which then waits for every load in flight whichever went first.
+        constexpr bool kXFirst = !LDS;
+        if constexpr (!kXFirst) stream.issue();
         // While the codes fly, the wave prepares its own K part: per / 8 whole 128-blocks a row, the statements of
         // dense_prep, into its LDS x stage [steps + 1][4][64 bytes] (the last step zeros). The block sums go to the
         // column block's own copy of xs (deferred MUL1 map only; the block's second workgroup column, if any, would
         // store the same values again).
-        // Every row's loads go out together (rows and blocks past the call's alias the last real one, so there is no
-        // branch among the loads): a further row then costs its butterfly, not another round trip.
+        // Every row's loads go out together (rows past the call's alias the last real one, so there is no branch among
+        // the loads): a further row then costs its butterfly, not another round trip. One row and one block a wave, the
+        // commonest call, has a copy of its own that loads nothing else (a load costs the wave its issue whether its
+        // value is used or not: 20 loads in front of the codes' held them back 0.6 us where 4 do the work).
         const uint32_t blocks = per >> 3;  // 1 or 2
-        float raw[kXldsRows][2][2], sc[2][2];
-        auto load_rows = [&](auto tag) {
-            constexpr int DT = decltype(tag)::value;
+        auto prepare = [&](auto nr_c, auto nb_c) {
+            constexpr uint32_t NR = decltype(nr_c)::value, NB = decltype(nb_c)::value;  // rows loaded, blocks a wave
+            float raw[NR][NB][2], sc[NB][2];
+            auto load_rows = [&](auto tag) {
+                constexpr int DT = decltype(tag)::value;
 #pragma unroll
-            for (uint32_t b = 0; b < 2u; ++b)
+                for (uint32_t b = 0; b < NB; ++b)
 #pragma unroll
-                for (uint32_t j = 0; j < 2u; ++j) {
-                    const uint32_t i = ((tk0 >> 3) + (b < blocks ? b : blocks - 1u)) * 128u + lane + 64u * j;
-                    sc[b][j] = half_value(a.suh[i]);
+                    for (uint32_t j = 0; j < 2u; ++j) {
+                        const uint32_t i = ((tk0 >> 3) + b) * 128u + lane + 64u * j;
+                        sc[b][j] = half_value(a.suh[i]);
 #pragma unroll
-                    for (uint32_t r = 0; r < kXldsRows; ++r)
-                        raw[r][b][j] = load_act<DT>(a.x, static_cast<size_t>(r < rows ? r : rows - 1u) * a.in + i);
-                }
-        };
-        if (a.dt == kF32) load_rows(std::integral_constant<int, kF32>{});
-        else if (a.dt == kF16) load_rows(std::integral_constant<int, kF16>{});
-        else load_rows(std::integral_constant<int, kBf16>{});
-#pragma unroll
-        for (uint32_t r = 0; r < kXldsRows; ++r) {
-            if (r >= rows) break;
-#pragma unroll
-            for (uint32_t b = 0; b < 2u; ++b) {
-                if (b >= blocks) break;
-                float v[2] = {round_half(raw[r][b][0]) * sc[b][0], round_half(raw[r][b][1]) * sc[b][1]};
-                uint32_t hv[2];
-                float sum;
-                prep_core(v, lane, hv, sum, kDefer);
-#pragma unroll
-                for (uint32_t j = 0; j < 2u; ++j) {
-                    const uint32_t i = b * 128u + lane + 64u * j;  // element of the wave's K part: step i / (16 R)
-                    x_step_store<R>(xst + ((i / (16u * R)) * kXldsRows + r) * 64u, i % (16u * R), hv[j]);
-                }
-                if (kDefer && lane == 0u && blk % kShare == 0u)
-                    store_coherent(a.xs + (static_cast<size_t>(b128) * rows + r) * inblk + (tk0 >> 3) + b, sum);
+                        for (uint32_t r = 0; r < NR; ++r)
+                            raw[r][b][j] = load_act<DT>(a.x, static_cast<size_t>(r < rows ? r : rows - 1u) * a.in + i);
+                    }
+            };
+            if (a.dt == kF32) load_rows(std::integral_constant<int, kF32>{});
+            else if (a.dt == kF16) load_rows(std::integral_constant<int, kF16>{});
+            else load_rows(std::integral_constant<int, kBf16>{});
+            if constexpr (kXFirst) {
+                __builtin_amdgcn_sched_barrier(0);
+                stream.issue();
+                __builtin_amdgcn_sched_barrier(0);
             }
+#pragma unroll
+            for (uint32_t r = 0; r < NR; ++r) {
+                if (r >= rows) break;
+#pragma unroll
+                for (uint32_t b = 0; b < NB; ++b) {
+                    float v[2] = {round_half(raw[r][b][0]) * sc[b][0], round_half(raw[r][b][1]) * sc[b][1]};
+                    uint32_t hv[2];
+                    float sum;
+                    prep_core(v, lane, hv, sum, kDefer);
+#pragma unroll
+                    for (uint32_t j = 0; j < 2u; ++j) {
+                        const uint32_t i = b * 128u + lane + 64u * j;  // element of the wave's K part: step i / (16 R)
+                        x_step_store<R>(xst + ((i / (16u * R)) * kXldsRows + r) * 64u, i % (16u * R), hv[j]);
+                    }
+                    if (kDefer && lane == 0u && blk % kShare == 0u)
+                        store_coherent(a.xs + (static_cast<size_t>(b128) * rows + r) * inblk + (tk0 >> 3) + b, sum);
+                }
+            }
+        };
+        typedef std::integral_constant<uint32_t, 1u> One;
+        typedef std::integral_constant<uint32_t, 2u> Two;
+        typedef std::integral_constant<uint32_t, kXldsRows> Rows;
+        if (rows == 1u) {
+            if (blocks == 1u) prepare(One{}, One{});
+            else prepare(One{}, Two{});
+        } else {
+            if (blocks == 1u) prepare(Rows{}, One{});
+            else prepare(Rows{}, Two{});
         }
         for (uint32_t i = lane; i < kXldsRows * 16u; i += 64u)
             *reinterpret_cast<uint32_t*>(xst + steps * (kXldsRows * 64u) + i * 4u) = 0u;
