@@ -144,6 +144,14 @@ __device__ __forceinline__ uint32_t pair_quad_slot(uint32_t i) {
     return (i & ~31u) + 8u * q + 4u * ((i >> 4u) & 1u) + m;
 }
 
+// Where arrival counter i of a launch's `count` counters sits in the workspace's head (16,384 words): a cache line apart
+// while they fit (32 words), else 8 words, else side by side. A launch's workgroups count themselves in within a
+// microsecond of one another, and atomics to one cache line queue up: sixteen counters to a line cost the routed decode's
+// down launch, 176 arrivals at one token, a microsecond.
+__device__ __forceinline__ uint32_t arrive_slot(uint32_t i, uint32_t count) {
+    return i * (count <= 512u ? 32u : (count <= 2048u ? 8u : 1u));
+}
+
 // MUL1's affine map w = A h + B with h = 1024 + t (format.zig:158-167): A = f16 0x1EEE, B = f16 0xC931
 __device__ __forceinline__ float mul1_a() { return half_value(0x1EEEu); }
 __device__ __forceinline__ float mul1_b() { return half_value(0xC931u); }

@@ -301,7 +301,7 @@ __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
         __syncthreads();
         if (threadIdx.x == 0u) {
             const uint32_t before =
-                __hip_atomic_fetch_add(a.arrive + b128, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_fetch_add(a.arrive + arrive_slot(b128, a.out / 128u), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             last_flag = before == a.ks * kShare - 1u;
         }
         __syncthreads();
@@ -314,7 +314,7 @@ __global__ void __launch_bounds__(256) dense_gemv(const GemvArgs a) {
                                                  b128, lane);
             }
             if (threadIdx.x == 0u)  // zero again for the next call
-                __hip_atomic_store(a.arrive + b128, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(a.arrive + arrive_slot(b128, a.out / 128u), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 }

@@ -107,6 +107,24 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
 #pragma unroll
     for (int t = 0; t < BT; ++t) acc[0][t] = float4v{0.f, 0.f, 0.f, 0.f};
 
+    // The down launch's workgroup holds a slot's complete sums of its 128 columns where it is the only one to make them
+    // (one K slice, eight tiles a load): it then finishes them itself (the map, H128, svh: the slot's own statements on
+    // the same values) and stores the finished values where the plane would go, and the row's last arriver only adds
+    // the slots up in their order. Left to the last arriver, the slots' finishes and their scale loads (an expert's
+    // svh comes from HBM) stood one behind the other at the very end of the call: 512 experts of 2048 x 512, one token,
+    // the combine 4 us of the down launch's 14.9.
+    constexpr bool kMayFinishHere = NPROJ == 1 && ARRIVE && PROF == 0 && BT == 8;
+    const bool finish_here = kMayFinishHere && a.ks_dn == 1u;
+    float wave_sum = 0.0f;  // the deferred map's block sum of the wave's own 128-block (the mid stage run here)
+    float sv_here[2] = {0.0f, 0.0f};
+    if constexpr (kMayFinishHere) {
+        if (finish_here && sg == 0u && s.live) {  // the scales go out now and are back long before they are needed
+            const uint16_t* svh = bank.down_svh + static_cast<size_t>(s.e) * a.hidden + blk * 128u;
+            sv_here[0] = half_value(svh[lane]);
+            sv_here[1] = half_value(svh[lane + 64u]);
+        }
+    }
+
     if (part < parts && s.live) {  // uniform over the wave; a wave past the last part adds zeros below
         uint32_t xoff[1];
         if constexpr (XLDS && NPROJ == 1) {
@@ -121,6 +139,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
             uint32_t hh[2];
             float sum;
             routed_mid_values<false, false, PROF, kDefer>(a, s, rk, tk0 >> 3, lane, hh, sum);
+            wave_sum = sum;
             // element i = 64 j + lane of the block belongs to step i / (16 R) of the wave's walk
 #pragma unroll
             for (uint32_t j = 0; j < 2u; ++j) {
@@ -133,7 +152,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
             // shared by every column workgroup of the slot takes hundreds of device-coherent stores to the same few
             // cache lines, which serialise: 512 experts of 2560 x 640 at one token, the deferred map, this launch
             // 30.5 us at K3 and 49.6 at K5 against 16.9 and 19.6 for the codebook without the map.)
-            if (kDefer && lane == 0u && blk % (8u / BT) == 0u)
+            if (kDefer && !finish_here && lane == 0u && blk % (8u / BT) == 0u)
                 store_coherent(a.hs + (static_cast<size_t>(blk / (8u / BT)) * rkt + rk) * hs_copy_stride(a.inter) + (tk0 >> 3), sum);
             for (uint32_t i = lane; i < kXldsRows * 16u; i += 64u)
                 *reinterpret_cast<uint32_t*>(xst + steps * (kXldsRows * 64u) + i * 4u) = 0u;
@@ -190,14 +209,43 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
         for (int t = 0; t < BT; ++t) red[sg][t * 4 + (lane >> 4)] = acc[0][t];
     __syncthreads();
     float* z = NPROJ == 1 ? a.zd : (proj ? a.zu : a.zg);
+    float* here = reinterpret_cast<float*>(smem + 4096u);  // finish_here: the 128 sums, then the waves' block sums
     if (threadIdx.x < static_cast<uint32_t>(BT * 4)) {
         const uint32_t i = threadIdx.x, t = i >> 2;
         const float4v v = ((red[0][i] + red[1][i]) + red[2][i]) + red[3][i];
         float* dst = z + (static_cast<size_t>(ksl) * rkt + rk) * out + (blk * BT + t) * 16u + 4u * (i & 3u);
-        if constexpr (ARRIVE) {
+        if (finish_here) {
+            *reinterpret_cast<float4v*>(here + t * 16u + 4u * (i & 3u)) = v;
+        } else if constexpr (ARRIVE) {
             if (s.live) store_coherent4(dst, v);
         } else {
             *reinterpret_cast<float4v*>(dst) = v;
+        }
+    }
+    if constexpr (kMayFinishHere) {
+        if (finish_here) {
+            if constexpr (XLDS) {
+                if (lane == 0u) here[128u + sg] = wave_sum;
+            }
+            __syncthreads();
+            if (sg == 0u && s.live) {
+                float v[2] = {here[lane], here[lane + 64u]};
+                if constexpr (kDefer != 0) {
+                    const uint32_t nbi = a.inter / 128u;  // = the waves that hold a block (one K slice)
+                    float xsum = 0.0f;
+                    if constexpr (XLDS) {
+                        for (uint32_t q = 0; q < nbi; ++q) xsum += here[128u + q];  // lane_ordered_sum's order
+                    } else {
+                        xsum = lane_ordered_sum<false>(a.hs + static_cast<size_t>(rk) * nbi, nbi, lane);
+                    }
+#pragma unroll
+                    for (uint32_t j = 0; j < 2u; ++j) v[j] = __builtin_fmaf(v[j], mul1_a(), mul1_b() * xsum);
+                }
+                finish_core(v, sv_here, lane);
+                float* dst = a.zd + static_cast<size_t>(rk) * a.hidden + blk * 128u;
+                store_coherent(dst + lane, v[0]);
+                store_coherent(dst + lane + 64u, v[1]);
+            }
         }
     }
 
@@ -205,7 +253,8 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
         constexpr uint32_t kShare = 8u / BT;  // workgroup columns a 128-column block
         const uint32_t b128 = blk / kShare, kt = a.topk + a.shared_slots;
         const uint32_t ks = NPROJ == 2 ? a.ks_gu : a.ks_dn;
-        const uint32_t counter = NPROJ == 2 ? rk * (a.inter / 128u) + b128 : s.row * (a.hidden / 128u) + b128;
+        const uint32_t counter = NPROJ == 2 ? arrive_slot(rk * (a.inter / 128u) + b128, rkt * (a.inter / 128u))
+                                            : arrive_slot(s.row * (a.hidden / 128u) + b128, a.rows * (a.hidden / 128u));
         const uint32_t full = NPROJ == 2 ? 2u * ks * kShare : kt * ks * kShare;
         wait_stores();
         __syncthreads();
@@ -265,7 +314,16 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
                     sk[r].e = info & 0x7FFFFFFFu;
                     qk[r] = s.row * kt + (k < kt ? k : 0u);
                 }
-                routed_down_finish_many<true, XLDS, 4, 0, kDefer>(a, sk, qk, b128, lane, v, ks);
+                if (finish_here) {  // the slots' workgroups finished them: their values, all in flight together
+#pragma unroll
+                    for (uint32_t r = 0; r < 4u; ++r) {
+                        const float* zf = a.zd + static_cast<size_t>(qk[r]) * a.hidden + b128 * 128u;
+                        v[r][0] = load_coherent(zf + lane);
+                        v[r][1] = load_coherent(zf + lane + 64u);
+                    }
+                } else {
+                    routed_down_finish_many<true, XLDS, 4, 0, kDefer>(a, sk, qk, b128, lane, v, ks);
+                }
 #pragma unroll
                 for (uint32_t r = 0; r < 4u; ++r)
                     if (sk[r].live) {
