@@ -46,9 +46,13 @@ __device__ __forceinline__ void store_coherent(float* p, float v) {
 __device__ __forceinline__ float load_coherent(const float* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// four adjacent floats (16-byte aligned) in one device-coherent store
+// four adjacent floats (16-byte aligned) in one device-coherent store. The two wait states behind it: a store of more
+// than 64 bits reads its data registers over several cycles, and a vector instruction that writes one of them right
+// behind the store changes what the later lanes store. The compiler keeps that distance for its own stores; it does not
+// look inside this one. (Seen once the register allocation put a v_mov into the store's first two data registers as
+// the next instruction: lanes 12-15 and 28-31 of the wave stored the new values in their first two floats.)
 __device__ __forceinline__ void store_coherent4(float* p, float4v v) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
 }
 // every store this lane has issued is acknowledged at its coherence level (with store_coherent: device-wide)
 __device__ __forceinline__ void wait_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
