@@ -361,6 +361,7 @@ typedef struct t3_moe_plan {
     uint32_t hidden, inter, topk, shared_slots;
     uint32_t tiles_a_wave_gu, k_slices_gu, tiles_a_load_gu;  /* gate|up GEMV (decode rows) */
     uint32_t tiles_a_wave_dn, k_slices_dn, tiles_a_load_dn;  /* down GEMV */
+    uint32_t k_slices_a_workgroup_dn;  /* 2: the two launches' down workgroups hold both K slices (eight waves); same bytes */
     uint32_t item_rows, max_items;                           /* prefill: rows a GEMM item, items at most */
     uint64_t expert_code_bytes;  /* one expert's three matrices */
     size_t workspace_bytes;

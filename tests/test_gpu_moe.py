@@ -152,6 +152,49 @@ def test_launch_forms_give_the_same_bytes(oracle, t3):
         assert not ws[:65536].any()
 
 
+def test_two_down_slices_in_one_workgroup_give_the_chains_bytes(oracle, t3):
+    # An intermediate size of 513..1024 has two K slices of four 128-blocks in its down projection. The served launches
+    # hold both in one workgroup of eight waves (five to eight of them with a block); the chains behind their own stage
+    # launches keep a workgroup a slice and two planes. Same bytes: every codebook form, eight and four tiles a load (a
+    # wide rate), one to sixteen rows, a skipped slot, a shared expert, and GLM's profile.
+    rng = np.random.default_rng(0x2D5)
+    for inter, codebook, n in ((640, MCG, 64), (1024, MUL1, 96), (896, MCG, 48), (768, MUL1, 32)):
+        hidden, experts, topk = 256, 6, 3
+        bank = oracle.synth_bank(rng, experts, hidden, inter, n)
+        shared = oracle.synth_bank(rng, 1, hidden, inter, n)
+        dbank, dshared = dev_bank(t3, bank), dev_bank(t3, shared)
+        x_dev, x_f32 = make_x(rng, 16, hidden, torch.bfloat16)
+        slots, scores = routing(rng, 16, topk, experts)
+        slots[0, 1] = -1
+        dec = t3.Decode(codebook, 16)
+        ref = RefBank(oracle, bank, codebook, 0xFFFF)
+        for rows in (1, 2, 4, 5, 16):
+            d_slots = torch.from_numpy(slots[:rows]).cuda().reshape(1, rows, topk)
+            d_scores = torch.from_numpy(scores[:rows]).cuda().reshape(1, rows, topk)
+            x = x_dev[:rows].reshape(1, rows, hidden)
+            calls = [lambda: t3.moe(x, dbank, d_slots, d_scores, dec),
+                     lambda: t3.moe_shared_expert(x, dbank, d_slots, d_scores, dec, 1, dshared)]
+            if codebook == MCG or n == 32:  # GLM's profile is served for MCG and for MUL1's deferred map
+                k = topk + 1
+                g_slots = np.concatenate([np.where(slots[:rows] < 0, 0, slots[:rows]), np.full((rows, 1), experts)], axis=1).astype(np.int32)
+                dg = torch.from_numpy(g_slots).cuda().reshape(1, rows, k)
+                calls.append(lambda: t3.moe_glm(x, dbank, dg, dec, 7, fill=float("nan")))
+            for ci, call in enumerate(calls):
+                served = call()
+                assert bytes_of(served) == bytes_of(call())
+                for form in (3, 6):
+                    t3.configure(decode_form=form)
+                    try:
+                        other = call()
+                    finally:
+                        t3.configure()
+                    assert bytes_of(served) == bytes_of(other), f"inter {inter} rows {rows} call {ci}: differs from form {form}"
+            got = to_f32(calls[0]()).reshape(rows, hidden)
+            for r in range(rows):
+                e = oracle.compare(got[r], ref.row(x_f32[r], slots[r], scores[r]))
+                assert e <= BF16_BAR, f"inter {inter} rows {rows} row {r}: {e:.3e}"
+
+
 def test_launch_forms_give_the_same_bytes_at_the_reference_rows(oracle, t3):
     # src/hip_tests.zig:891-895,907: the reference's model-sized case (2560 x 640, 16 experts, top-10, K3, MUL1's deferred
     # map, bf16) at its rows 1-5, 8 and 16

@@ -127,6 +127,19 @@ def test_config3_routed_partition(lib):
     assert (p.path, p.launches) == (3, 9)
 
 
+def test_down_slices_a_workgroup(lib):
+    # a down projection of two K slices (inter 513..1024): one workgroup of eight waves holds both while those workgroups
+    # are resident at once (512 of them); 512 experts of 2560 x 640 top-10 have 20 column blocks x 10 r
+    plans = [moe_plan(lib, rows, 512, 2560, 640, 10, 48, 48) for rows in (1, 2, 3, 4, 8)]
+    assert [p.k_slices_dn for p in plans] == [2] * 5               # the sums' partition does not move
+    assert [p.k_slices_a_workgroup_dn for p in plans] == [2, 2, 1, 1, 1]
+    # four tiles a load (K5): twice the column workgroups
+    assert [moe_plan(lib, rows, 512, 2560, 640, 10, 80, 80).k_slices_a_workgroup_dn for rows in (1, 2)] == [2, 1]
+    # one slice, or four: a workgroup a slice
+    assert moe_plan(lib, 1, 512, 2048, 512, 10, 48, 48).k_slices_a_workgroup_dn == 1
+    assert moe_plan(lib, 1, 64, 4096, 2048, 8, 64, 64).k_slices_a_workgroup_dn == 1
+
+
 def test_config4_prefill_items(lib):
     p = moe_plan(lib, 2048, 256, 7168, 2048, 8, 32, 48)
     assert p.path == 3 and p.row_slots == 16384

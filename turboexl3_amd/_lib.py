@@ -71,6 +71,7 @@ class MoePlan(C.Structure):
                 ("hidden", C.c_uint32), ("inter", C.c_uint32), ("topk", C.c_uint32), ("shared_slots", C.c_uint32),
                 ("tiles_a_wave_gu", C.c_uint32), ("k_slices_gu", C.c_uint32), ("tiles_a_load_gu", C.c_uint32),
                 ("tiles_a_wave_dn", C.c_uint32), ("k_slices_dn", C.c_uint32), ("tiles_a_load_dn", C.c_uint32),
+                ("k_slices_a_workgroup_dn", C.c_uint32),
                 ("item_rows", C.c_uint32), ("max_items", C.c_uint32), ("expert_code_bytes", C.c_uint64),
                 ("workspace_bytes", C.c_size_t), ("route_order_at", C.c_size_t), ("route_inv_at", C.c_size_t),
                 ("route_items_at", C.c_size_t), ("route_counts_at", C.c_size_t)]

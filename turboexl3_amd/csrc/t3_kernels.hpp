@@ -92,6 +92,7 @@ struct MoeLaunch {
     uint32_t hidden = 0, inter = 0, rows = 0, topk = 0, shared_slots = 0;
     uint32_t n_gu = 0, n_dn = 0, wbits = 16;
     uint32_t per_gu = 8, per_dn = 8, parts_gu = 0, parts_dn = 0, ks_gu = 1, ks_dn = 1, bt_gu = 8, bt_dn = 8;
+    uint32_t dn_slices_a_wg = 1;  // K slices one workgroup of the served down launch holds (2: eight waves)
     int codebook = 0, dtype = 0, score_dt = 0, defer = 0;
     int pair_order = 0;  // decode rows: the GEMVs take two tile rows a step (the f16-weight codebook forms) and read their
                          // activations as plain f16 in pair-quad order; else one, doubled f16 in quad order

@@ -143,6 +143,15 @@ int32_t check_moe(const t3_array* x, const t3_bank* bank, const t3_array* inds, 
     // launch is small at eight tiles, within 2048 workgroups: large experts fill the GPU at one row already.)
     const uint64_t gu_wgs = static_cast<uint64_t>(l.inter / 128u) * l.rows * (l.topk + l.shared_slots) * 2u * l.ks_gu;
     if (l.rows <= kMoeFewRows && l.bt_gu == 8u && gu_wgs <= 2048u) l.bt_gu = 4u;
+    // A down projection of two K slices (an intermediate size of 513 to 1024): the served launches hold both in one
+    // workgroup of eight waves where those workgroups are resident all at once (two a CU): half the arrivals, no
+    // second plane, and at eight tiles a load the workgroup finishes the slot's sums itself. The sums are added in the
+    // planes' order, so the bytes are the chain's. Measured, a call, a workgroup a slice -> both in one: 512 experts of
+    // 2560 x 640 top-10, MUL1 K3, one / two rows 28.5 -> 25.7 / 36.9 -> 34.1 us; MCG K4 27.0 -> 25.4 / 34.9 -> 33.8;
+    // 2048 x 768 one / three rows 26.8 -> 25.2 / 41.0 -> 39.5. Past one round nothing is gained (the same shapes at
+    // four rows 56.4 -> 56.4, 53.6 -> 54.4), nor where the experts are large (4096 x 1024: 39.4 -> 39.7).
+    const uint64_t dn_wgs = static_cast<uint64_t>((l.hidden / 16u) / l.bt_dn) * l.rows * (l.topk + l.shared_slots);
+    l.dn_slices_a_wg = l.ks_dn == 2u && dn_wgs <= 512u ? 2u : 1u;
     return T3_OK;
 }
 
@@ -343,6 +352,7 @@ int32_t t3_moe_plan_of(const t3_array* x, const t3_bank* bank, const t3_array* i
         p.tiles_a_wave_dn = l.per_dn;
         p.k_slices_dn = l.ks_dn;
         p.tiles_a_load_dn = l.bt_dn;
+        p.k_slices_a_workgroup_dn = form == t3::kMoeTwoLaunches ? l.dn_slices_a_wg : 1u;
     }
     p.workspace_bytes = call.workspace;
     *plan = p;

@@ -54,19 +54,28 @@ constexpr uint32_t kMidInDownRows = kMoeFewRows;
 // the register ring: a row-slot's waves walk eight tile rows (the LDS ring pays from about 32 a wave)
 constexpr bool kMoeLdsRing = T3_GEMV_LDS_RING_FROM <= 8;
 
-// a workgroup's static LDS: the four waves' rings while they stream, their partial sums afterwards
+// a wave's share of its workgroup's LDS: its ring while it streams, its partial sums afterwards (the last arriver's
+// sixteen finished slots, 8 KB, lie over the first waves' shares)
 template <int BT>
-constexpr uint32_t role_lds_bytes() {
-    constexpr uint32_t stage = 4u * GemvStream<kMoeLdsRing, kMcg, kNarrow, 1, BT, XLds>::kStageBytes, red = 4u * BT * 4u * 16u;
+constexpr uint32_t role_wave_lds_bytes() {
+    constexpr uint32_t stage = GemvStream<kMoeLdsRing, kMcg, kNarrow, 1, BT, XLds>::kStageBytes, red = BT * 4u * 16u;
     return stage > red ? stage : red;
 }
 
-template <int CB, int WIDE, int BT, int NPROJ, bool XLDS, bool ARRIVE, int PROF>
+// NW: the waves a workgroup, four a K slice. Eight: the workgroup holds both K slices of a down projection that has two
+// (an intermediate size of 513 to 1024), one wave a 128-block of the input (a wave past the last block adds zeros), and
+// adds their sums as the stage behind the planes would: slice 0's four first, then slice 1's. (Five to eight waves by
+// the blocks, their LDS sized by the launch, was measured too: 0.2 to 0.8 us slower at one to three rows than eight
+// waves always, and its 320-thread workgroups of 512 experts of 2560 x 640 at four rows no longer fit one round: 30.8
+// -> 37.6 us.) smem: the waves' shares; xbase: the waves' prepared activations where the launch makes them (XLDS).
+template <int CB, int WIDE, int BT, int NPROJ, bool XLDS, bool ARRIVE, int PROF, int NW>
 __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint32_t yidx, uint32_t ksl,
-                                          unsigned char* smem, uint32_t& last_flag, uint32_t* cinfo, float* cscore) {
+                                          unsigned char* smem, unsigned char* xbase, uint32_t& last_flag, uint32_t* cinfo,
+                                          float* cscore) {
     typedef GemvStream<kMoeLdsRing, CB, WIDE, 1, BT, XLds> StreamL;
     typedef GemvStream<kMoeLdsRing, CB, WIDE, 1, BT, XGlobal> StreamG;
     constexpr uint32_t kStage = StreamG::kStageBytes;
+    static_assert(kStage <= role_wave_lds_bytes<BT>() && StreamL::kStageBytes <= role_wave_lds_bytes<BT>(), "a wave's ring fits its share");
     constexpr int R = gemv_step_rows<CB>();   // tile rows a step
     // the codebook form says whether MUL1's map is deferred (a.defer repeats it): the other forms' kernels carry none of
     // the map's loads, sums and stores
@@ -96,7 +105,7 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
     const uint32_t in_tiles = in >> 4, out_tiles = out >> 4, nw = n >> 1;
     const uint32_t* wmat = (NPROJ == 1 ? bank.down_t : (proj ? bank.up_t : bank.gate_t)) +
                            static_cast<size_t>(s.e) * in_tiles * out_tiles * nw;
-    const uint32_t part = ksl * 4u + sg;
+    const uint32_t part = ksl * NW + sg;
     const uint32_t tk0 = part * per;
     const uint64_t wstride = static_cast<uint64_t>(out_tiles) * nw;
     const uint32_t* wbase = wmat + static_cast<uint64_t>(blk) * BT * nw + tk0 * wstride;
@@ -130,9 +139,8 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
         if constexpr (XLDS && NPROJ == 1) {
             // The down's input made here: the wave runs the mid stage of its own 128-block (its eight input tiles) over
             // the gate|up launch's planes and keeps the prepared block in LDS.
-            extern __shared__ __attribute__((aligned(16))) unsigned char xdyn[];
             const uint32_t steps = per / R;
-            unsigned char* xst = xdyn + sg * ((steps + 1u) * (kXldsRows * 64u));
+            unsigned char* xst = xbase + sg * ((steps + 1u) * (kXldsRows * 64u));
             xoff[0] = (lane >> 4) * 16u;
             StreamL stream(wbase, wstep, per, n, a.wbits, XLds{xst}, xoff, smem + sg * kStage, lane);
             stream.issue();
@@ -158,9 +166,8 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
                 *reinterpret_cast<uint32_t*>(xst + steps * (kXldsRows * 64u) + i * 4u) = 0u;
             stream.run(acc);
         } else if constexpr (XLDS) {
-            extern __shared__ __attribute__((aligned(16))) unsigned char xdyn[];
             const uint32_t steps = per / R;
-            unsigned char* xst = xdyn + sg * ((steps + 1u) * (kXldsRows * 64u));
+            unsigned char* xst = xbase + sg * ((steps + 1u) * (kXldsRows * 64u));
             xoff[0] = (lane >> 4) * 16u;  // every activation row of the fragment is the slot's one row
             StreamL stream(wbase, wstep, per, n, a.wbits, XLds{xst}, xoff, smem + sg * kStage, lane);
             stream.issue();
@@ -212,7 +219,8 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
     float* here = reinterpret_cast<float*>(smem + 4096u);  // finish_here: the 128 sums, then the waves' block sums
     if (threadIdx.x < static_cast<uint32_t>(BT * 4)) {
         const uint32_t i = threadIdx.x, t = i >> 2;
-        const float4v v = ((red[0][i] + red[1][i]) + red[2][i]) + red[3][i];
+        float4v v = ((red[0][i] + red[1][i]) + red[2][i]) + red[3][i];
+        if constexpr (NW == 8) v = v + (((red[4][i] + red[5][i]) + red[6][i]) + red[7][i]);  // plane 0 + plane 1
         float* dst = z + (static_cast<size_t>(ksl) * rkt + rk) * out + (blk * BT + t) * 16u + 4u * (i & 3u);
         if (finish_here) {
             *reinterpret_cast<float4v*>(here + t * 16u + 4u * (i & 3u)) = v;
@@ -251,6 +259,8 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
 
     if constexpr (ARRIVE) {
         constexpr uint32_t kShare = 8u / BT;  // workgroup columns a 128-column block
+        // the last arriver finishes the row's slots sixteen at a time, slot k0 + NW r + wave the wave's r-th
+        constexpr uint32_t kMine = 16u / NW;
         const uint32_t b128 = blk / kShare, kt = a.topk + a.shared_slots;
         const uint32_t ks = NPROJ == 2 ? a.ks_gu : a.ks_dn;
         const uint32_t counter = NPROJ == 2 ? arrive_slot(rk * (a.inter / 128u) + b128, rkt * (a.inter / 128u))
@@ -273,12 +283,12 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
             // GLM's profile ends with each live slot's own finished output, f32 [row-slot][hidden]: four slots a wave,
             // every load of the four in flight together, nothing to add up
             for (uint32_t k0 = 0; k0 < kt; k0 += 16u) {
-                SlotRef sk[4];
-                uint32_t qk[4];
-                float v[4][2];
+                SlotRef sk[kMine];
+                uint32_t qk[kMine];
+                float v[kMine][2];
 #pragma unroll
-                for (uint32_t r = 0; r < 4u; ++r) {
-                    const uint32_t k = k0 + 4u * r + sg;
+                for (uint32_t r = 0; r < kMine; ++r) {
+                    const uint32_t k = k0 + NW * r + sg;
                     const uint32_t info = k < kt ? cinfo[k] : 0xFFFFFFFFu;
                     sk[r].row = s.row;
                     sk[r].live = info != 0xFFFFFFFFu;
@@ -286,9 +296,9 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
                     sk[r].e = info & 0x7FFFFFFFu;
                     qk[r] = s.row * kt + (k < kt ? k : 0u);
                 }
-                routed_down_finish_many<true, XLDS, 4, 1, kDefer>(a, sk, qk, b128, lane, v, ks);
+                routed_down_finish_many<true, XLDS, kMine, 1, kDefer>(a, sk, qk, b128, lane, v, ks);
 #pragma unroll
-                for (uint32_t r = 0; r < 4u; ++r)
+                for (uint32_t r = 0; r < kMine; ++r)
                     if (sk[r].live) {
                         float* o = static_cast<float*>(a.y) + static_cast<size_t>(qk[r]) * a.hidden + b128 * 128u + lane;
                         o[0] = v[r][0];
@@ -296,17 +306,17 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
                     }
             }
         } else {
-            // The slots' finishes sixteen at a time, four a wave (slot k0 + 4 r + wave) with every load of the four in
-            // flight together; wave 0 adds them in slot order.
+            // The slots' finishes sixteen at a time, 16 / NW a wave with every load of a wave's slots in flight
+            // together; wave 0 adds them in slot order.
             float(*fin)[128] = reinterpret_cast<float(*)[128]>(smem);
             float acc2[2] = {0.0f, 0.0f}, gated[2] = {0.0f, 0.0f};
             for (uint32_t k0 = 0; k0 < kt; k0 += 16u) {
-                SlotRef sk[4];
-                uint32_t qk[4];
-                float v[4][2];
+                SlotRef sk[kMine];
+                uint32_t qk[kMine];
+                float v[kMine][2];
 #pragma unroll
-                for (uint32_t r = 0; r < 4u; ++r) {
-                    const uint32_t k = k0 + 4u * r + sg;
+                for (uint32_t r = 0; r < kMine; ++r) {
+                    const uint32_t k = k0 + NW * r + sg;
                     const uint32_t info = k < kt ? cinfo[k] : 0xFFFFFFFFu;
                     sk[r].row = s.row;
                     sk[r].live = info != 0xFFFFFFFFu;
@@ -316,19 +326,19 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
                 }
                 if (finish_here) {  // the slots' workgroups finished them: their values, all in flight together
 #pragma unroll
-                    for (uint32_t r = 0; r < 4u; ++r) {
+                    for (uint32_t r = 0; r < kMine; ++r) {
                         const float* zf = a.zd + static_cast<size_t>(qk[r]) * a.hidden + b128 * 128u;
                         v[r][0] = load_coherent(zf + lane);
                         v[r][1] = load_coherent(zf + lane + 64u);
                     }
                 } else {
-                    routed_down_finish_many<true, XLDS, 4, 0, kDefer>(a, sk, qk, b128, lane, v, ks);
+                    routed_down_finish_many<true, XLDS, kMine, 0, kDefer>(a, sk, qk, b128, lane, v, ks);
                 }
 #pragma unroll
-                for (uint32_t r = 0; r < 4u; ++r)
+                for (uint32_t r = 0; r < kMine; ++r)
                     if (sk[r].live) {
-                        fin[4u * r + sg][lane] = v[r][0];
-                        fin[4u * r + sg][lane + 64u] = v[r][1];
+                        fin[NW * r + sg][lane] = v[r][0];
+                        fin[NW * r + sg][lane + 64u] = v[r][1];
                     }
                 __syncthreads();
                 if (sg == 0u)
@@ -350,13 +360,14 @@ __device__ __forceinline__ void gemv_role(const MoeLaunch& a, uint32_t blk, uint
     }
 }
 
-template <int CB, int WIDE, int BT, int NPROJ, bool XLDS, bool ARRIVE, int PROF>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ? 2 : (gemv_step_rows<CB>() == 2 ? 3 : 4)))) moe_gemv(const MoeLaunch a) {
-    __shared__ __attribute__((aligned(16))) unsigned char smem[role_lds_bytes<BT>()];
+template <int CB, int WIDE, int BT, int NPROJ, bool XLDS, bool ARRIVE, int PROF, int NW = 4>
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(WIDE ? 2 : (gemv_step_rows<CB>() == 2 ? 3 : 4)))) moe_gemv(const MoeLaunch a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char xdyn[];
+    __shared__ __attribute__((aligned(16))) unsigned char smem[NW * role_wave_lds_bytes<BT>()];
     __shared__ uint32_t last_flag, cinfo[64];
     __shared__ float cscore[64];
-    gemv_role<CB, WIDE, BT, NPROJ, XLDS, ARRIVE, PROF>(a, blockIdx.x, blockIdx.y, blockIdx.z, smem, last_flag, cinfo,
-                                                       cscore);
+    gemv_role<CB, WIDE, BT, NPROJ, XLDS, ARRIVE, PROF, NW>(a, blockIdx.x, blockIdx.y, blockIdx.z, smem, xdyn, last_flag,
+                                                           cinfo, cscore);
 }
 
 // ---- the grouped form ------------------------------------------------------------------------------------------
@@ -534,8 +545,29 @@ hipError_t launch_gemv_bt(const MoeLaunch& a, hipStream_t s) {
     const uint32_t out = NPROJ == 2 ? a.inter : a.hidden;
     const uint32_t bt = NPROJ == 2 ? a.bt_gu : a.bt_dn, ks = NPROJ == 2 ? a.ks_gu : a.ks_dn;
     const uint32_t rkt = a.rows * (a.topk + a.shared_slots);
+    const size_t dyn_wave = XLDS ? ((NPROJ == 2 ? a.per_gu : a.per_dn) / gemv_step_rows<CB>() + 1u) * (kXldsRows * 64u) : 0u;
+    if constexpr (NPROJ == 1 && ARRIVE) {
+        // Both K slices of the down projection in one workgroup of eight waves (the host's rule: MoeLaunch::
+        // dn_slices_a_wg): the kernel sees one slice and one plane. The launches behind their own stage launches keep a
+        // workgroup a slice; the sums are added in the same order either way.
+        if (ks == 2u && a.dn_slices_a_wg == 2u) {
+            MoeLaunch b = a;
+            b.ks_dn = 1u;
+            const size_t dyn8 = 8u * dyn_wave;
+            const dim3 grid8((out / 16u) / bt, rkt, 1u), block8(512);
+            if constexpr (WIDE == kNarrow) {
+                if (bt == 8u) {
+                    hipLaunchKernelGGL((moe_gemv<CB, WIDE, 8, 1, XLDS, true, PROF, 8>), grid8, block8, dyn8, s, b);
+                    return hipGetLastError();
+                }
+            }
+            if (bt != 4u) return hipErrorInvalidValue;
+            hipLaunchKernelGGL((moe_gemv<CB, WIDE, 4, 1, XLDS, true, PROF, 8>), grid8, block8, dyn8, s, b);
+            return hipGetLastError();
+        }
+    }
     const dim3 grid((out / 16u) / bt, rkt * NPROJ, ks), block(256);
-    const size_t dyn = XLDS ? 4u * ((NPROJ == 2 ? a.per_gu : a.per_dn) / gemv_step_rows<CB>() + 1u) * (kXldsRows * 64u) : 0u;
+    const size_t dyn = 4u * dyn_wave;
     if constexpr (WIDE == kNarrow) {
         if (bt == 8u) {
             hipLaunchKernelGGL((moe_gemv<CB, WIDE, 8, NPROJ, XLDS, ARRIVE, PROF>), grid, block, dyn, s, a);
