@@ -19,7 +19,8 @@ stage timed alone, and the same call over MUL1's codebook; TFLOP/s against the 2
 dense f16 GEMM measured in this process, `measured_dense_f16_peak`), `dense_prefill` (config 5's 4096 rows and its
 resident-weight forms),
 `measured_hbm_read_peak` (a plain 16-byte-a-lane read of 2 GiB in this process: every HBM fraction is also given against
-it), `streaming` (one row of 4096 -> 151936 at K = 3, 4, 5: matrices of 233 to 389 MB, where a launch's ramp, tail and
+it), `plain_read_of_the_same_bytes` (the same read kernel over the headline's own 25 MB weight copies, launch by launch:
+what start, first bytes and drain cost a launch of this size whatever it computes), `streaming` (one row of 4096 -> 151936 at K = 3, 4, 5: matrices of 233 to 389 MB, where a launch's ramp, tail and
 hand-off vanish and the kernel's steady state shows), `reference_workload` (the reference's own published workload:
 2560 x 640, 512 experts, top-10, bf16, MUL1, K2..K8 at 1 and 4 rows as chains of 48 dependent calls over fresh experts,
 prefill at 8192 and 1328 rows; context beside docs/models/qwen38/results.md, never the target),
@@ -666,6 +667,20 @@ def main() -> int:
 
     out["measured_hbm_read_peak"] = hbm_read
     out["roofline"]["frac_of_measured_read_peak"] = head["call_gbps"] / READ_PEAK_GBPS
+    # what a launch that only reads the headline's bytes takes: the same rotating copies, the same graph of back-to-back
+    # launches, the plain read kernel (start, first bytes and drain of a 25 MB launch included, as in `value`)
+    sink = torch.empty(4096 * 256, dtype=torch.int32, device="cuda")
+
+    def plain(i, stream, wgs):
+        st = d.L.t3_test_hbm_read(stream, d.trellis[i % d.copies].data_ptr(), d.cb, sink.data_ptr(), wgs)
+        if st != 0:
+            raise RuntimeError(d.L.t3_error_name(st).decode())
+
+    reads = {wgs: graph_time(torch, lambda i, s2: plain(i, s2, wgs), sub_steps, 10, 3) for wgs in (768, 1536, 2048)}
+    wgs = min(reads, key=reads.get)
+    out["plain_read_of_the_same_bytes"] = {"us_per_launch": reads[wgs] * 1e6, "workgroups": wgs, "bytes": d.cb,
+                                           "gbps": d.cb / reads[wgs] / 1e9,
+                                           "kernel": "t3_test_hbm_read over the headline's rotating weight copies"}
 
     if "sweep" in sections:
         out["sweep"] = []

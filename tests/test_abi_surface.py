@@ -80,3 +80,20 @@ def test_null_arguments_are_bad_args(lib):
     need = C.c_size_t(0)
     assert lib.t3_error_name(lib.t3_linear_workspace_bytes(None, None, Decode(1, 16), C.byref(need))).decode() == "BadArgs"
     assert lib.t3_error_name(lib.t3_test_codebooks(None, None, None, None)).decode() == "BadArgs"
+
+
+def test_hand_written_wide_stores_keep_their_wait_states():
+    """A vector-memory store of more than 64 bits reads its data registers over several cycles; the compiler keeps two
+    wait states between such a store and a vector write of those registers for its own stores, not for one inside an
+    `asm` statement. Every hand-written wide store in the kernels carries them in the same statement."""
+    src = os.path.join(ROOT, "turboexl3_amd", "csrc")
+    wide = re.compile(r"(global|buffer|flat)_store_(dwordx[34]|b96|b128)")
+    found = 0
+    for name in sorted(os.listdir(src)):
+        text = open(os.path.join(src, name)).read()
+        for m in re.finditer(r"\basm\b[^;]*?\(([^;]*?)\)\s*;", text, re.S):
+            body = m.group(1)
+            if wide.search(body):
+                found += 1
+                assert re.search(r"_store_\w+[^\"]*\\n\\ts_nop [1-9]", body), f"{name}: a wide store without wait states behind it"
+    assert found >= 1  # store_coherent4 (t3_common.hpp)
