@@ -174,6 +174,10 @@ def test_two_down_slices_in_one_workgroup_give_the_chains_bytes(oracle, t3):
             x = x_dev[:rows].reshape(1, rows, hidden)
             calls = [lambda: t3.moe(x, dbank, d_slots, d_scores, dec),
                      lambda: t3.moe_shared_expert(x, dbank, d_slots, d_scores, dec, 1, dshared)]
+            if rows <= 4:  # the gated shared expert rides the same launches up to four rows
+                table = sigmoid_table(torch.bfloat16).cuda()
+                logit = torch.from_numpy(rng.standard_normal(rows).astype(np.float32)).to(torch.bfloat16).cuda()
+                calls.append(lambda: t3.moe_fused_shared(x, dbank, d_slots, d_scores, dec, dshared, table, logit))
             if codebook == MCG or n == 32:  # GLM's profile is served for MCG and for MUL1's deferred map
                 k = topk + 1
                 g_slots = np.concatenate([np.where(slots[:rows] < 0, 0, slots[:rows]), np.full((rows, 1), experts)], axis=1).astype(np.int32)
