@@ -51,7 +51,13 @@
 namespace t3 {
 
 constexpr uint32_t kTileSlot = 256u;  // register ring: LDS bytes a staged tile (2n <= 256)
-constexpr uint32_t kXldsRows = 4u;    // activation rows the in-LDS form of the prepared input holds
+// Activation rows the in-LDS form of the prepared input holds. (A build-time override for measuring the one-launch dense
+// form at more rows, with T3_ONE_ROWS_BT8 of t3_linear.cpp: 16 rows took 23.3 us a call against the chain's 18.1 at
+// 4096 x 12288 K4: every column workgroup prepares every row of its K part again.)
+#ifndef T3_XLDS_ROWS
+#define T3_XLDS_ROWS 4u
+#endif
+constexpr uint32_t kXldsRows = T3_XLDS_ROWS;
 constexpr uint32_t kRowSlot = 1024u;  // LDS ring: bytes one load of a wave fills: 64 lanes x 16 bytes
 constexpr uint32_t kNoBytes = 0x80000000u;  // a lane offset no buffer reaches: zeros, no traffic
 
