@@ -101,7 +101,11 @@ __device__ __forceinline__ uint32_t weight_halves(uint32_t cw_lo, uint32_t cw_hi
             : "=v"(d)
             : "v"(pa));
         // the two wait states a sub-dword write needs before a matrix instruction reads the register: the compiler
-        // adds them for its own SDWA instructions, not for this one
+        // adds them for its own SDWA instructions, not for this one. (The second add keeps the first one's half of d, so
+        // it reads d: a sub-dword write wants one wait state before such a read as well. The two adds are separate
+        // statements so that the compiler can put the second weight's hash between them, which it does in every
+        // kernel compiled from this tree: no pair is adjacent in their ISA. A change that made them adjacent would show
+        // as wrong low halves in every parity test that decodes MCG through a GEMV or a GEMM.)
         asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1\n\t"
             "s_nop 1"
             : "+v"(d)
